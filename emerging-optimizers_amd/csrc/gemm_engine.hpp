@@ -1,0 +1,307 @@
+// bf16 MFMA tile engine for gfx950 (MI355X): OUT[M x N] = epilogue( sum_k P[m][k] * Q[n][k] ).
+//
+// One template covers the three products of a Newton-Schulz step:
+//   SYRK mode : P == Q, only lower-triangle tiles are launched, results are mirrored on store
+//   GEMM mode : OUT = beta * Cin + alpha * acc  (the AXPY of X' = a X + B X lives in the epilogue)
+// Each operand is either "K-contiguous" (element (r, k) at r*ld + k) or "K-strided"
+// (element (r, k) at k*ld + r); K-strided tiles are transposed in registers (v_perm_b32 on 8x8
+// blocks) on their way to LDS, so the MFMA fragment reads are always 16-byte ds_read_b128.
+//
+// Wavefront = 64 lanes; MFMA = v_mfma_f32_32x32x16_bf16.  Fragment/accumulator mapping used here:
+//   A operand (32 x 16): lane l supplies row (l % 32), k = 8*(l / 32) .. +7
+//   B operand (16 x 32): lane l supplies col (l % 32), k = 8*(l / 32) .. +7
+//   D (32 x 32)        : lane l holds col (l % 32); acc[4*g + r] is row 8*g + 4*(l / 32) + r
+// The Q fragment is passed as the A operand and the P fragment as the B operand, so a lane ends up
+// holding one output row (P index) and groups of 4 consecutive output columns (Q index).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mi {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+enum { MODE_SYRK = 0, MODE_GEMM = 1 };
+
+struct GemmParams {
+  const uint16_t* P;
+  const uint16_t* Q;
+  int64_t ldp, ldq, p_bs, q_bs;  // leading dims / batch strides in elements
+  const uint16_t* Cin;           // bf16, indexed like OUT; may be null when beta == 0
+  int64_t ldc, c_bs;
+  void* Out;                     // bf16 or float32, row-major (M x N)
+  int64_t ldo, o_bs;
+  int M, N, K;
+  float alpha, beta, out_scale;
+  int tiles_m, tiles_n;
+  int skip_upper;
+};
+
+// Byte offset of 16-byte chunk `chunk` of row `row` in an LDS tile whose rows hold BK bf16 values.
+// The XOR swizzle spreads the 16 rows that one quarter-wave reads (same chunk, consecutive rows)
+// over all LDS banks, and keeps row-contiguous writes conflict free.
+template <int BK>
+__device__ __forceinline__ int lds_off(int row, int chunk) {
+  constexpr int CPR = BK / 8;
+  return row * (BK * 2) + (((chunk ^ (row >> 1) ^ (row >> 3)) & (CPR - 1)) << 4);
+}
+
+// Linear lower-triangle tile id -> (ti, tj) with tj <= ti.  ti = floor((sqrt(8 pid + 1) - 1) / 2),
+// fixed up with integer arithmetic so float rounding can never produce tj > ti.
+__device__ __forceinline__ void tri_decode(int pid, int& ti, int& tj) {
+  int t = (int)((sqrtf(8.0f * (float)pid + 1.0f) - 1.0f) * 0.5f);
+  while ((t + 1) * (t + 2) / 2 <= pid) ++t;
+  while (t * (t + 1) / 2 > pid) --t;
+  ti = t;
+  tj = pid - t * (t + 1) / 2;
+}
+
+__device__ __forceinline__ uint32_t dword_of(const uint4& v, int c) {
+  return c == 0 ? v.x : (c == 1 ? v.y : (c == 2 ? v.z : v.w));
+}
+
+// ---------------------------------------------------------------------------------------------
+// Global -> register -> LDS tile loaders.  ROWS x BK bf16 tile, NT threads.
+// ---------------------------------------------------------------------------------------------
+template <int ROWS, int BK, int NT, bool KS>
+struct TileLoader;
+
+// K-contiguous source: 16-byte chunks copied straight through.
+template <int ROWS, int BK, int NT>
+struct TileLoader<ROWS, BK, NT, false> {
+  static constexpr int CPR = BK / 8;
+  static constexpr int NCH = (ROWS * CPR + NT - 1) / NT;
+  uint4 r[NCH];
+
+  __device__ __forceinline__ void load(const uint16_t* __restrict__ base, int64_t ld, int row0, int k0, int R,
+                                       int K, int tid) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      int ch = tid + i * NT;
+      int row = ch / CPR, kc = ch % CPR;
+      int gr = row0 + row, gk = k0 + kc * 8;
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      if (ch < ROWS * CPR && gr < R && gk < K) v = *reinterpret_cast<const uint4*>(base + (int64_t)gr * ld + gk);
+      r[i] = v;
+    }
+  }
+  __device__ __forceinline__ void store(char* lds, int tid) const {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      int ch = tid + i * NT;
+      int row = ch / CPR, kc = ch % CPR;
+      if (ch < ROWS * CPR) *reinterpret_cast<uint4*>(lds + lds_off<BK>(row, kc)) = r[i];
+    }
+  }
+};
+
+// K-strided source: each thread owns 8(k) x 8(rows) blocks, transposes them in registers.
+template <int ROWS, int BK, int NT>
+struct TileLoader<ROWS, BK, NT, true> {
+  static constexpr int KB = BK / 8;
+  static constexpr int NBLK = (ROWS / 8) * KB;
+  static constexpr int NB = (NBLK + NT - 1) / NT;
+  uint4 r[NB][8];
+
+  __device__ __forceinline__ static void decode(int idx, int& rb, int& kb) {
+    // 8 consecutive lanes walk along the contiguous (row) dimension: 128-byte global segments.
+    int rb_lo = idx & 7;
+    kb = (idx >> 3) % KB;
+    int rb_hi = (idx >> 3) / KB;
+    rb = rb_hi * 8 + rb_lo;
+  }
+  __device__ __forceinline__ void load(const uint16_t* __restrict__ base, int64_t ld, int row0, int k0, int R,
+                                       int K, int tid) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      int rb, kb;
+      decode(tid + i * NT, rb, kb);
+      int gr = row0 + rb * 8;
+      bool ok = (tid + i * NT) < NBLK && gr < R;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        int gk = k0 + kb * 8 + e;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (ok && gk < K) v = *reinterpret_cast<const uint4*>(base + (int64_t)gk * ld + gr);
+        r[i][e] = v;
+      }
+    }
+  }
+  __device__ __forceinline__ void store(char* lds, int tid) const {
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      int rb, kb;
+      decode(tid + i * NT, rb, kb);
+      if ((tid + i * NT) >= NBLK) continue;
+      // r[i][e] dword c = (x[k=e][row 2c], x[k=e][row 2c+1]); output chunk for row j = x[k=0..7][row j].
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        uint32_t lo[4], hi[4];
+#pragma unroll
+        for (int pr = 0; pr < 4; ++pr) {
+          uint32_t ka = dword_of(r[i][2 * pr], c);
+          uint32_t kbv = dword_of(r[i][2 * pr + 1], c);
+          lo[pr] = __builtin_amdgcn_perm(kbv, ka, 0x05040100u);  // (ka.lo16, kb.lo16)
+          hi[pr] = __builtin_amdgcn_perm(kbv, ka, 0x07060302u);  // (ka.hi16, kb.hi16)
+        }
+        int row_even = rb * 8 + 2 * c;
+        *reinterpret_cast<uint4*>(lds + lds_off<BK>(row_even, kb)) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+        *reinterpret_cast<uint4*>(lds + lds_off<BK>(row_even + 1, kb)) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+      }
+    }
+  }
+};
+
+__device__ __forceinline__ f32x4_t load_bf16x4_as_f32(const uint16_t* p) {
+  uint2 raw = *reinterpret_cast<const uint2*>(p);
+  f32x4_t v;
+  v[0] = __uint_as_float(raw.x << 16);
+  v[1] = __uint_as_float(raw.x & 0xffff0000u);
+  v[2] = __uint_as_float(raw.y << 16);
+  v[3] = __uint_as_float(raw.y & 0xffff0000u);
+  return v;
+}
+
+// ---------------------------------------------------------------------------------------------
+// The kernel.  grid = (tiles, batch); block = WGM*WGN wavefronts; dynamic LDS = 2 stages.
+// ---------------------------------------------------------------------------------------------
+template <int BM, int BN, int BK, int WGM, int WGN, bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
+__global__ void __launch_bounds__(WGM* WGN * 64) gemm_bf16_kernel(GemmParams p) {
+  constexpr int NT = WGM * WGN * 64;
+  constexpr int TM = BM / WGM, TN = BN / WGN;
+  constexpr int FM = TM / 32, FN = TN / 32;
+  constexpr int P_BYTES = BM * BK * 2, Q_BYTES = BN * BK * 2, STAGE = P_BYTES + Q_BYTES;
+  static_assert(TM % 32 == 0 && TN % 32 == 0 && BK % 16 == 0, "tile shape");
+  static_assert(MODE != MODE_SYRK || BM == BN, "SYRK needs square tiles");
+
+  extern __shared__ __align__(16) char smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave % WGM, wn = wave / WGM;
+  const int64_t batch = blockIdx.y;
+
+  int tm, tn;
+  if (MODE == MODE_SYRK) {
+    tri_decode((int)blockIdx.x, tm, tn);
+  } else {
+    tm = (int)blockIdx.x % p.tiles_m;
+    tn = (int)blockIdx.x / p.tiles_m;
+  }
+  const int m0 = tm * BM, n0 = tn * BN;
+  const uint16_t* __restrict__ Pb = p.P + batch * p.p_bs;
+  const uint16_t* __restrict__ Qb = p.Q + batch * p.q_bs;
+
+  TileLoader<BM, BK, NT, P_KS> lp;
+  TileLoader<BN, BK, NT, Q_KS> lq;
+
+  f32x16_t acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  const int nk = (p.K + BK - 1) / BK;
+  lp.load(Pb, p.ldp, m0, 0, p.M, p.K, tid);
+  lq.load(Qb, p.ldq, n0, 0, p.N, p.K, tid);
+  lp.store(smem, tid);
+  lq.store(smem + P_BYTES, tid);
+  __syncthreads();
+
+  const int frow = lane & 31, fk = lane >> 5;
+  for (int kt = 0; kt < nk; ++kt) {
+    const char* cur = smem + (kt & 1) * STAGE;
+    char* nxt = smem + ((kt + 1) & 1) * STAGE;
+    const bool more = (kt + 1) < nk;
+    if (more) {
+      lp.load(Pb, p.ldp, m0, (kt + 1) * BK, p.M, p.K, tid);
+      lq.load(Qb, p.ldq, n0, (kt + 1) * BK, p.N, p.K, tid);
+    }
+#pragma unroll
+    for (int q = 0; q < BK / 16; ++q) {
+      bf16x8_t fp[FM], fq[FN];
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+        fp[i] = *reinterpret_cast<const bf16x8_t*>(cur + lds_off<BK>(wm * TM + i * 32 + frow, 2 * q + fk));
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+        fq[j] = *reinterpret_cast<const bf16x8_t*>(cur + P_BYTES + lds_off<BK>(wn * TN + j * 32 + frow, 2 * q + fk));
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fq[j], fp[i], acc[i][j], 0, 0, 0);
+    }
+    if (more) {
+      lp.store(nxt, tid);
+      lq.store(nxt + P_BYTES, tid);
+    }
+    __syncthreads();
+  }
+
+  // ------------------------------------------------------------------ epilogue
+  const float alpha = p.alpha, beta = p.beta;
+  const uint16_t* __restrict__ Cb = p.Cin ? p.Cin + batch * p.c_bs : nullptr;
+  const bool diag = (MODE == MODE_SYRK) && (tm == tn);
+#pragma unroll
+  for (int i = 0; i < FM; ++i) {
+    const int m = m0 + wm * TM + i * 32 + frow;
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = n0 + wn * TN + j * 32 + 8 * g + 4 * fk;
+        if (m >= p.M || n >= p.N) continue;
+        f32x4_t v;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][4 * g + r];
+        if (beta != 0.0f) {
+          f32x4_t c = load_bf16x4_as_f32(Cb + (int64_t)m * p.ldc + n);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) v[r] = __builtin_fmaf(beta, c[r], v[r]);
+        }
+        if (OUT_F32) {
+          float* o = reinterpret_cast<float*>(p.Out) + batch * p.o_bs + (int64_t)m * p.ldo + n;
+          f32x4_t w;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) w[r] = v[r] * p.out_scale;
+          *reinterpret_cast<f32x4_t*>(o) = w;
+        } else {
+          uint16_t* ob = reinterpret_cast<uint16_t*>(p.Out) + batch * p.o_bs;
+          bf16x4_t h = __builtin_convertvector(v, bf16x4_t);
+          if (MODE == MODE_GEMM) {
+            *reinterpret_cast<bf16x4_t*>(ob + (int64_t)m * p.ldo + n) = h;
+          } else {
+            const uint2 hb = __builtin_bit_cast(uint2, h);
+            const uint16_t e0 = (uint16_t)(hb.x & 0xffffu), e1 = (uint16_t)(hb.x >> 16);
+            const uint16_t e2 = (uint16_t)(hb.y & 0xffffu), e3 = (uint16_t)(hb.y >> 16);
+            const uint16_t ev[4] = {e0, e1, e2, e3};
+            if (!diag) {
+              *reinterpret_cast<uint2*>(ob + (int64_t)m * p.ldo + n) = hb;
+              if (!p.skip_upper) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) ob[(int64_t)(n + r) * p.ldo + m] = ev[r];
+              }
+            } else if (p.skip_upper) {
+              *reinterpret_cast<uint2*>(ob + (int64_t)m * p.ldo + n) = hb;
+            } else {
+              // Diagonal tile: the lower half is stored and mirrored, the computed upper half is
+              // dropped, so the result is symmetric bit for bit by construction.
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                if (n + r <= m) ob[(int64_t)m * p.ldo + n + r] = ev[r];
+                if (n + r < m) ob[(int64_t)(n + r) * p.ldo + m] = ev[r];
+              }
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+}  // namespace mi

@@ -1,0 +1,452 @@
+// libmi_ns.so: C ABI over the gfx950 kernels (see include/mi_ns.h for the contract of each entry).
+#include "../../include/mi_ns.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <string>
+
+#include "gemm_engine.hpp"
+#include "gemm_fast.hpp"
+
+namespace mi {
+
+static thread_local std::string g_last_error;
+
+static int fail(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return code;
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---------------------------------------------------------------------------------------------
+// Tile-shape classes.  BIG is the MFMA-bound shape (one 4-wave workgroup per CU, 128 KB of LDS);
+// MID/SMALL keep small and batched problems from launching mostly-empty tiles.
+// ---------------------------------------------------------------------------------------------
+enum TileClass { TILE_SMALL = 0, TILE_MID = 1, TILE_BIG = 2 };
+
+static TileClass pick_class(int64_t extent) {
+  if (extent >= 1024) return TILE_BIG;
+  if (extent >= 256) return TILE_MID;
+  return TILE_SMALL;
+}
+
+template <int BM, int BN, int BK, int WGM, int WGN, bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
+static int launch_one(const GemmParams& p, int64_t batch, hipStream_t stream) {
+  auto kern = gemm_bf16_kernel<BM, BN, BK, WGM, WGN, P_KS, Q_KS, MODE, OUT_F32>;
+  constexpr int LDS_BYTES = 2 * (BM + BN) * BK * 2;
+  static bool attr_set = false;  // benign race: setting the attribute twice is harmless
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "hipFuncSetAttribute(%d B LDS): %s", LDS_BYTES, hipGetErrorString(e));
+    attr_set = true;
+  }
+  GemmParams q = p;
+  q.tiles_m = (p.M + BM - 1) / BM;
+  q.tiles_n = (p.N + BN - 1) / BN;
+  int64_t tiles = (MODE == MODE_SYRK) ? (int64_t)q.tiles_m * (q.tiles_m + 1) / 2 : (int64_t)q.tiles_m * q.tiles_n;
+  if (tiles <= 0 || batch <= 0) return MI_OK;
+  if (batch > 65535) return fail(MI_ERR_UNSUPPORTED_SHAPE, "batch %lld exceeds the grid limit 65535", (long long)batch);
+  dim3 grid((unsigned)tiles, (unsigned)batch, 1), block(WGM * WGN * 64, 1, 1);
+  hipLaunchKernelGGL(kern, grid, block, LDS_BYTES, stream, q);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+  return MI_OK;
+}
+
+template <bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
+static int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream) {
+  GemmParams q = p;
+  q.tiles_m = p.M / fast::BM;
+  q.tiles_n = p.N / fast::BN;
+  const int64_t tiles = (MODE == MODE_SYRK) ? (int64_t)q.tiles_m * (q.tiles_m + 1) / 2 : (int64_t)q.tiles_m * q.tiles_n;
+  if (batch > 65535) return fail(MI_ERR_UNSUPPORTED_SHAPE, "batch %lld exceeds the grid limit 65535", (long long)batch);
+  dim3 grid((unsigned)tiles, (unsigned)batch, 1), block(fast::NT, 1, 1);
+  hipLaunchKernelGGL((gemm_fast_kernel<P_KS, Q_KS, MODE, OUT_F32>), grid, block, 0, stream, q);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+  return MI_OK;
+}
+
+static bool fast_eligible(const GemmParams& p) {
+  return p.M >= 1024 && p.N >= 1024 && p.M % fast::BM == 0 && p.N % fast::BN == 0 && p.K % fast::BK == 0 && p.K >= fast::BK;
+}
+
+template <bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
+static int launch_class(TileClass tc, const GemmParams& p, int64_t batch, hipStream_t stream) {
+  if (fast_eligible(p)) return launch_fast<P_KS, Q_KS, MODE, OUT_F32>(p, batch, stream);
+  switch (tc) {
+    case TILE_BIG:
+      return launch_one<256, 256, 64, 2, 2, P_KS, Q_KS, MODE, OUT_F32>(p, batch, stream);
+    case TILE_MID:
+      return launch_one<128, 128, 64, 2, 2, P_KS, Q_KS, MODE, OUT_F32>(p, batch, stream);
+    default:
+      return launch_one<64, 64, 64, 2, 2, P_KS, Q_KS, MODE, OUT_F32>(p, batch, stream);
+  }
+}
+
+// D = alpha * A A^T + beta * C, bf16 out.
+static int syrk_impl(const void* A, int64_t batch, int64_t n, int64_t k, int64_t a_bs, int64_t a_ld, int a_trans,
+                     const void* C, int64_t c_bs, int64_t c_ld, float alpha, float beta, void* D, int64_t d_bs,
+                     int64_t d_ld, int skip_upper, hipStream_t stream) {
+  if (!A || !D) return fail(MI_ERR_BAD_ARG, "mi_syrk_bf16: A and D must not be null");
+  if (batch < 0 || n < 0 || k < 0) return fail(MI_ERR_BAD_ARG, "mi_syrk_bf16: negative extent");
+  if (beta != 0.0f && !C) return fail(MI_ERR_BAD_ARG, "mi_syrk_bf16: C is null but beta != 0");
+  if (n % 8 || k % 8) return fail(MI_ERR_UNSUPPORTED_SHAPE, "N and K must be multiples of 8, got N=%lld, K=%lld", (long long)n, (long long)k);
+  if (a_ld % 8 || d_ld % 8 || a_bs % 8 || d_bs % 8 || (C && (c_ld % 8 || c_bs % 8)))
+    return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_syrk_bf16: leading dimensions and batch strides must be multiples of 8");
+  if (!aligned16(A) || !aligned16(D) || (C && !aligned16(C)))
+    return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_syrk_bf16: pointers must be 16-byte aligned");
+  if (a_ld < (a_trans ? n : k) || d_ld < n || (C && c_ld < n)) return fail(MI_ERR_BAD_ARG, "mi_syrk_bf16: leading dimension too small");
+  if (n > (1 << 30) || k > (1 << 30)) return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_syrk_bf16: extent too large");
+  if (batch == 0 || n == 0) return MI_OK;
+
+  GemmParams p{};
+  p.P = p.Q = static_cast<const uint16_t*>(A);
+  p.ldp = p.ldq = a_ld;
+  p.p_bs = p.q_bs = a_bs;
+  p.Cin = (beta != 0.0f) ? static_cast<const uint16_t*>(C) : nullptr;
+  p.ldc = c_ld;
+  p.c_bs = c_bs;
+  p.Out = D;
+  p.ldo = d_ld;
+  p.o_bs = d_bs;
+  p.M = p.N = (int)n;
+  p.K = (int)k;
+  p.alpha = alpha;
+  p.beta = beta;
+  p.out_scale = 1.0f;
+  p.skip_upper = skip_upper ? 1 : 0;
+  TileClass tc = pick_class(n);
+  return a_trans ? launch_class<true, true, MODE_SYRK, false>(tc, p, batch, stream)
+                 : launch_class<false, false, MODE_SYRK, false>(tc, p, batch, stream);
+}
+
+// Xout = beta * X + alpha * (Bm X)
+static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void* X, int64_t x_bs,
+                          int64_t x_ld, int x_trans, void* Xout, int64_t o_bs, int64_t o_ld, int64_t batch,
+                          int64_t m, int64_t n, float alpha, float beta, int out_fp32, float out_scale,
+                          hipStream_t stream) {
+  if (!Bm || !X || !Xout) return fail(MI_ERR_BAD_ARG, "mi_gemm_axpy_bf16: null pointer");
+  if (batch < 0 || m < 0 || n < 0) return fail(MI_ERR_BAD_ARG, "mi_gemm_axpy_bf16: negative extent");
+  if (m % 8 || n % 8) return fail(MI_ERR_UNSUPPORTED_SHAPE, "M and N must be multiples of 8, got M=%lld, N=%lld", (long long)m, (long long)n);
+  if (b_ld % 8 || x_ld % 8 || b_bs % 8 || x_bs % 8 || o_ld % 4 || o_bs % 4)
+    return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_gemm_axpy_bf16: leading dimensions and batch strides must be multiples of 8");
+  if (!aligned16(Bm) || !aligned16(X) || !aligned16(Xout))
+    return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_gemm_axpy_bf16: pointers must be 16-byte aligned");
+  const int64_t x_inner = x_trans ? m : n;
+  if (b_ld < m || x_ld < x_inner || o_ld < x_inner) return fail(MI_ERR_BAD_ARG, "mi_gemm_axpy_bf16: leading dimension too small");
+  if (m > (1 << 30) || n > (1 << 30)) return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_gemm_axpy_bf16: extent too large");
+  if (batch == 0 || m == 0 || n == 0) return MI_OK;
+
+  GemmParams p{};
+  p.Cin = (beta != 0.0f) ? static_cast<const uint16_t*>(X) : nullptr;
+  p.ldc = x_ld;
+  p.c_bs = x_bs;
+  p.Out = Xout;
+  p.ldo = o_ld;
+  p.o_bs = o_bs;
+  p.K = (int)m;
+  p.alpha = alpha;
+  p.beta = beta;
+  p.out_scale = out_scale;
+  TileClass tc = pick_class(m);
+  if (!x_trans) {
+    // OUT (m x n): P = Bm rows (K-contiguous), Q[j][k] = X[k][j] (K-strided).
+    p.P = static_cast<const uint16_t*>(Bm);
+    p.ldp = b_ld;
+    p.p_bs = b_bs;
+    p.Q = static_cast<const uint16_t*>(X);
+    p.ldq = x_ld;
+    p.q_bs = x_bs;
+    p.M = (int)m;
+    p.N = (int)n;
+    return out_fp32 ? launch_class<false, true, MODE_GEMM, true>(tc, p, batch, stream)
+                    : launch_class<false, true, MODE_GEMM, false>(tc, p, batch, stream);
+  }
+  // Memory holds X^T (n x m): OUT^T[j][i] = sum_k X^T[j][k] * Bm[i][k], both operands K-contiguous.
+  p.P = static_cast<const uint16_t*>(X);
+  p.ldp = x_ld;
+  p.p_bs = x_bs;
+  p.Q = static_cast<const uint16_t*>(Bm);
+  p.ldq = b_ld;
+  p.q_bs = b_bs;
+  p.M = (int)n;
+  p.N = (int)m;
+  return out_fp32 ? launch_class<false, false, MODE_GEMM, true>(tc, p, batch, stream)
+                  : launch_class<false, false, MODE_GEMM, false>(tc, p, batch, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Frobenius normalisation: a sum-of-squares pass that leaves one partial per workgroup, and a
+// scale/cast pass whose workgroups each re-add those partials in a fixed order (deterministic,
+// no atomics, no extra launch for the final reduction).
+// ---------------------------------------------------------------------------------------------
+static constexpr int NORM_THREADS = 256;
+static constexpr int NORM_MAX_BLOCKS = 1024;  // partials per matrix
+
+static int norm_blocks(int64_t numel) {
+  int64_t vec = numel / 4;  // float4 units
+  int64_t want = (vec + (int64_t)NORM_THREADS * 8 - 1) / ((int64_t)NORM_THREADS * 8);
+  if (want < 1) want = 1;
+  if (want > NORM_MAX_BLOCKS) want = NORM_MAX_BLOCKS;
+  return (int)want;
+}
+
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  return v;
+}
+
+template <typename T>
+__device__ __forceinline__ T block_sum(T v, T* scratch) {
+  v = wave_sum(v);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  T total = 0;
+  if (threadIdx.x == 0) {
+    for (int w = 0; w < NORM_THREADS / 64; ++w) total += scratch[w];
+    scratch[0] = total;
+  }
+  __syncthreads();
+  total = scratch[0];
+  __syncthreads();
+  return total;
+}
+
+template <bool F64>
+__global__ void __launch_bounds__(NORM_THREADS) sumsq_kernel(const float* __restrict__ x, int64_t numel,
+                                                             double* __restrict__ partials) {
+  const int64_t b = blockIdx.y;
+  const float4* __restrict__ xv = reinterpret_cast<const float4*>(x + b * numel);
+  const int64_t nvec = numel / 4;
+  const int64_t stride = (int64_t)gridDim.x * NORM_THREADS;
+  __shared__ double scratch_d[NORM_THREADS / 64];
+  double total;
+  if (F64) {
+    double s0 = 0, s1 = 0, s2 = 0, s3 = 0;
+    for (int64_t i = (int64_t)blockIdx.x * NORM_THREADS + threadIdx.x; i < nvec; i += stride) {
+      float4 v = xv[i];
+      s0 += (double)v.x * (double)v.x;
+      s1 += (double)v.y * (double)v.y;
+      s2 += (double)v.z * (double)v.z;
+      s3 += (double)v.w * (double)v.w;
+    }
+    total = block_sum<double>((s0 + s1) + (s2 + s3), scratch_d);
+  } else {
+    float s0 = 0, s1 = 0, s2 = 0, s3 = 0;
+    for (int64_t i = (int64_t)blockIdx.x * NORM_THREADS + threadIdx.x; i < nvec; i += stride) {
+      float4 v = xv[i];
+      s0 = __builtin_fmaf(v.x, v.x, s0);
+      s1 = __builtin_fmaf(v.y, v.y, s1);
+      s2 = __builtin_fmaf(v.z, v.z, s2);
+      s3 = __builtin_fmaf(v.w, v.w, s3);
+    }
+    // squares are formed in float32 (tiny inputs underflow exactly like a float32 reduction);
+    // the cross-thread tree is carried in float64 so the result does not depend on its shape.
+    total = block_sum<double>((double)((s0 + s1) + (s2 + s3)), scratch_d);
+  }
+  if (threadIdx.x == 0) partials[b * gridDim.x + blockIdx.x] = total;
+}
+
+template <bool F64, bool OUT_BF16>
+__global__ void __launch_bounds__(NORM_THREADS) scale_cast_kernel(const float* __restrict__ x, int64_t numel,
+                                                                  const double* __restrict__ partials, int nparts,
+                                                                  float eps, float post_scale, void* __restrict__ out,
+                                                                  float* __restrict__ dev_norm) {
+  const int64_t b = blockIdx.y;
+  __shared__ double scratch_d[NORM_THREADS / 64];
+  double s = 0;
+  for (int i = threadIdx.x; i < nparts; i += NORM_THREADS) s += partials[b * nparts + i];
+  s = block_sum<double>(s, scratch_d);
+  float divisor;
+  if (F64) {
+    divisor = (float)sqrt(s);
+  } else {
+    divisor = fmaxf(sqrtf((float)s), eps);
+  }
+  if (dev_norm && blockIdx.x == 0 && threadIdx.x == 0) dev_norm[b] = divisor;
+
+  const int64_t nvec8 = numel / 8;
+  const float4* __restrict__ xv = reinterpret_cast<const float4*>(x + b * numel);
+  const int64_t stride = (int64_t)gridDim.x * NORM_THREADS;
+  for (int64_t i = (int64_t)blockIdx.x * NORM_THREADS + threadIdx.x; i < nvec8; i += stride) {
+    float4 a = xv[2 * i], c = xv[2 * i + 1];
+    f32x4_t lo = {a.x / divisor, a.y / divisor, a.z / divisor, a.w / divisor};
+    f32x4_t hi = {c.x / divisor, c.y / divisor, c.z / divisor, c.w / divisor};
+    if (OUT_BF16) {
+      bf16x4_t hl = __builtin_convertvector(lo, bf16x4_t);
+      bf16x4_t hh = __builtin_convertvector(hi, bf16x4_t);
+      uint2 ul = __builtin_bit_cast(uint2, hl), uh = __builtin_bit_cast(uint2, hh);
+      reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(out) + b * numel)[i] = make_uint4(ul.x, ul.y, uh.x, uh.y);
+    } else {
+      f32x4_t* o = reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(out) + b * numel);
+      o[2 * i] = lo * post_scale;
+      o[2 * i + 1] = hi * post_scale;
+    }
+  }
+}
+
+static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, int f64, void* out, int out_bf16,
+                     float post_scale, double* partials, float* dev_norm, hipStream_t stream) {
+  if (!x || !out || !partials) return fail(MI_ERR_BAD_ARG, "mi_frob_normalize: null pointer");
+  if (batch < 0 || numel < 0) return fail(MI_ERR_BAD_ARG, "mi_frob_normalize: negative extent");
+  if (numel % 8) return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_frob_normalize: numel must be a multiple of 8, got %lld", (long long)numel);
+  if (!aligned16(x) || !aligned16(out)) return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_frob_normalize: pointers must be 16-byte aligned");
+  if (batch > 65535) return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_frob_normalize: batch exceeds 65535");
+  if (batch == 0 || numel == 0) return MI_OK;
+  const int nb = norm_blocks(numel);
+  dim3 grid1(nb, (unsigned)batch), block(NORM_THREADS);
+  if (f64)
+    hipLaunchKernelGGL(sumsq_kernel<true>, grid1, block, 0, stream, x, numel, partials);
+  else
+    hipLaunchKernelGGL(sumsq_kernel<false>, grid1, block, 0, stream, x, numel, partials);
+  int64_t want = (numel / 8 + (int64_t)NORM_THREADS * 4 - 1) / ((int64_t)NORM_THREADS * 4);
+  if (want < 1) want = 1;
+  if (want > 4096) want = 4096;
+  dim3 grid2((unsigned)want, (unsigned)batch);
+#define MI_SC(F, B) hipLaunchKernelGGL((scale_cast_kernel<F, B>), grid2, block, 0, stream, x, numel, partials, nb, eps, post_scale, out, dev_norm)
+  if (f64) {
+    if (out_bf16) MI_SC(true, true); else MI_SC(true, false);
+  } else {
+    if (out_bf16) MI_SC(false, true); else MI_SC(false, false);
+  }
+#undef MI_SC
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "mi_frob_normalize launch failed: %s", hipGetErrorString(e));
+  return MI_OK;
+}
+
+static size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+struct NsWorkspace {
+  size_t x0, x1, a, b, partials, norm, total;
+};
+
+static NsWorkspace ns_layout(int64_t batch, int64_t rows, int64_t cols) {
+  const int64_t m = rows < cols ? rows : cols;
+  NsWorkspace w{};
+  size_t off = 0;
+  const size_t xbytes = align_up((size_t)batch * rows * cols * 2, 256);
+  const size_t gbytes = align_up((size_t)batch * m * m * 2, 256);
+  w.x0 = off; off += xbytes;
+  w.x1 = off; off += xbytes;
+  w.a = off; off += gbytes;
+  w.b = off; off += gbytes;
+  w.partials = off; off += align_up((size_t)batch * NORM_MAX_BLOCKS * sizeof(double), 256);
+  w.norm = off; off += align_up((size_t)batch * sizeof(float), 256);
+  w.total = off;
+  return w;
+}
+
+}  // namespace mi
+
+using namespace mi;
+
+extern "C" {
+
+int mi_version(void) { return 100; }
+
+const char* mi_last_error(void) { return g_last_error.c_str(); }
+
+int mi_syrk_bf16(const void* A, int64_t batch, int64_t n, int64_t k, int64_t a_batch_stride, int64_t a_ld, int a_trans,
+                 const void* C, int64_t c_batch_stride, int64_t c_ld, float alpha, float beta, void* D,
+                 int64_t d_batch_stride, int64_t d_ld, int skip_upper, void* stream) {
+  return syrk_impl(A, batch, n, k, a_batch_stride, a_ld, a_trans, C, c_batch_stride, c_ld, alpha, beta, D,
+                   d_batch_stride, d_ld, skip_upper, static_cast<hipStream_t>(stream));
+}
+
+int mi_gemm_axpy_bf16(const void* Bm, int64_t b_batch_stride, int64_t b_ld, const void* X,
+                      int64_t x_batch_stride, int64_t x_ld, int x_trans, void* Xout, int64_t o_batch_stride,
+                      int64_t o_ld, int64_t batch, int64_t m, int64_t n, float alpha, float beta, int out_fp32,
+                      float out_scale, void* stream) {
+  return gemm_axpy_impl(Bm, b_batch_stride, b_ld, X, x_batch_stride, x_ld, x_trans, Xout, o_batch_stride,
+                        o_ld, batch, m, n, alpha, beta, out_fp32, out_scale, static_cast<hipStream_t>(stream));
+}
+
+size_t mi_frob_partials_len(int64_t batch, int64_t numel) {
+  (void)numel;
+  return (size_t)(batch < 0 ? 0 : batch) * NORM_MAX_BLOCKS;
+}
+
+int mi_frob_normalize(const float* x, int64_t batch, int64_t numel, float eps, int accumulate_fp64, void* out,
+                      int out_bf16, double* partials, float* dev_norm, void* stream) {
+  return frob_impl(x, batch, numel, eps, accumulate_fp64, out, out_bf16, 1.0f, partials, dev_norm,
+                   static_cast<hipStream_t>(stream));
+}
+
+size_t mi_newton_schulz_workspace_bytes(int64_t batch, int64_t rows, int64_t cols) {
+  if (batch <= 0 || rows <= 0 || cols <= 0) return 0;
+  return ns_layout(batch, rows, cols).total;
+}
+
+int mi_newton_schulz_bf16(const float* x, float* out, int64_t batch, int64_t rows, int64_t cols, const float* abc,
+                          int steps, float eps, int accumulate_fp64, float out_scale, void* workspace,
+                          size_t workspace_bytes, void* stream_v) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_v);
+  if (!x || !out) return fail(MI_ERR_BAD_ARG, "mi_newton_schulz_bf16: null tensor pointer");
+  if (batch < 0 || rows < 0 || cols < 0 || steps < 0) return fail(MI_ERR_BAD_ARG, "mi_newton_schulz_bf16: negative argument");
+  if (steps > 0 && !abc) return fail(MI_ERR_BAD_ARG, "mi_newton_schulz_bf16: abc is null");
+  if (rows % 8 || cols % 8)
+    return fail(MI_ERR_UNSUPPORTED_SHAPE, "rows and cols must be multiples of 8, got %lld x %lld", (long long)rows, (long long)cols);
+  if (batch == 0 || rows == 0 || cols == 0) return MI_OK;
+  const NsWorkspace w = ns_layout(batch, rows, cols);
+  if (!workspace || workspace_bytes < w.total)
+    return fail(MI_ERR_WORKSPACE, "workspace too small: need %zu bytes, got %zu", w.total, workspace_bytes);
+  if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(MI_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+
+  char* ws = static_cast<char*>(workspace);
+  uint16_t* xbuf[2] = {reinterpret_cast<uint16_t*>(ws + w.x0), reinterpret_cast<uint16_t*>(ws + w.x1)};
+  uint16_t* gram = reinterpret_cast<uint16_t*>(ws + w.a);
+  uint16_t* poly = reinterpret_cast<uint16_t*>(ws + w.b);
+  double* partials = reinterpret_cast<double*>(ws + w.partials);
+  float* norm = reinterpret_cast<float*>(ws + w.norm);
+
+  const int64_t numel = rows * cols;
+  if (steps == 0)
+    return frob_impl(x, batch, numel, eps, accumulate_fp64, out, /*out_bf16=*/0, out_scale, partials, norm, stream);
+
+  int rc = frob_impl(x, batch, numel, eps, accumulate_fp64, xbuf[0], /*out_bf16=*/1, 1.0f, partials, norm, stream);
+  if (rc != MI_OK) return rc;
+
+  // The iteration runs on the (m x n) orientation with m <= n.  When rows > cols that orientation is
+  // the transpose of what memory holds, which the kernels read in place (a_trans / x_trans).
+  const int trans = rows > cols;
+  const int64_t m = trans ? cols : rows, n = trans ? rows : cols;
+  const int64_t ld = cols;  // row-major (rows x cols) in memory either way
+  const int64_t x_bs = numel, g_bs = m * m;
+  int cur = 0;
+  for (int s = 0; s < steps; ++s) {
+    const float a = abc[3 * s], b = abc[3 * s + 1], c = abc[3 * s + 2];
+    const bool last = (s + 1 == steps);
+    rc = syrk_impl(xbuf[cur], batch, m, n, x_bs, ld, trans, nullptr, 0, m, 1.0f, 0.0f, gram, g_bs, m, 0, stream);
+    if (rc != MI_OK) return rc;
+    const uint16_t* mult = gram;
+    float alpha = b;
+    if (c != 0.0f) {
+      rc = syrk_impl(gram, batch, m, m, g_bs, m, 0, gram, g_bs, m, c, b, poly, g_bs, m, 0, stream);
+      if (rc != MI_OK) return rc;
+      mult = poly;
+      alpha = 1.0f;
+    }
+    void* dst = last ? static_cast<void*>(out) : static_cast<void*>(xbuf[cur ^ 1]);
+    rc = gemm_axpy_impl(mult, g_bs, m, xbuf[cur], x_bs, ld, trans, dst, x_bs, ld, batch, m, n, alpha, a,
+                        last ? 1 : 0, last ? out_scale : 1.0f, stream);
+    if (rc != MI_OK) return rc;
+    cur ^= 1;
+  }
+  return MI_OK;
+}
+
+}  // extern "C"

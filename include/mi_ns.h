@@ -1,0 +1,128 @@
+/*
+ * mi_ns.h - C ABI of libmi_ns.so: bf16 SYRK, GEMM+AXPY, Frobenius normalisation and the
+ * Newton-Schulz orthogonalisation driver for AMD MI355X (gfx950).
+ *
+ * The reference project (NVIDIA-NeMo/Emerging-Optimizers) is pure Python and has no FFI for this
+ * path; each entry point below names the Python call site(s) of the reference that it stands
+ * in for.  All pointers are DEVICE pointers owned by the caller.  Unless stated otherwise the
+ * library allocates nothing, never synchronises the host, and enqueues its kernels on `stream`
+ * (a hipStream_t passed as void*; NULL is the legacy default stream).
+ *
+ * Conventions
+ *   - bf16 data are raw 16-bit words (bfloat16 bit patterns).
+ *   - Leading dimensions (`*_ld`) and batch strides are in ELEMENTS, not bytes.
+ *   - Every bf16 matrix must have its contiguous dimension a multiple of 8 elements, `*_ld` a
+ *     multiple of 8 and a 16-byte aligned base pointer (16-byte vector loads).  Violations return
+ *     MI_ERR_UNSUPPORTED_SHAPE; the host wrapper turns that into the exception the reference raises.
+ *   - Return value: MI_OK (0) or a negative MI_ERR_* code; mi_last_error() gives the text.
+ */
+#ifndef MI_NS_H_
+#define MI_NS_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI_OK 0
+#define MI_ERR_BAD_ARG (-1)
+#define MI_ERR_UNSUPPORTED_SHAPE (-2)
+#define MI_ERR_LAUNCH (-3)
+#define MI_ERR_WORKSPACE (-4)
+
+/* Library version (major*10000 + minor*100 + patch). */
+int mi_version(void);
+
+/* Thread-local text of the last error returned on this host thread ("" if none). */
+const char* mi_last_error(void);
+
+/*
+ * D[b] = alpha * A[b] * A[b]^T + beta * C[b]      (bf16 in, fp32 accumulate, bf16 out)
+ *
+ * Replaces: tsyrk_ex              emerging_optimizers/triton_kernels/syrk.py:335-408
+ *           tsyrk_ex_small_matrix emerging_optimizers/triton_kernels/syrk.py:411-500
+ *           batched_tsyrk_ex      emerging_optimizers/triton_kernels/batched_syrk.py:266-363
+ * (one kernel family; batch == 1 is the 2-D case).
+ *
+ * A[b] is logically (n, k).  a_trans == 0: memory holds A[b] row-major, element (i, p) at
+ * A + b*a_batch_stride + i*a_ld + p.  a_trans != 0: memory holds A[b]^T row-major, element (i, p)
+ * at A + b*a_batch_stride + p*a_ld + i  (the reference's TRANS constexpr, syrk.py:200-207).
+ * C[b] is (n, n), must be symmetric, may be NULL iff beta == 0.  D[b] is (n, n) row-major.
+ * Only lower-triangle tiles are computed; every strictly-lower element is also stored at its
+ * mirrored position unless skip_upper != 0, so D[b] is bitwise symmetric (syrk.py:221-224).
+ * D may alias neither A nor C.
+ */
+int mi_syrk_bf16(const void* A, int64_t batch, int64_t n, int64_t k,
+                 int64_t a_batch_stride, int64_t a_ld, int a_trans,
+                 const void* C, int64_t c_batch_stride, int64_t c_ld,
+                 float alpha, float beta,
+                 void* D, int64_t d_batch_stride, int64_t d_ld,
+                 int skip_upper, void* stream);
+
+/*
+ * Xout[b] = beta * X[b] + alpha * (Bm[b] * X[b])      (bf16 in, fp32 accumulate)
+ *
+ * Replaces the third product of a Newton-Schulz step:
+ *   torch.addmm(X, B, X, alpha=1.0, beta=a) / torch.addmm(X, A, X, alpha=b, beta=a)
+ *     emerging_optimizers/orthogonalized_optimizers/muon_utils.py:374-377, 438-441
+ *   torch.baddbmm twins   muon_utils.py:407-410, 472-475
+ *
+ * Bm[b] is (m, m) row-major (b_ld).  X[b] is logically (m, n).  x_trans == 0: X[b] and Xout[b]
+ * are row-major (m, n), element (i, j) at i*ld + j.  x_trans != 0: memory holds X[b]^T and
+ * Xout[b]^T row-major (n, m), element (i, j) at j*ld + i (the layout a tall parameter has after the
+ * `.mT` view of muon_utils.py:207-208).  Bm need not be symmetric.
+ * out_fp32 == 0: Xout is bf16.  out_fp32 != 0: Xout is float32 and is additionally multiplied by
+ * out_scale (folds the final `.to(float32)` of muon_utils.py:269 and the Muon scale factor of
+ * muon.py:131-132 into the epilogue).  Xout must not alias X or Bm.
+ */
+int mi_gemm_axpy_bf16(const void* Bm, int64_t b_batch_stride, int64_t b_ld,
+                      const void* X, int64_t x_batch_stride, int64_t x_ld, int x_trans,
+                      void* Xout, int64_t o_batch_stride, int64_t o_ld,
+                      int64_t batch, int64_t m, int64_t n,
+                      float alpha, float beta, int out_fp32, float out_scale, void* stream);
+
+/*
+ * Per-matrix Frobenius normalisation of a float32 batch, result cast to bf16 or kept float32:
+ *   accumulate_fp64 == 0:  out[b] = x[b] / max(||x[b]||_F, eps)      (sum of squares in float32)
+ *   accumulate_fp64 != 0:  out[b] = x[b] / float(||x[b]||_F in fp64) (no eps clamp)
+ *
+ * Replaces: torch.nn.functional.normalize(x, p=2, dim=(-2,-1), eps)   muon_utils.py:216
+ *           the float64 vector_norm variant                           muon_utils.py:221-222
+ *           X.to(torch.bfloat16)                                      muon_utils.py:262
+ *
+ * x[b] is `numel` contiguous float32 values at x + b*numel (any 2-D shape: the norm does not
+ * depend on it).  out has the same element order.  numel must be a multiple of 8.
+ * partials: float64 scratch of at least mi_frob_partials_len(batch, numel) elements.
+ * dev_norm: optional (may be NULL) float32[batch] that receives the divisor actually used.
+ */
+int mi_frob_normalize(const float* x, int64_t batch, int64_t numel, float eps, int accumulate_fp64,
+                      void* out, int out_bf16, double* partials, float* dev_norm, void* stream);
+size_t mi_frob_partials_len(int64_t batch, int64_t numel);
+
+/*
+ * Whole Newton-Schulz orthogonalisation of a float32 batch in one call:
+ *   normalise -> bf16 -> `steps` x { A = X X^T ; B = b A + c A^2 ; X = a X + B X } -> float32 * out_scale
+ * (cubic step X = a X + b A X when c == 0), i.e. the "medium"-precision body of
+ *   newton_schulz                     muon_utils.py:149-274
+ *   (batched_)newton_schulz_step_tsyrk muon_utils.py:414-476
+ * plus the scale multiplication of Muon's closure (muon.py:131-132).
+ *
+ * x, out: float32, batch matrices of (rows, cols) row-major contiguous.  The iteration always runs on
+ * the orientation with the smaller leading dimension (muon_utils.py:205-208); no transposed copy is
+ * made, kernels for both memory orientations exist.  out must not alias x.
+ * abc: HOST array of 3*steps floats (a, b, c per step, already expanded by the coefficient iterator).
+ * steps == 0 returns the normalised input.  rows and cols must be multiples of 8.
+ * workspace: device scratch of at least mi_newton_schulz_workspace_bytes(batch, rows, cols) bytes,
+ * 256-byte aligned.
+ */
+int mi_newton_schulz_bf16(const float* x, float* out, int64_t batch, int64_t rows, int64_t cols,
+                          const float* abc, int steps, float eps, int accumulate_fp64,
+                          float out_scale, void* workspace, size_t workspace_bytes, void* stream);
+size_t mi_newton_schulz_workspace_bytes(int64_t batch, int64_t rows, int64_t cols);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI_NS_H_ */

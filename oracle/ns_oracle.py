@@ -1,0 +1,316 @@
+"""CPU oracle for the Muon orthogonalisation path -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+
+A plain numpy restatement of what NVIDIA-NeMo/Emerging-Optimizers computes on this path.  Only
+``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may import it; the
+package under ``emerging-optimizers_amd/`` never does.
+
+Every function cites the reference lines it follows (paths relative to the reference checkout).
+How each one is pinned (``tests/test_oracle.py``):
+
+* coefficient tables        -- literal constants; fixed-point identities p(1) of three tables
+* coefficient_iterator      -- closed form ``sets[i % L]`` / ``sets[min(i, L-1)]``
+* newton_schulz (fp32/fp64) -- SVD closed form: singular vectors are invariant, singular values follow
+                               the scalar recurrence ``s <- a s + b s^3 + c s^5`` (``svd_polynomial``)
+* newton_schulz_step        -- same closed form with one step; cubic case against ``a x + b (x x^T) x``
+* syrk / gemm_axpy          -- brute-force Python loops on tiny integer inputs (exact arithmetic)
+* round_to_bf16             -- exhaustive comparison with the IEEE definition on a value sweep incl. ties
+* muon_scale_factor         -- ``math.sqrt`` closed forms
+* optimizer step            -- equals textbook SGD / SGD-with-momentum updates on integer data
+* tri_decode                -- brute-force bijection onto ``{(i, j): j <= i < T}``
+
+The reference itself holds no stored golden vectors for this path (all of its expectations are computed at
+test time), so the checks above are what anchors this file.
+"""
+
+from __future__ import annotations
+
+import itertools
+import math
+from typing import Iterator, Sequence
+
+import numpy as np
+
+
+# --------------------------------------------------------------------------------------------
+# Coefficient tables: emerging_optimizers/orthogonalized_optimizers/muon_utils.py:30-90 (data).
+# --------------------------------------------------------------------------------------------
+COEFFICIENT_SETS: dict[str, list[tuple[float, float, float]]] = {
+    "simple": [(3.4445, -4.7750, 2.0315)],
+    "quintic": [
+        (4.0848, -6.8946, 2.9270),
+        (3.9505, -6.3029, 2.6377),
+        (3.7418, -5.5913, 2.3037),
+        (2.8769, -3.1427, 1.2046),
+        (2.8366, -3.0525, 1.2012),
+    ],
+    "polar_express": [
+        (8.2051, -22.9019, 16.4607),
+        (4.0664, -2.8612, 0.5184),
+        (3.9096, -2.8234, 0.5250),
+        (3.2856, -2.4153, 0.4853),
+        (2.2779, -1.6198, 0.3985),
+        (1.8726, -1.2307, 0.3585),
+        (1.8564, -1.2132, 0.3568),
+        (1.8750, -1.2500, 0.3750),
+    ],
+    "cans": [
+        (8.4703, -25.1081, 18.6293),
+        (4.1828, -3.1087, 0.5806),
+        (3.9619, -2.9541, 0.5630),
+        (3.2866, -2.4647, 0.5074),
+        (2.2737, -1.6447, 0.4162),
+    ],
+    "aol": [
+        (4.0098, -7.0585, 2.4635),
+        (3.4585, -5.5479, 2.5959),
+        (2.7573, -3.2939, 1.4254),
+        (2.7215, -3.0494, 1.3169),
+    ],
+    "deepseekv4": [(3.4445, -4.7750, 2.0315)] * 8 + [(2.0, -1.5, 0.5)] * 2,
+    "cubic5": [
+        (3.3656576, -3.3420992, 0.0),
+        (2.5744352, -1.4957376, 0.0),
+        (2.5368962, -1.4312570, 0.0),
+        (2.4418906, -1.2764040, 0.0),
+        (2.2230472, -0.9630650, 0.0),
+    ],
+}
+
+# muon_utils.py:239-240: these families keep repeating their last tuple, the others cycle.
+REPEAT_LAST_TYPES = ("polar_express", "cans", "deepseekv4")
+
+
+def coefficient_iterator(steps: int, sets: Sequence[tuple[float, float, float]], mode: str = "cycle") -> Iterator:
+    """muon_utils.py:93-129.  ``cycle``: sets[i % L]; ``repeat_last``: sets[min(i, L-1)]."""
+    if not sets:
+        raise ValueError("coefficient_sets must be non-empty.")
+    if mode not in ("cycle", "repeat_last"):
+        raise ValueError(f"Invalid mode: {mode}. Expected 'cycle' or 'repeat_last'.")
+    n = len(sets)
+    for i in range(steps):
+        yield sets[i % n] if mode == "cycle" else sets[min(i, n - 1)]
+
+
+def expand_coefficients(steps: int, coefficient_type: str, custom=None) -> list[tuple[float, float, float]]:
+    """Table lookup + iteration mode of muon_utils.py:224-241 as a flat list of ``steps`` tuples."""
+    if coefficient_type in COEFFICIENT_SETS:
+        sets = COEFFICIENT_SETS[coefficient_type]
+    elif coefficient_type == "custom":
+        if custom is None:
+            raise ValueError("custom_coefficient_sets must be provided when coefficient_type is 'custom'.")
+        sets = custom
+    else:
+        raise ValueError(f"Invalid coefficient type: {coefficient_type}")
+    if coefficient_type == "cubic5" and steps != len(sets):
+        raise ValueError(f"cubic5 is a fixed {len(sets)}-step schedule; got steps={steps}. Use steps=5.")
+    mode = "repeat_last" if coefficient_type in REPEAT_LAST_TYPES else "cycle"
+    return list(coefficient_iterator(steps, sets, mode))
+
+
+# --------------------------------------------------------------------------------------------
+# bfloat16 emulation (numpy has no bf16): round-to-nearest-even on the upper 16 bits of float32.
+# --------------------------------------------------------------------------------------------
+def round_to_bf16(x: np.ndarray) -> np.ndarray:
+    """float32 -> nearest bfloat16 (ties to even), returned as float32.  NaN stays NaN."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32).astype(np.uint64)
+    rounded = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    out = rounded.astype(np.uint32).view(np.float32).reshape(x.shape)
+    return np.where(np.isnan(x), x, out)
+
+
+def _mT(x: np.ndarray) -> np.ndarray:
+    return np.swapaxes(x, -1, -2)
+
+
+# --------------------------------------------------------------------------------------------
+# SYRK and the AXPY-GEMM as the reference defines them.
+# --------------------------------------------------------------------------------------------
+def syrk(a: np.ndarray, c: np.ndarray | None = None, alpha: float = 1.0, beta: float = 0.0) -> np.ndarray:
+    """``bf16(alpha * a a^T + beta * c)`` with float32 accumulation and float32 epilogue.
+
+    triton_kernels/syrk.py:198-215 (2-D) and triton_kernels/batched_syrk.py:203-224 (batched): the product
+    is accumulated in float32, scaled by alpha, beta*c added in float32, then rounded once to bf16.
+    ``a`` holds bf16-representable float32 values; the result is returned as float32 holding bf16 values.
+    """
+    a = np.asarray(a, dtype=np.float32)
+    acc = np.matmul(a, _mT(a))
+    acc = np.float32(alpha) * acc
+    if beta != 0.0:
+        acc = np.float32(beta) * np.asarray(c, dtype=np.float32) + acc
+    return round_to_bf16(acc)
+
+
+def gemm_axpy(bm: np.ndarray, x: np.ndarray, alpha: float, beta: float, *, round_bf16: bool = True) -> np.ndarray:
+    """``beta * x + alpha * (bm @ x)``: torch.addmm(X, B, X, alpha=alpha, beta=beta) of muon_utils.py:374-377."""
+    acc = np.matmul(np.asarray(bm, dtype=np.float32), np.asarray(x, dtype=np.float32))
+    out = np.float32(beta) * np.asarray(x, dtype=np.float32) + np.float32(alpha) * acc
+    return round_to_bf16(out) if round_bf16 else out
+
+
+# --------------------------------------------------------------------------------------------
+# Newton-Schulz.
+# --------------------------------------------------------------------------------------------
+def frobenius_normalize(x: np.ndarray, eps: float = 1e-15, in_double: bool = False) -> np.ndarray:
+    """muon_utils.py:212-222.  float32: x / max(||x||_F, eps).  double: x / float32(||x||_F) with no clamp."""
+    x = np.asarray(x, dtype=np.float32)
+    if in_double:
+        norm = np.sqrt(np.sum(x.astype(np.float64) ** 2, axis=(-2, -1), keepdims=True)).astype(np.float32)
+        return x / norm
+    norm = np.sqrt(np.sum(x * x, axis=(-2, -1), keepdims=True, dtype=np.float32))
+    return x / np.maximum(norm, np.float32(eps))
+
+
+def newton_schulz_step(x: np.ndarray, a: float, b: float, c: float, *, bf16: bool = False) -> np.ndarray:
+    """One iteration, muon_utils.py:348-378 (and its batched / SYRK twins :381-476).
+
+    ``A = X X^T``; quintic (c != 0): ``B = b A + c A A``, ``X' = a X + B X``; cubic (c == 0): ``X' = a X + b A X``.
+    With ``bf16=True`` every product is rounded to bf16 after a float32 epilogue, which is what the reference
+    executes under matmul precision "medium" (X, A and B are bf16 tensors there).
+    """
+    dt = x.dtype
+    if bf16:
+        gram = syrk(x)
+        if c != 0.0:
+            poly = syrk(gram, gram, alpha=c, beta=b)
+            return gemm_axpy(poly, x, 1.0, a)
+        return gemm_axpy(gram, x, b, a)
+    gram = np.matmul(x, _mT(x))
+    if c != 0.0:
+        poly = dt.type(b) * gram + dt.type(c) * np.matmul(gram, gram)
+        return dt.type(a) * x + np.matmul(poly, x)
+    return dt.type(a) * x + dt.type(b) * np.matmul(gram, x)
+
+
+def newton_schulz(
+    x: np.ndarray,
+    steps: int,
+    coefficient_type: str = "quintic",
+    custom_coefficient_sets=None,
+    eps: float = 1e-15,
+    transpose: bool | None = None,
+    normalize_in_double: bool = False,
+    precision: str = "highest",
+    compute_dtype=np.float32,
+) -> np.ndarray:
+    """muon_utils.py:149-274 on one process (tp_group=None).
+
+    precision "highest": float32 (or ``compute_dtype``) arithmetic throughout.
+    precision "medium" : the reference's bf16 schedule (:245-269): normalise in float32, round X to bf16,
+    iterate with bf16-rounded products, return float32.
+    """
+    x = np.asarray(x)
+    if x.ndim < 2 or x.ndim > 3:
+        raise TypeError(f"Input tensor x must be 2d or 3d (batched 2d), got {x.ndim}d")
+    if x.dtype != np.float32:
+        raise TypeError(f"Input tensor x must be in float32, got {x.dtype}")
+    if transpose is None:
+        transpose = x.shape[-2] > x.shape[-1]
+    if transpose:
+        x = _mT(x)
+    X = frobenius_normalize(x, eps, normalize_in_double)
+    coeffs = expand_coefficients(steps, coefficient_type, custom_coefficient_sets)
+    bf16 = precision == "medium"
+    if bf16:
+        X = round_to_bf16(X)
+    else:
+        X = X.astype(compute_dtype)
+    for a, b, c in coeffs:
+        X = newton_schulz_step(X, a, b, c, bf16=bf16)
+    X = X.astype(np.float32)
+    return _mT(X) if transpose else X
+
+
+def svd_polynomial(x: np.ndarray, coeffs: Sequence[tuple[float, float, float]], eps: float = 1e-15) -> np.ndarray:
+    """Closed form of the iteration in float64, independent of any matrix-product code path.
+
+    With x / ||x||_F = U diag(s) V^T, one step maps it to U diag(a s + b s^3 + c s^5) V^T, because
+    X X^T = U diag(s^2) U^T.  So the result of the whole schedule is U diag(p_k(...p_1(s))) V^T.
+    """
+    x = np.asarray(x, dtype=np.float64)
+    transpose = x.shape[-2] > x.shape[-1]
+    if transpose:
+        x = _mT(x)
+    x = x / max(np.linalg.norm(x), eps)
+    u, s, vt = np.linalg.svd(x, full_matrices=False)
+    for a, b, c in coeffs:
+        s = a * s + b * s**3 + c * s**5
+    out = (u * s) @ vt
+    return _mT(out) if transpose else out
+
+
+# --------------------------------------------------------------------------------------------
+# Muon pieces around the iteration.
+# --------------------------------------------------------------------------------------------
+def muon_scale_factor(size_out: int, size_in: int, mode: str = "spectral") -> float:
+    """orthogonalized_optimizers/muon.py:190-216."""
+    if mode == "shape_scaling":
+        return max(1, size_out / size_in) ** 0.5
+    if mode == "spectral":
+        return max(size_out, size_in) ** 0.5
+    if mode == "unit_rms_norm":
+        return (size_out / size_in) ** 0.5
+    raise ValueError(f"Invalid mode for Muon update scale factor: {mode}")
+
+
+def optimizer_step(
+    p: np.ndarray,
+    grad: np.ndarray,
+    momentum_buffer: np.ndarray,
+    *,
+    lr: float,
+    momentum: float,
+    weight_decay: float,
+    weight_decay_method: str = "decoupled",
+    nesterov: bool = False,
+    orthogonalize=lambda g: g,
+) -> tuple[np.ndarray, np.ndarray]:
+    """One parameter update of OrthogonalizedOptimizer.step, orthogonalized_optimizer.py:164-212 with the
+    weight-decay variants of mixin.py:43-56.  Returns ``(new_p, new_momentum_buffer)``; float32 throughout."""
+    f = np.float32
+    p = np.asarray(p, dtype=np.float32).copy()
+    grad = np.asarray(grad, dtype=np.float32).copy()
+    buf = np.asarray(momentum_buffer, dtype=np.float32).copy()
+    if weight_decay != 0.0:
+        if weight_decay_method == "decoupled":
+            p = p + f(-weight_decay * lr) * p
+        elif weight_decay_method == "independent":
+            p = p + f(-weight_decay) * p
+        elif weight_decay_method == "l2":
+            grad = grad + f(weight_decay) * p
+        elif weight_decay_method == "palm":
+            p = p + f(-(weight_decay * lr * lr)) * p
+        else:
+            raise ValueError(f"Invalid weight decay method: {weight_decay_method}")
+    # lerp_(grad, 1 - momentum): buf + w (grad - buf)
+    buf = buf + f(1 - momentum) * (grad - buf)
+    g = grad + f(momentum) * (buf - grad) if nesterov else buf
+    update = np.asarray(orthogonalize(g), dtype=np.float32)
+    p = p + f(-lr) * update
+    return p, buf
+
+
+def muon_orthogonalize(grad, *, steps=5, coefficient_type="quintic", scale_mode="spectral", extra_scale_factor=1.0,
+                       precision="medium"):
+    """Muon's closure, muon.py:117-132: newton_schulz(grad) * scale_factor * extra_scale_factor."""
+    orth = newton_schulz(grad, steps, coefficient_type, precision=precision)
+    scale = muon_scale_factor(grad.shape[-2], grad.shape[-1], scale_mode)
+    return orth * np.float32(scale) * np.float32(extra_scale_factor)
+
+
+# --------------------------------------------------------------------------------------------
+# Lower-triangle tile enumeration used by the triangular launch grids.
+# --------------------------------------------------------------------------------------------
+def tri_decode(pid: int) -> tuple[int, int]:
+    """Linear tile id -> (i, j), j <= i: i = floor((sqrt(8 pid + 1) - 1) / 2), j = pid - i (i + 1) / 2
+    (triton_kernels/syrk.py:285-291, batched_syrk.py:185-193), evaluated with exact integer arithmetic."""
+    i = (math.isqrt(8 * pid + 1) - 1) // 2
+    return i, pid - i * (i + 1) // 2
+
+
+def flops_sym(m: int, n: int, steps: int, batch: int = 1) -> int:
+    """Symmetric-halved FLOP count of ``steps`` quintic iterations on a batch of (m, n), m <= n."""
+    return batch * steps * (3 * m * m * n + m**3)
+
+
+__all__ = [name for name in dir() if not name.startswith("_") and name not in ("itertools", "math", "np")]
