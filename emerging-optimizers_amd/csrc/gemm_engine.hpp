@@ -38,7 +38,19 @@ struct GemmParams {
   float alpha, beta, out_scale;
   int tiles_m, tiles_n;
   int skip_upper;
+  // Diagonal-shift bookkeeping of the fused Newton-Schulz driver (all null / 0 for plain calls).
+  // The Gram matrix is stored as A' = A - s I with s ~ tr(A)/M, so that bf16 rounding acts on the small
+  // deviations of the diagonal instead of on its O(1) magnitude; the identity part is folded back into
+  // the epilogue scalars of the two kernels that consume A', which keeps the algebra exact for any s.
+  int shift_mode;            // SHIFT_*
+  float cb, cc;              // step coefficients b, c (host values)
+  const float* slots_in;     // SHIFT_GRAM: per-tile partial sums of squares of X, [batch][nslots_in]
+  int nslots_in;
+  float* shift_io;           // [batch]: written by SHIFT_GRAM, read by SHIFT_POLY / SHIFT_APPLY
+  float* slots_out;          // GEMM mode: per-tile sum of squares of the output, [batch][gridDim.x]
 };
+
+enum { SHIFT_NONE = 0, SHIFT_GRAM = 1, SHIFT_POLY = 2, SHIFT_APPLY = 3 };
 
 // Byte offset of 16-byte chunk `chunk` of row `row` in an LDS tile whose rows hold BK bf16 values.
 // The XOR swizzle spreads the 16 rows that one quarter-wave reads (same chunk, consecutive rows)
@@ -165,6 +177,123 @@ __device__ __forceinline__ f32x4_t load_bf16x4_as_f32(const uint16_t* p) {
   return v;
 }
 
+__device__ __forceinline__ float wave_sum_f32(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+// Sum over the workgroup in a fixed order (same result in every workgroup and every run).
+template <int NT>
+__device__ __forceinline__ float block_sum_f32(float v, float* red) {
+  v = wave_sum_f32(v);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float t = 0.0f;
+#pragma unroll
+  for (int w = 0; w < NT / 64; ++w) t += red[w];
+  __syncthreads();
+  return t;
+}
+
+// Resolves the diagonal shift s for this workgroup and returns the effective (alpha, beta).
+template <int NT>
+__device__ __forceinline__ float resolve_shift(const GemmParams& p, int64_t batch, float* red, float& beta) {
+  float s = 0.0f;
+  if (p.shift_mode == SHIFT_GRAM) {
+    float part = 0.0f;
+    const float* sl = p.slots_in + batch * p.nslots_in;
+    for (int i = threadIdx.x; i < p.nslots_in; i += NT) part += sl[i];
+    s = block_sum_f32<NT>(part, red) / (float)p.M;
+    if (blockIdx.x == 0 && threadIdx.x == 0) p.shift_io[batch] = s;
+  } else if (p.shift_mode == SHIFT_POLY) {
+    s = p.shift_io[batch];
+    beta = beta + 2.0f * p.cc * s;  // B' = c A'^2 + (b + 2 c s) A'
+  } else if (p.shift_mode == SHIFT_APPLY) {
+    s = p.shift_io[batch];
+    beta = beta + p.cb * s + p.cc * s * s;  // X' = (a + b s + c s^2) X + B' X
+  }
+  return s;
+}
+
+// Epilogue shared by both kernels.  A lane owns output row m = m_base + 32 i + (lane & 31) and, for each
+// (j, g), the four columns n .. n+3 with n = n_base + 32 j + 8 g + 4 (lane >> 5).
+template <int MODE, bool OUT_F32, bool GUARD, int FM, int FN, int NT>
+__device__ __forceinline__ void tile_epilogue(const GemmParams& p, f32x16_t (&acc)[FM][FN], int m_base, int n_base,
+                                              int lane, int64_t batch, bool diag, float alpha, float beta, float shift,
+                                              float* red) {
+  const int frow = lane & 31, fk = lane >> 5;
+  const uint16_t* __restrict__ Cb = p.Cin ? p.Cin + batch * p.c_bs : nullptr;
+  float ssq = 0.0f;
+#pragma unroll
+  for (int i = 0; i < FM; ++i) {
+    const int m = m_base + i * 32 + frow;
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = n_base + j * 32 + 8 * g + 4 * fk;
+        if (GUARD && (m >= p.M || n >= p.N)) continue;
+        f32x4_t v;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][4 * g + r];
+        if (beta != 0.0f && Cb != nullptr) {
+          f32x4_t c = load_bf16x4_as_f32(Cb + (int64_t)m * p.ldc + n);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) v[r] = __builtin_fmaf(beta, c[r], v[r]);
+        }
+        if (MODE == MODE_SYRK && p.shift_mode == SHIFT_GRAM && diag) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (n + r == m) v[r] -= shift;
+        }
+        if (MODE == MODE_GEMM) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) ssq = __builtin_fmaf(v[r], v[r], ssq);
+        }
+        if (OUT_F32) {
+          float* o = reinterpret_cast<float*>(p.Out) + batch * p.o_bs + (int64_t)m * p.ldo + n;
+          f32x4_t w;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) w[r] = v[r] * p.out_scale;
+          *reinterpret_cast<f32x4_t*>(o) = w;
+        } else {
+          uint16_t* ob = reinterpret_cast<uint16_t*>(p.Out) + batch * p.o_bs;
+          bf16x4_t h = __builtin_convertvector(v, bf16x4_t);
+          if (MODE == MODE_GEMM) {
+            *reinterpret_cast<bf16x4_t*>(ob + (int64_t)m * p.ldo + n) = h;
+          } else {
+            const uint2 hb = __builtin_bit_cast(uint2, h);
+            const uint16_t ev[4] = {(uint16_t)(hb.x & 0xffffu), (uint16_t)(hb.x >> 16), (uint16_t)(hb.y & 0xffffu),
+                                    (uint16_t)(hb.y >> 16)};
+            if (!diag) {
+              *reinterpret_cast<uint2*>(ob + (int64_t)m * p.ldo + n) = hb;
+              if (!p.skip_upper) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) ob[(int64_t)(n + r) * p.ldo + m] = ev[r];
+              }
+            } else if (p.skip_upper) {
+              *reinterpret_cast<uint2*>(ob + (int64_t)m * p.ldo + n) = hb;
+            } else {
+              // Diagonal tile: the lower half is stored and mirrored, the computed upper half is
+              // dropped, so the result is symmetric bit for bit by construction.
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                if (n + r <= m) ob[(int64_t)m * p.ldo + n + r] = ev[r];
+                if (n + r < m) ob[(int64_t)(n + r) * p.ldo + m] = ev[r];
+              }
+            }
+          }
+        }
+      }
+    }
+  }
+  if (MODE == MODE_GEMM && p.slots_out != nullptr) {
+    const float total = block_sum_f32<NT>(ssq, red);
+    if (threadIdx.x == 0) p.slots_out[batch * gridDim.x + blockIdx.x] = total;
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // The kernel.  grid = (tiles, batch); block = WGM*WGN wavefronts; dynamic LDS = 2 stages.
 // ---------------------------------------------------------------------------------------------
@@ -178,6 +307,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_bf16_kernel(GemmParams p) 
   static_assert(MODE != MODE_SYRK || BM == BN, "SYRK needs square tiles");
 
   extern __shared__ __align__(16) char smem[];
+  __shared__ float red[NT / 64];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave % WGM, wn = wave / WGM;
@@ -243,65 +373,11 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_bf16_kernel(GemmParams p) 
     __syncthreads();
   }
 
-  // ------------------------------------------------------------------ epilogue
-  const float alpha = p.alpha, beta = p.beta;
-  const uint16_t* __restrict__ Cb = p.Cin ? p.Cin + batch * p.c_bs : nullptr;
+  float beta = p.beta;
+  const float shift = resolve_shift<NT>(p, batch, red, beta);
   const bool diag = (MODE == MODE_SYRK) && (tm == tn);
-#pragma unroll
-  for (int i = 0; i < FM; ++i) {
-    const int m = m0 + wm * TM + i * 32 + frow;
-#pragma unroll
-    for (int j = 0; j < FN; ++j) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int n = n0 + wn * TN + j * 32 + 8 * g + 4 * fk;
-        if (m >= p.M || n >= p.N) continue;
-        f32x4_t v;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][4 * g + r];
-        if (beta != 0.0f) {
-          f32x4_t c = load_bf16x4_as_f32(Cb + (int64_t)m * p.ldc + n);
-#pragma unroll
-          for (int r = 0; r < 4; ++r) v[r] = __builtin_fmaf(beta, c[r], v[r]);
-        }
-        if (OUT_F32) {
-          float* o = reinterpret_cast<float*>(p.Out) + batch * p.o_bs + (int64_t)m * p.ldo + n;
-          f32x4_t w;
-#pragma unroll
-          for (int r = 0; r < 4; ++r) w[r] = v[r] * p.out_scale;
-          *reinterpret_cast<f32x4_t*>(o) = w;
-        } else {
-          uint16_t* ob = reinterpret_cast<uint16_t*>(p.Out) + batch * p.o_bs;
-          bf16x4_t h = __builtin_convertvector(v, bf16x4_t);
-          if (MODE == MODE_GEMM) {
-            *reinterpret_cast<bf16x4_t*>(ob + (int64_t)m * p.ldo + n) = h;
-          } else {
-            const uint2 hb = __builtin_bit_cast(uint2, h);
-            const uint16_t e0 = (uint16_t)(hb.x & 0xffffu), e1 = (uint16_t)(hb.x >> 16);
-            const uint16_t e2 = (uint16_t)(hb.y & 0xffffu), e3 = (uint16_t)(hb.y >> 16);
-            const uint16_t ev[4] = {e0, e1, e2, e3};
-            if (!diag) {
-              *reinterpret_cast<uint2*>(ob + (int64_t)m * p.ldo + n) = hb;
-              if (!p.skip_upper) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) ob[(int64_t)(n + r) * p.ldo + m] = ev[r];
-              }
-            } else if (p.skip_upper) {
-              *reinterpret_cast<uint2*>(ob + (int64_t)m * p.ldo + n) = hb;
-            } else {
-              // Diagonal tile: the lower half is stored and mirrored, the computed upper half is
-              // dropped, so the result is symmetric bit for bit by construction.
-#pragma unroll
-              for (int r = 0; r < 4; ++r) {
-                if (n + r <= m) ob[(int64_t)m * p.ldo + n + r] = ev[r];
-                if (n + r < m) ob[(int64_t)(n + r) * p.ldo + m] = ev[r];
-              }
-            }
-          }
-        }
-      }
-    }
-  }
+  tile_epilogue<MODE, OUT_F32, true, FM, FN, NT>(p, acc, m0 + wm * TM, n0 + wn * TN, lane, batch, diag, p.alpha, beta,
+                                                 shift, red);
 }
 
 }  // namespace mi

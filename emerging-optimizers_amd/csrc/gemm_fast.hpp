@@ -101,6 +101,7 @@ __global__ void __launch_bounds__(fast::NT) gemm_fast_kernel(GemmParams p) {
   using namespace fast;
   __shared__ __align__(1024) char stage0[STAGE_BYTES];
   __shared__ __align__(1024) char stage1[STAGE_BYTES];
+  __shared__ float red[NT / 64];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave % WGM, wn = wave / WGM;
@@ -167,62 +168,11 @@ __global__ void __launch_bounds__(fast::NT) gemm_fast_kernel(GemmParams p) {
     }
   }
 
-  // ------------------------------------------------------------------ epilogue
-  const int frow = lane & 31, fk = lane >> 5;
-  const float alpha = p.alpha, beta = p.beta;
-  const uint16_t* __restrict__ Cb = p.Cin ? p.Cin + batch * p.c_bs : nullptr;
+  float beta = p.beta;
+  const float shift = resolve_shift<NT>(p, batch, red, beta);
   const bool diag = (MODE == MODE_SYRK) && (tm == tn);
-#pragma unroll
-  for (int i = 0; i < FM; ++i) {
-    const int m = m0 + wm * TM + i * 32 + frow;
-#pragma unroll
-    for (int j = 0; j < FN; ++j) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int n = n0 + wn * TN + j * 32 + 8 * g + 4 * fk;
-        f32x4_t v;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][4 * g + r];
-        if (beta != 0.0f) {
-          f32x4_t c = load_bf16x4_as_f32(Cb + (int64_t)m * p.ldc + n);
-#pragma unroll
-          for (int r = 0; r < 4; ++r) v[r] = __builtin_fmaf(beta, c[r], v[r]);
-        }
-        if (OUT_F32) {
-          float* o = reinterpret_cast<float*>(p.Out) + batch * p.o_bs + (int64_t)m * p.ldo + n;
-          f32x4_t w;
-#pragma unroll
-          for (int r = 0; r < 4; ++r) w[r] = v[r] * p.out_scale;
-          *reinterpret_cast<f32x4_t*>(o) = w;
-        } else {
-          uint16_t* ob = reinterpret_cast<uint16_t*>(p.Out) + batch * p.o_bs;
-          bf16x4_t h = __builtin_convertvector(v, bf16x4_t);
-          if (MODE == MODE_GEMM) {
-            *reinterpret_cast<bf16x4_t*>(ob + (int64_t)m * p.ldo + n) = h;
-          } else {
-            const uint2 hb = __builtin_bit_cast(uint2, h);
-            const uint16_t ev[4] = {(uint16_t)(hb.x & 0xffffu), (uint16_t)(hb.x >> 16), (uint16_t)(hb.y & 0xffffu),
-                                    (uint16_t)(hb.y >> 16)};
-            if (!diag) {
-              *reinterpret_cast<uint2*>(ob + (int64_t)m * p.ldo + n) = hb;
-              if (!p.skip_upper) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) ob[(int64_t)(n + r) * p.ldo + m] = ev[r];
-              }
-            } else if (p.skip_upper) {
-              *reinterpret_cast<uint2*>(ob + (int64_t)m * p.ldo + n) = hb;
-            } else {
-#pragma unroll
-              for (int r = 0; r < 4; ++r) {
-                if (n + r <= m) ob[(int64_t)m * p.ldo + n + r] = ev[r];
-                if (n + r < m) ob[(int64_t)(n + r) * p.ldo + m] = ev[r];
-              }
-            }
-          }
-        }
-      }
-    }
-  }
+  tile_epilogue<MODE, OUT_F32, false, FM, FN, NT>(p, acc, m0 + wm * TM, n0 + wn * TN, lane, batch, diag, p.alpha, beta,
+                                                  shift, red);
 }
 
 }  // namespace mi

@@ -5,7 +5,9 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
 #include <string>
+#include <vector>
 
 #include "gemm_engine.hpp"
 #include "gemm_fast.hpp"
@@ -24,6 +26,38 @@ static int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Optional per-kernel timing of the fused driver: HIP event pairs recorded on the caller's stream.
+// Off by default; mi_profile_begin() switches it on, mi_profile_end() waits for the events and reports.
+// ---------------------------------------------------------------------------------------------
+enum { PROF_NORMALIZE = 0, PROF_GRAM = 1, PROF_POLY = 2, PROF_APPLY = 3, PROF_KINDS = 4 };
+struct ProfSpan {
+  int kind;
+  hipEvent_t start, stop;
+};
+static std::mutex g_prof_mutex;
+static bool g_prof_on = false;
+static std::vector<ProfSpan> g_prof_spans;
+
+struct ProfScope {
+  hipStream_t stream;
+  hipEvent_t stop = nullptr;
+  bool active = false;
+  ProfScope(int kind, hipStream_t st) : stream(st) {
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
+    if (!g_prof_on) return;
+    ProfSpan span{kind, nullptr, nullptr};
+    if (hipEventCreate(&span.start) != hipSuccess || hipEventCreate(&span.stop) != hipSuccess) return;
+    (void)hipEventRecord(span.start, stream);
+    stop = span.stop;
+    active = true;
+    g_prof_spans.push_back(span);
+  }
+  ~ProfScope() {
+    if (active) (void)hipEventRecord(stop, stream);
+  }
+};
+
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // ---------------------------------------------------------------------------------------------
@@ -37,6 +71,9 @@ static TileClass pick_class(int64_t extent) {
   if (extent >= 256) return TILE_MID;
   return TILE_SMALL;
 }
+
+// Number of workgroups (per batch entry) the last launch_class call on this thread used.
+static thread_local int g_last_tiles = 0;
 
 template <int BM, int BN, int BK, int WGM, int WGN, bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
 static int launch_one(const GemmParams& p, int64_t batch, hipStream_t stream) {
@@ -55,6 +92,7 @@ static int launch_one(const GemmParams& p, int64_t batch, hipStream_t stream) {
   int64_t tiles = (MODE == MODE_SYRK) ? (int64_t)q.tiles_m * (q.tiles_m + 1) / 2 : (int64_t)q.tiles_m * q.tiles_n;
   if (tiles <= 0 || batch <= 0) return MI_OK;
   if (batch > 65535) return fail(MI_ERR_UNSUPPORTED_SHAPE, "batch %lld exceeds the grid limit 65535", (long long)batch);
+  g_last_tiles = (int)tiles;
   dim3 grid((unsigned)tiles, (unsigned)batch, 1), block(WGM * WGN * 64, 1, 1);
   hipLaunchKernelGGL(kern, grid, block, LDS_BYTES, stream, q);
   hipError_t e = hipGetLastError();
@@ -69,6 +107,7 @@ static int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream) {
   q.tiles_n = p.N / fast::BN;
   const int64_t tiles = (MODE == MODE_SYRK) ? (int64_t)q.tiles_m * (q.tiles_m + 1) / 2 : (int64_t)q.tiles_m * q.tiles_n;
   if (batch > 65535) return fail(MI_ERR_UNSUPPORTED_SHAPE, "batch %lld exceeds the grid limit 65535", (long long)batch);
+  g_last_tiles = (int)tiles;
   dim3 grid((unsigned)tiles, (unsigned)batch, 1), block(fast::NT, 1, 1);
   hipLaunchKernelGGL((gemm_fast_kernel<P_KS, Q_KS, MODE, OUT_F32>), grid, block, 0, stream, q);
   hipError_t e = hipGetLastError();
@@ -93,10 +132,29 @@ static int launch_class(TileClass tc, const GemmParams& p, int64_t batch, hipStr
   }
 }
 
+// Diagonal-shift wiring of one launch inside the fused driver (see GemmParams).
+struct ShiftArgs {
+  int mode;
+  float cb, cc;
+  const float* slots_in;
+  int nslots_in;
+  float* shift_io;
+  float* slots_out;
+  void apply(GemmParams& p) const {
+    p.shift_mode = mode;
+    p.cb = cb;
+    p.cc = cc;
+    p.slots_in = slots_in;
+    p.nslots_in = nslots_in;
+    p.shift_io = shift_io;
+    p.slots_out = slots_out;
+  }
+};
+
 // D = alpha * A A^T + beta * C, bf16 out.
 static int syrk_impl(const void* A, int64_t batch, int64_t n, int64_t k, int64_t a_bs, int64_t a_ld, int a_trans,
                      const void* C, int64_t c_bs, int64_t c_ld, float alpha, float beta, void* D, int64_t d_bs,
-                     int64_t d_ld, int skip_upper, hipStream_t stream) {
+                     int64_t d_ld, int skip_upper, hipStream_t stream, const ShiftArgs* sh = nullptr) {
   if (!A || !D) return fail(MI_ERR_BAD_ARG, "mi_syrk_bf16: A and D must not be null");
   if (batch < 0 || n < 0 || k < 0) return fail(MI_ERR_BAD_ARG, "mi_syrk_bf16: negative extent");
   if (beta != 0.0f && !C) return fail(MI_ERR_BAD_ARG, "mi_syrk_bf16: C is null but beta != 0");
@@ -125,6 +183,7 @@ static int syrk_impl(const void* A, int64_t batch, int64_t n, int64_t k, int64_t
   p.beta = beta;
   p.out_scale = 1.0f;
   p.skip_upper = skip_upper ? 1 : 0;
+  if (sh) sh->apply(p);
   TileClass tc = pick_class(n);
   return a_trans ? launch_class<true, true, MODE_SYRK, false>(tc, p, batch, stream)
                  : launch_class<false, false, MODE_SYRK, false>(tc, p, batch, stream);
@@ -134,7 +193,7 @@ static int syrk_impl(const void* A, int64_t batch, int64_t n, int64_t k, int64_t
 static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void* X, int64_t x_bs,
                           int64_t x_ld, int x_trans, void* Xout, int64_t o_bs, int64_t o_ld, int64_t batch,
                           int64_t m, int64_t n, float alpha, float beta, int out_fp32, float out_scale,
-                          hipStream_t stream) {
+                          hipStream_t stream, const ShiftArgs* sh = nullptr) {
   if (!Bm || !X || !Xout) return fail(MI_ERR_BAD_ARG, "mi_gemm_axpy_bf16: null pointer");
   if (batch < 0 || m < 0 || n < 0) return fail(MI_ERR_BAD_ARG, "mi_gemm_axpy_bf16: negative extent");
   if (m % 8 || n % 8) return fail(MI_ERR_UNSUPPORTED_SHAPE, "M and N must be multiples of 8, got M=%lld, N=%lld", (long long)m, (long long)n);
@@ -158,6 +217,7 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
   p.alpha = alpha;
   p.beta = beta;
   p.out_scale = out_scale;
+  if (sh) sh->apply(p);
   TileClass tc = pick_class(m);
   if (!x_trans) {
     // OUT (m x n): P = Bm rows (K-contiguous), Q[j][k] = X[k][j] (K-strided).
@@ -264,7 +324,8 @@ template <bool F64, bool OUT_BF16>
 __global__ void __launch_bounds__(NORM_THREADS) scale_cast_kernel(const float* __restrict__ x, int64_t numel,
                                                                   const double* __restrict__ partials, int nparts,
                                                                   float eps, float post_scale, void* __restrict__ out,
-                                                                  float* __restrict__ dev_norm) {
+                                                                  float* __restrict__ dev_norm,
+                                                                  float* __restrict__ sumsq_out) {
   const int64_t b = blockIdx.y;
   __shared__ double scratch_d[NORM_THREADS / 64];
   double s = 0;
@@ -277,6 +338,11 @@ __global__ void __launch_bounds__(NORM_THREADS) scale_cast_kernel(const float* _
     divisor = fmaxf(sqrtf((float)s), eps);
   }
   if (dev_norm && blockIdx.x == 0 && threadIdx.x == 0) dev_norm[b] = divisor;
+  if (sumsq_out && blockIdx.x == 0 && threadIdx.x == 0) {
+    // squared Frobenius norm of the normalised matrix: 1 unless the divisor was clamped
+    const float ratio = sqrtf((float)s) / divisor;
+    sumsq_out[b] = (divisor > 0.0f && ratio == ratio) ? ratio * ratio : 0.0f;
+  }
 
   const int64_t nvec8 = numel / 8;
   const float4* __restrict__ xv = reinterpret_cast<const float4*>(x + b * numel);
@@ -299,7 +365,8 @@ __global__ void __launch_bounds__(NORM_THREADS) scale_cast_kernel(const float* _
 }
 
 static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, int f64, void* out, int out_bf16,
-                     float post_scale, double* partials, float* dev_norm, hipStream_t stream) {
+                     float post_scale, double* partials, float* dev_norm, hipStream_t stream,
+                     float* sumsq_out = nullptr) {
   if (!x || !out || !partials) return fail(MI_ERR_BAD_ARG, "mi_frob_normalize: null pointer");
   if (batch < 0 || numel < 0) return fail(MI_ERR_BAD_ARG, "mi_frob_normalize: negative extent");
   if (numel % 8) return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_frob_normalize: numel must be a multiple of 8, got %lld", (long long)numel);
@@ -316,7 +383,7 @@ static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, in
   if (want < 1) want = 1;
   if (want > 4096) want = 4096;
   dim3 grid2((unsigned)want, (unsigned)batch);
-#define MI_SC(F, B) hipLaunchKernelGGL((scale_cast_kernel<F, B>), grid2, block, 0, stream, x, numel, partials, nb, eps, post_scale, out, dev_norm)
+#define MI_SC(F, B) hipLaunchKernelGGL((scale_cast_kernel<F, B>), grid2, block, 0, stream, x, numel, partials, nb, eps, post_scale, out, dev_norm, sumsq_out)
   if (f64) {
     if (out_bf16) MI_SC(true, true); else MI_SC(true, false);
   } else {
@@ -331,7 +398,8 @@ static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, in
 static size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct NsWorkspace {
-  size_t x0, x1, a, b, partials, norm, total;
+  size_t x0, x1, a, b, partials, norm, slots, shift, total;
+  int64_t max_slots;
 };
 
 static NsWorkspace ns_layout(int64_t batch, int64_t rows, int64_t cols) {
@@ -346,6 +414,10 @@ static NsWorkspace ns_layout(int64_t batch, int64_t rows, int64_t cols) {
   w.b = off; off += gbytes;
   w.partials = off; off += align_up((size_t)batch * NORM_MAX_BLOCKS * sizeof(double), 256);
   w.norm = off; off += align_up((size_t)batch * sizeof(float), 256);
+  // one float per GEMM workgroup; the smallest tile class (64 x 64) bounds the count
+  w.max_slots = ((rows + 63) / 64) * ((cols + 63) / 64);
+  w.slots = off; off += align_up((size_t)batch * w.max_slots * sizeof(float), 256);
+  w.shift = off; off += align_up((size_t)batch * sizeof(float), 256);
   w.total = off;
   return w;
 }
@@ -386,6 +458,41 @@ int mi_frob_normalize(const float* x, int64_t batch, int64_t numel, float eps, i
                    static_cast<hipStream_t>(stream));
 }
 
+int mi_profile_begin(void) {
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  for (auto& sp : g_prof_spans) {
+    (void)hipEventDestroy(sp.start);
+    (void)hipEventDestroy(sp.stop);
+  }
+  g_prof_spans.clear();
+  g_prof_on = true;
+  return MI_OK;
+}
+
+int mi_profile_end(float* ms_by_kind, int* launches_by_kind) {
+  std::lock_guard<std::mutex> lock(g_prof_mutex);
+  g_prof_on = false;
+  if (!ms_by_kind || !launches_by_kind) return fail(MI_ERR_BAD_ARG, "mi_profile_end: null output");
+  for (int k = 0; k < PROF_KINDS; ++k) {
+    ms_by_kind[k] = 0.0f;
+    launches_by_kind[k] = 0;
+  }
+  int rc = MI_OK;
+  for (auto& sp : g_prof_spans) {
+    float ms = 0.0f;
+    if (hipEventSynchronize(sp.stop) != hipSuccess || hipEventElapsedTime(&ms, sp.start, sp.stop) != hipSuccess) {
+      rc = fail(MI_ERR_LAUNCH, "mi_profile_end: event query failed");
+    } else {
+      ms_by_kind[sp.kind] += ms;
+      launches_by_kind[sp.kind] += 1;
+    }
+    (void)hipEventDestroy(sp.start);
+    (void)hipEventDestroy(sp.stop);
+  }
+  g_prof_spans.clear();
+  return rc;
+}
+
 size_t mi_newton_schulz_workspace_bytes(int64_t batch, int64_t rows, int64_t cols) {
   if (batch <= 0 || rows <= 0 || cols <= 0) return 0;
   return ns_layout(batch, rows, cols).total;
@@ -417,7 +524,13 @@ int mi_newton_schulz_bf16(const float* x, float* out, int64_t batch, int64_t row
   if (steps == 0)
     return frob_impl(x, batch, numel, eps, accumulate_fp64, out, /*out_bf16=*/0, out_scale, partials, norm, stream);
 
-  int rc = frob_impl(x, batch, numel, eps, accumulate_fp64, xbuf[0], /*out_bf16=*/1, 1.0f, partials, norm, stream);
+  float* slots = reinterpret_cast<float*>(ws + w.slots);
+  float* shift = reinterpret_cast<float*>(ws + w.shift);
+  int rc;
+  {
+    ProfScope prof(PROF_NORMALIZE, stream);
+    rc = frob_impl(x, batch, numel, eps, accumulate_fp64, xbuf[0], /*out_bf16=*/1, 1.0f, partials, norm, stream, slots);
+  }
   if (rc != MI_OK) return rc;
 
   // The iteration runs on the (m x n) orientation with m <= n.  When rows > cols that orientation is
@@ -427,23 +540,41 @@ int mi_newton_schulz_bf16(const float* x, float* out, int64_t batch, int64_t row
   const int64_t ld = cols;  // row-major (rows x cols) in memory either way
   const int64_t x_bs = numel, g_bs = m * m;
   int cur = 0;
+  int nslots = 1;  // the normalisation kernel left one value per matrix
   for (int s = 0; s < steps; ++s) {
     const float a = abc[3 * s], b = abc[3 * s + 1], c = abc[3 * s + 2];
     const bool last = (s + 1 == steps);
-    rc = syrk_impl(xbuf[cur], batch, m, n, x_bs, ld, trans, nullptr, 0, m, 1.0f, 0.0f, gram, g_bs, m, 0, stream);
+    // A' = X X^T - s I  (s = ||X||_F^2 / m from the partial sums the previous kernel left)
+    ShiftArgs sh_gram{SHIFT_GRAM, b, c, slots, nslots, shift, nullptr};
+    {
+      ProfScope prof(PROF_GRAM, stream);
+      rc = syrk_impl(xbuf[cur], batch, m, n, x_bs, ld, trans, nullptr, 0, m, 1.0f, 0.0f, gram, g_bs, m, 0, stream, &sh_gram);
+    }
     if (rc != MI_OK) return rc;
     const uint16_t* mult = gram;
     float alpha = b;
     if (c != 0.0f) {
-      rc = syrk_impl(gram, batch, m, m, g_bs, m, 0, gram, g_bs, m, c, b, poly, g_bs, m, 0, stream);
+      // B' = c A'^2 + (b + 2 c s) A'
+      ShiftArgs sh_poly{SHIFT_POLY, b, c, nullptr, 0, shift, nullptr};
+      {
+        ProfScope prof(PROF_POLY, stream);
+        rc = syrk_impl(gram, batch, m, m, g_bs, m, 0, gram, g_bs, m, c, b, poly, g_bs, m, 0, stream, &sh_poly);
+      }
       if (rc != MI_OK) return rc;
       mult = poly;
       alpha = 1.0f;
     }
+    // X' = (a + b s + c s^2) X + B' X      (cubic: (a + b s) X + b A' X)
     void* dst = last ? static_cast<void*>(out) : static_cast<void*>(xbuf[cur ^ 1]);
-    rc = gemm_axpy_impl(mult, g_bs, m, xbuf[cur], x_bs, ld, trans, dst, x_bs, ld, batch, m, n, alpha, a,
-                        last ? 1 : 0, last ? out_scale : 1.0f, stream);
+    ShiftArgs sh_apply{SHIFT_APPLY, b, c, nullptr, 0, shift, last ? nullptr : slots};
+    {
+      ProfScope prof(PROF_APPLY, stream);
+      rc = gemm_axpy_impl(mult, g_bs, m, xbuf[cur], x_bs, ld, trans, dst, x_bs, ld, batch, m, n, alpha, a,
+                          last ? 1 : 0, last ? out_scale : 1.0f, stream, &sh_apply);
+    }
     if (rc != MI_OK) return rc;
+    nslots = g_last_tiles;
+    if (nslots > w.max_slots) return fail(MI_ERR_WORKSPACE, "internal: %d partial-sum slots exceed the %lld reserved", nslots, (long long)w.max_slots);
     cur ^= 1;
   }
   return MI_OK;

@@ -1,0 +1,33 @@
+"""Python entry points of the gfx950 kernels (SYRK, GEMM+AXPY, Frobenius normalise, fused Newton-Schulz)."""
+
+from .. import _hip
+from .batched_syrk import batched_tsyrk_ex, can_use_batched_tsyrk
+from .newton_schulz import fused_newton_schulz, fused_supported, gemm_axpy
+from .syrk import tsyrk_ex, tsyrk_ex_small_matrix
+
+
+def _device_ready() -> bool:
+    import torch
+
+    if not _hip.available() or not torch.cuda.is_available():
+        return False
+    arch = getattr(torch.cuda.get_device_properties(0), "gcnArchName", "")
+    return arch.startswith("gfx950")
+
+
+#: True when libmi_ns.so is loadable.  The reference's call sites test ``HAS_TRITON_340`` before taking
+#: the SYRK path (muon.py:106, muon_utils.py:431,465); the same attribute name is kept for them.
+HAS_HIP_KERNELS = _hip.available()
+HAS_TRITON_340 = HAS_HIP_KERNELS
+
+__all__ = [
+    "HAS_HIP_KERNELS",
+    "HAS_TRITON_340",
+    "batched_tsyrk_ex",
+    "can_use_batched_tsyrk",
+    "fused_newton_schulz",
+    "fused_supported",
+    "gemm_axpy",
+    "tsyrk_ex",
+    "tsyrk_ex_small_matrix",
+]

@@ -1,0 +1,124 @@
+"""GEMM+AXPY and the single-call Newton-Schulz driver of libmi_ns.so."""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Sequence
+
+import torch
+
+from .. import _hip
+from . import _launch
+
+
+__all__ = ["gemm_axpy", "fused_newton_schulz", "fused_supported"]
+
+
+def gemm_axpy(
+    bm: torch.Tensor,
+    x: torch.Tensor,
+    alpha: float = 1.0,
+    beta: float = 1.0,
+    *,
+    out_dtype: torch.dtype = torch.bfloat16,
+    out_scale: float = 1.0,
+) -> torch.Tensor:
+    """``beta * x + alpha * (bm @ x)`` for bf16 ``bm`` (.., m, m) and ``x`` (.., m, n), 2-D or batched 3-D.
+
+    The HIP counterpart of ``torch.addmm(X, B, X, alpha=alpha, beta=beta)`` / ``torch.baddbmm`` in a
+    Newton-Schulz step (muon_utils.py:374-377, 407-410 of the reference).  ``x`` or ``x.mT`` must be
+    contiguous; the result has the layout of ``x``.  ``out_dtype=torch.float32`` returns
+    ``out_scale * (...)`` without the intermediate bf16 rounding.
+    """
+    if bm.dtype != torch.bfloat16 or x.dtype != torch.bfloat16:
+        raise TypeError("gemm_axpy operands must be bfloat16")
+    if x.dim() not in (2, 3) or bm.dim() != x.dim():
+        raise TypeError("gemm_axpy operands must both be 2D or both be 3D")
+    _launch.require_gpu(x, "gemm_axpy")
+    batch = x.shape[0] if x.dim() == 3 else 1
+    m, n = x.shape[-2], x.shape[-1]
+    if tuple(bm.shape[-2:]) != (m, m) or (x.dim() == 3 and bm.shape[0] != batch):
+        raise RuntimeError(f"bm must be of shape (..., {m}, {m}), got {tuple(bm.shape)}")
+    if not (x.is_contiguous() or x.mT.is_contiguous()):
+        raise TypeError("invalid input tensor layout. x or x.mT must be contiguous.")
+    if m % 8 or n % 8:
+        raise RuntimeError(f"M and N must be multiples of 8 for 16-byte bf16 loads, got M={m}, N={n}")
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError("out_dtype must be bfloat16 or float32")
+    bm = bm.contiguous()
+    x_trans = not x.is_contiguous()
+    mem_x = x.mT if x_trans else x
+    out_mem = torch.empty(mem_x.shape, device=x.device, dtype=out_dtype)
+    lib = _hip.lib()
+    with torch.cuda.device(x.device):
+        rc = lib.mi_gemm_axpy_bf16(
+            _launch.ptr(bm), m * m, m,
+            _launch.ptr(mem_x), m * n, mem_x.shape[-1], int(x_trans),
+            _launch.ptr(out_mem), m * n, mem_x.shape[-1],
+            batch, m, n, float(alpha), float(beta),
+            int(out_dtype == torch.float32), float(out_scale), _hip.current_stream_ptr(x.device),
+        )  # fmt: skip
+    _hip.check(rc)
+    return out_mem.mT if x_trans else out_mem
+
+
+def fused_supported(x: torch.Tensor) -> bool:
+    """True when :func:`fused_newton_schulz` can take ``x``: GPU float32, 2-D/3-D, both dims multiples of 8."""
+    return (
+        _hip.available()
+        and x.is_cuda
+        and x.dtype == torch.float32
+        and x.dim() in (2, 3)
+        and x.shape[-1] % 8 == 0
+        and x.shape[-2] % 8 == 0
+        and x.numel() > 0
+    )
+
+
+# One cached workspace per (device, stream): Newton-Schulz calls on one stream are serialised by the
+# stream itself, so they can share scratch; different streams get different buffers.
+_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+
+
+def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    key = (device.index if device.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, device=device, dtype=torch.uint8)
+        _workspaces[key] = ws
+    return ws
+
+
+def fused_newton_schulz(
+    x: torch.Tensor,
+    coefficients: Sequence[tuple[float, float, float]],
+    eps: float = 1e-15,
+    normalize_in_double: bool = False,
+    out_scale: float = 1.0,
+) -> torch.Tensor:
+    """Normalise, iterate and rescale in one library call; returns a new float32 tensor shaped like ``x``.
+
+    Covers the "medium"-precision body of the reference's ``newton_schulz`` (muon_utils.py:212-273) for one
+    process.  The iteration runs on the orientation with the shorter leading dimension, read in place.
+    """
+    if not fused_supported(x):
+        raise RuntimeError(f"fused_newton_schulz cannot take a {x.dtype} tensor of shape {tuple(x.shape)} on {x.device}")
+    xc = x if x.is_contiguous() else x.contiguous()
+    batch = xc.shape[0] if xc.dim() == 3 else 1
+    rows, cols = xc.shape[-2], xc.shape[-1]
+    out = torch.empty_like(xc)
+    lib = _hip.lib()
+    steps = len(coefficients)
+    flat = [float(v) for abc in coefficients for v in abc]
+    abc = (ctypes.c_float * max(1, len(flat)))(*flat)
+    with torch.cuda.device(x.device):
+        nbytes = lib.mi_newton_schulz_workspace_bytes(batch, rows, cols)
+        ws = _workspace(x.device, nbytes)
+        rc = lib.mi_newton_schulz_bf16(
+            _launch.ptr(xc), _launch.ptr(out), batch, rows, cols, abc, steps, float(eps),
+            int(bool(normalize_in_double)), float(out_scale), _launch.ptr(ws), ws.numel(),
+            _hip.current_stream_ptr(x.device),
+        )  # fmt: skip
+    _hip.check(rc)
+    return out

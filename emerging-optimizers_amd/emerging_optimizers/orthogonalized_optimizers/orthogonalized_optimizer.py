@@ -1,0 +1,129 @@
+"""Momentum-SGD skeleton whose update is passed through an orthogonalisation function.
+
+Behaviour follows the reference's ``OrthogonalizedOptimizer``
+(orthogonalized_optimizers/orthogonalized_optimizer.py:47-272): per parameter, in this order,
+weight decay -> EMA momentum -> optional Nesterov blend -> ``orthogonalize`` (under the configured float32
+matmul precision) -> pre hooks -> ``p += -lr * update`` -> post hooks.  The only optimizer state is
+``momentum_buffer``.
+"""
+
+from __future__ import annotations
+
+import logging
+from typing import Any, Callable, Generic, Optional
+
+import torch
+from torch.optim.optimizer import Optimizer, ParamsT
+
+from emerging_optimizers import utils
+from emerging_optimizers.mixin import WeightDecayMixin, WeightDecayT
+from emerging_optimizers.utils import FP32MatmulPrecT
+from emerging_optimizers.weight_update_hooks import NoOpWeightUpdateHook, WeightUpdateHook
+from emerging_optimizers.weight_update_hooks.base import HookStateT
+
+
+_log = logging.getLogger(__name__)
+
+_args_doc = """params: parameters (or parameter-group dicts) to optimize
+        lr: learning rate of the inner SGD
+        momentum: EMA coefficient of the momentum buffer (``buf = momentum * buf + (1 - momentum) * grad``)
+        weight_decay: weight-decay strength; how it is applied is set by ``weight_decay_method``
+        nesterov: blend the fresh gradient with the buffer once more before orthogonalising
+        weight_decay_method: one of the flavours of :class:`~emerging_optimizers.mixin.WeightDecayMixin`
+        fp32_matmul_prec: float32 matmul precision in force while orthogonalising ("medium" = bf16 kernels)
+        weight_update_hook: optional object called right before and after the in-place weight update
+"""
+
+
+class OrthogonalizedOptimizer(WeightDecayMixin, Optimizer, Generic[HookStateT]):
+    """SGD-with-momentum whose per-parameter update goes through ``scaled_orthogonalize_fn`` first.
+
+    Subclasses usually only supply ``scaled_orthogonalize_fn``.  To treat fused parameters (e.g. a stacked
+    QKV weight) piecewise, override :meth:`orthogonalize`, split ``grad`` there and call
+    ``self.scaled_orthogonalize_fn`` on each piece (it also accepts a stacked 3-D tensor).
+
+    Args:
+        {_args_doc}
+        scaled_orthogonalize_fn: maps the momentum tensor to the update; identity when omitted.
+        **kwargs: extra per-group defaults, stored unchecked.
+    """
+
+    def __init__(
+        self,
+        params: ParamsT,
+        lr: float,
+        momentum: float,
+        weight_decay: float,
+        *,
+        nesterov: bool,
+        weight_decay_method: WeightDecayT,
+        fp32_matmul_prec: FP32MatmulPrecT,
+        scaled_orthogonalize_fn: Optional[Callable] = None,
+        weight_update_hook: Optional[WeightUpdateHook[HookStateT]] = None,
+        **kwargs: Any,
+    ):
+        if scaled_orthogonalize_fn is None:
+            _log.warning("scaled_orthogonalize_fn not provided. Using noop")
+            scaled_orthogonalize_fn = torch.nn.Identity()
+        self.fp32_matmul_prec = fp32_matmul_prec
+        self.nesterov = nesterov
+        self.weight_decay_method = weight_decay_method
+        self._weight_update_hook = weight_update_hook if weight_update_hook is not None else NoOpWeightUpdateHook()
+        super().__init__(params, dict(lr=lr, momentum=momentum, weight_decay=weight_decay, **kwargs))
+        self.scaled_orthogonalize_fn = scaled_orthogonalize_fn
+
+    @torch.no_grad()
+    def _init_group(self, group: dict, skip_non_grad_params: bool = True) -> None:
+        """Create the zero momentum buffer of every parameter of ``group`` that does not have one yet."""
+        for p in group["params"]:
+            if p.grad is None and skip_non_grad_params:
+                continue
+            state = self.state[p]
+            if not state:
+                state["momentum_buffer"] = torch.zeros_like(p.data)
+
+    @torch.no_grad()
+    def step(self, closure: Optional[Callable[[], float]] = None) -> Optional[float]:
+        """One optimisation step.  ``closure`` is not supported and must be ``None``."""
+        if closure is not None:
+            raise ValueError("closure is not supported")
+        for group in self.param_groups:
+            self._init_group(group)
+            lr, beta = group["lr"], group["momentum"]
+            extras = {k: v for k, v in group.items() if k != "params"}
+            for p in group["params"]:
+                grad = p.grad
+                if grad is None:
+                    continue
+                buf = self.state[p]["momentum_buffer"]
+                self._apply_weight_decay_inplace(p, grad, lr, group["weight_decay"])
+                buf.lerp_(grad, 1 - beta)
+                direction = grad.lerp(buf, beta) if self.nesterov else buf
+                with utils.fp32_matmul_precision(self.fp32_matmul_prec):
+                    update = self.orthogonalize(p, direction, **extras)
+                self.pre_weight_update_fn_inplace(p, update)
+                hook_state = self._weight_update_hook.pre_weight_update_inplace(p, update)
+                p.add_(update, alpha=-lr)
+                self.post_weight_update_fn_inplace(p)
+                self._weight_update_hook.post_weight_update_inplace(p, hook_state)
+        return None
+
+    def orthogonalize(self, p: torch.Tensor, grad: torch.Tensor, **kwargs: Any) -> torch.Tensor:
+        """Turn the momentum ``grad`` of parameter ``p`` into the update.
+
+        The base version accepts 2-D tensors only and applies ``scaled_orthogonalize_fn``.  ``p`` and the
+        parameter-group entries in ``kwargs`` are there for overrides that need per-parameter attributes
+        (fused QKV splits, reshaped convolution weights, per-head stacking).
+        """
+        if grad.ndim != 2:
+            raise ValueError("Only 2D parameters are supported.")
+        return self.scaled_orthogonalize_fn(grad)
+
+    def pre_weight_update_fn_inplace(self, p: torch.Tensor, update: torch.Tensor) -> None:
+        """Subclass hook, called with the final update just before ``p.add_(update, alpha=-lr)``."""
+
+    def post_weight_update_fn_inplace(self, p: torch.Tensor) -> None:
+        """Subclass hook, called with the already updated parameter."""
+
+
+OrthogonalizedOptimizer.__doc__ = OrthogonalizedOptimizer.__doc__.format(_args_doc=_args_doc)  # type: ignore[union-attr]

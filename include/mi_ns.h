@@ -122,6 +122,18 @@ int mi_newton_schulz_bf16(const float* x, float* out, int64_t batch, int64_t row
                           float out_scale, void* workspace, size_t workspace_bytes, void* stream);
 size_t mi_newton_schulz_workspace_bytes(int64_t batch, int64_t rows, int64_t cols);
 
+/*
+ * Per-kernel timing of mi_newton_schulz_bf16 for benchmarks (no counterpart in the reference, whose
+ * benchmark brackets whole calls with torch.cuda.profiler.start/stop, benchmarks/newton_schulz_benchmark.py:155-164).
+ * Between mi_profile_begin() and mi_profile_end() every kernel group the driver enqueues is bracketed by a
+ * HIP event pair on the caller's stream.  mi_profile_end() waits for those events and fills two arrays of
+ * 4 entries indexed by kind: 0 = normalise+cast (2 launches per call), 1 = SYRK X X^T, 2 = SYRK c A^2 + b A,
+ * 3 = GEMM+AXPY; ms_by_kind = summed milliseconds, launches_by_kind = number of bracketed groups.
+ * Profiling is process-wide and meant for single-threaded benchmark loops.
+ */
+int mi_profile_begin(void);
+int mi_profile_end(float* ms_by_kind, int* launches_by_kind);
+
 #ifdef __cplusplus
 }
 #endif

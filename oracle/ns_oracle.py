@@ -221,6 +221,50 @@ def newton_schulz(
     return _mT(X) if transpose else X
 
 
+def newton_schulz_shifted_bf16(
+    x: np.ndarray,
+    steps: int,
+    coefficient_type: str = "quintic",
+    custom_coefficient_sets=None,
+    eps: float = 1e-15,
+    normalize_in_double: bool = False,
+) -> np.ndarray:
+    """CPU model of the rounding schedule of the single-call GPU driver (``mi_newton_schulz_bf16``).
+
+    Not a restatement of the reference: the reference rounds X, A = X X^T and B = b A + c A^2 to bf16 in every
+    step (muon_utils.py:262, 414-476), which leaves it 1.0e-2 .. 1.3e-2 (relative Frobenius) away from its own
+    float32 path because bf16 rounding of the O(1) diagonal of A dominates.  The driver stores A' = A - s I
+    with s = ||X||_F^2 / m instead and folds the identity part into the epilogue scalars
+        B' = c A'^2 + (b + 2 c s) A',      X' = (a + b s + c s^2) X + B' X,
+    which is algebraically the same iteration for any s.  The last step is written to float32 unrounded.
+    This function reproduces those rounding points so that GPU results can be compared tightly.
+    """
+    x = np.asarray(x)
+    if x.dtype != np.float32 or x.ndim not in (2, 3):
+        raise TypeError("float32 2-D or 3-D input expected")
+    transpose = x.shape[-2] > x.shape[-1]
+    if transpose:
+        x = _mT(x)
+    X = round_to_bf16(frobenius_normalize(x, eps, normalize_in_double))
+    m = X.shape[-2]
+    f = np.float32
+    sumsq = np.ones(X.shape[:-2] + (1, 1), dtype=np.float32)
+    coeffs = expand_coefficients(steps, coefficient_type, custom_coefficient_sets)
+    eye = np.eye(m, dtype=np.float32)
+    for i, (a, b, c) in enumerate(coeffs):
+        s = sumsq / f(m)
+        gram = round_to_bf16(np.matmul(X, _mT(X)) - s * eye)
+        if c != 0.0:
+            poly = round_to_bf16(f(c) * np.matmul(gram, gram) + (f(b) + f(2.0) * f(c) * s) * gram)
+            Xn = (f(a) + f(b) * s + f(c) * s * s) * X + np.matmul(poly, X)
+        else:
+            Xn = (f(a) + f(b) * s) * X + f(b) * np.matmul(gram, X)
+        sumsq = np.sum(Xn * Xn, axis=(-2, -1), keepdims=True, dtype=np.float32)
+        X = Xn if i + 1 == len(coeffs) else round_to_bf16(Xn)
+    X = X.astype(np.float32)
+    return _mT(X) if transpose else X
+
+
 def svd_polynomial(x: np.ndarray, coeffs: Sequence[tuple[float, float, float]], eps: float = 1e-15) -> np.ndarray:
     """Closed form of the iteration in float64, independent of any matrix-product code path.
 

@@ -1,0 +1,99 @@
+"""The shared library loads and exports exactly what include/mi_ns.h declares; argument validation that
+needs no GPU returns the documented error codes.  No kernel is launched here."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from emerging_optimizers import _hip, hip_kernels, triton_kernels
+
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(REPO, "include", "mi_ns.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mi_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported():
+    names = _declared_symbols()
+    assert names == sorted(n for n, _, _ in _hip.EXPORTS), "binding table and header disagree"
+    lib = _hip.lib()
+    for name in names:
+        assert getattr(lib, name) is not None
+
+
+def test_version_and_flags():
+    assert _hip.lib().mi_version() >= 100
+    assert hip_kernels.HAS_HIP_KERNELS is True and triton_kernels.HAS_TRITON_340 is True
+    assert triton_kernels.tsyrk_ex is hip_kernels.tsyrk_ex
+
+
+def test_validation_codes_without_gpu():
+    lib = _hip.lib()
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.cast(ctypes.addressof(buf) & ~15, ctypes.c_void_p)
+    # N not a multiple of 8
+    rc = lib.mi_syrk_bf16(p, 1, 12, 16, 192, 16, 0, None, 0, 12, 1.0, 0.0, p, 144, 12, 0, None)
+    assert rc == _hip.MI_ERR_UNSUPPORTED_SHAPE and "multiples of 8" in _hip.last_error()
+    # beta != 0 without C
+    assert lib.mi_syrk_bf16(p, 1, 16, 16, 256, 16, 0, None, 0, 16, 1.0, 0.5, p, 256, 16, 0, None) == _hip.MI_ERR_BAD_ARG
+    assert lib.mi_syrk_bf16(None, 1, 16, 16, 256, 16, 0, None, 0, 16, 1.0, 0.0, p, 256, 16, 0, None) == _hip.MI_ERR_BAD_ARG
+    assert lib.mi_gemm_axpy_bf16(p, 0, 12, p, 0, 16, 0, p, 0, 16, 1, 12, 16, 1.0, 1.0, 0, 1.0, None) == _hip.MI_ERR_UNSUPPORTED_SHAPE
+    assert lib.mi_frob_normalize(p, 1, 12, 1e-15, 0, p, 1, p, None, None) == _hip.MI_ERR_UNSUPPORTED_SHAPE
+    # empty problems are no-ops
+    assert lib.mi_syrk_bf16(p, 0, 16, 16, 256, 16, 0, None, 0, 16, 1.0, 0.0, p, 256, 16, 0, None) == _hip.MI_OK
+    assert lib.mi_newton_schulz_workspace_bytes(1, 4096, 14336) >= 2 * 4096 * 14336 * 2 + 2 * 4096 * 4096 * 2
+    assert lib.mi_newton_schulz_workspace_bytes(0, 8, 8) == 0
+    abc = (ctypes.c_float * 3)(1, 2, 3)
+    assert lib.mi_newton_schulz_bf16(p, p, 1, 12, 16, abc, 1, 1e-15, 0, 1.0, p, 10**9, None) == _hip.MI_ERR_UNSUPPORTED_SHAPE
+    assert lib.mi_newton_schulz_bf16(p, p, 1, 16, 16, abc, 1, 1e-15, 0, 1.0, p, 8, None) == _hip.MI_ERR_WORKSPACE
+    assert lib.mi_frob_partials_len(3, 1024) >= 3
+
+
+def test_python_validation_messages_cpu():
+    """Exception types and messages of the SYRK wrappers (test_triton_kernels.py:220-441 of the reference);
+    all of these fire before any device work, so they can be checked on CPU tensors."""
+    bf = torch.bfloat16
+    for fn in (triton_kernels.tsyrk_ex, triton_kernels.tsyrk_ex_small_matrix):
+        with pytest.raises(TypeError, match="must be bfloat16"):
+            fn(torch.randn(4, 4))
+        with pytest.raises(TypeError, match="must be 2D"):
+            fn(torch.randn(4).to(bf))
+        with pytest.raises(TypeError, match="must be contiguous"):
+            fn(torch.randn(8, 8).to(bf)[:, ::2])
+        with pytest.raises(RuntimeError, match=r"c must be of shape \(N, N\)"):
+            fn(torch.randn(4, 4).to(bf), torch.randn(3, 3).to(bf), beta=1.0)
+        with pytest.raises(RuntimeError, match="c or c.T must be contiguous"):
+            fn(torch.randn(8, 8).to(bf), torch.randn(16, 16).to(bf)[::2, ::2], beta=1.0)
+    with pytest.raises(RuntimeError, match="out must be same shape/device/dtype"):
+        triton_kernels.tsyrk_ex_small_matrix(torch.randn(4, 4).to(bf), out=torch.empty(3, 3, dtype=bf))
+    with pytest.raises(RuntimeError, match="out must be contiguous"):
+        triton_kernels.tsyrk_ex_small_matrix(torch.randn(4, 4).to(bf), out=torch.empty(8, 8, dtype=bf)[::2, ::2])
+    b = triton_kernels.batched_tsyrk_ex
+    with pytest.raises(TypeError, match="must be bfloat16"):
+        b(torch.randn(2, 16, 16))
+    with pytest.raises(TypeError, match="must be 3D"):
+        b(torch.randn(16, 16).to(bf))
+    with pytest.raises(TypeError, match="must be contiguous"):
+        b(torch.randn(2, 16, 32).to(bf)[:, :, ::2])
+    for shape in [(2, 12, 16), (2, 16, 12)]:
+        with pytest.raises(RuntimeError, match="must be multiples of 8"):
+            b(torch.randn(*shape).to(bf))
+    with pytest.raises(RuntimeError, match=r"c must be of shape \(B, N, N\)"):
+        b(torch.randn(2, 16, 16).to(bf), torch.randn(2, 8, 8).to(bf), beta=1.0)
+    with pytest.raises(RuntimeError, match="c or c.mT must be contiguous"):
+        b(torch.randn(2, 16, 16).to(bf), torch.randn(2, 32, 32).to(bf)[:, ::2, ::2], beta=1.0)
+    with pytest.raises(RuntimeError, match="out must be same shape/device/dtype"):
+        b(torch.randn(2, 16, 16).to(bf), out=torch.empty(2, 8, 8, dtype=bf))
+    with pytest.raises(RuntimeError, match="out must be contiguous"):
+        b(torch.randn(2, 16, 16).to(bf), out=torch.empty(2, 32, 32, dtype=bf)[:, ::2, ::2])
+    # CPU tensors are refused loudly rather than computed some other way
+    with pytest.raises(RuntimeError, match="GPU only"):
+        triton_kernels.tsyrk_ex(torch.randn(8, 8).to(bf))
+    assert triton_kernels.can_use_batched_tsyrk(torch.randn(2, 16, 16).to(bf)) is False  # not on the GPU
