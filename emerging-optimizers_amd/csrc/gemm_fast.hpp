@@ -1,12 +1,9 @@
-// Fast path of the bf16 tile engine for shapes that tile exactly (M % 256 == N % 256 == K % 64 == 0).
+// Fast path of the bf16 tile engine for the MFMA-bound shapes (K % 64 == 0, no K tail; row edges are
+// allowed and handled by clamped loads plus a guarded epilogue).
 //
-// 256 x 256 x 64 workgroup tile, 8 wavefronts (2 per SIMD) laid out 2 (M) x 4 (N), each owning a
-// 128 x 64 sub-tile = 4 x 2 MFMA 32x32x16 accumulators (128 accumulator VGPRs).  Two wavefronts per
-// SIMD let one issue MFMAs while the other waits on LDS or the barrier.
-//
-// Global -> LDS goes through the direct-to-LDS load (16 bytes per lane, a wavefront fills 1 KB of
-// LDS at base + 16 * lane), two 64 KB stages, one barrier per K tile:
-//     wait own loads of tile kt | barrier | issue loads of tile kt+1 into the other stage | MFMAs on tile kt
+// A variant is described by FastCfg: square workgroup tile, wavefront grid, ring-slot depth BK and number
+// of ring slots.  Global -> LDS goes through the direct-to-LDS load (16 bytes per lane, a wavefront fills
+// 1 KB of LDS at base + 16 * lane); the slots form a ring with one barrier per K tile (see the kernel).
 // Because LDS placement is fixed by the lane id, swizzling is done by choosing which global chunk a
 // lane fetches:
 //   K-contiguous operand: LDS row = 128 B (8 chunks); chunk c of row r sits at slot c ^ ((r >> 1) & 7),
@@ -21,58 +18,96 @@ namespace mi {
 
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 
-namespace fast {
-constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int WGM = 2, WGN = 4, NW = WGM * WGN, NT = NW * 64;
-constexpr int TM = BM / WGM, TN = BN / WGN, FM = TM / 32, FN = TN / 32;
-constexpr int TILE_BYTES = 256 * BK * 2;  // one operand tile: 32 KB
-constexpr int STAGE_BYTES = 2 * TILE_BYTES;
-constexpr int LPT = TILE_BYTES / 1024 / NW;  // direct-to-LDS loads per wavefront per operand tile (4)
-}  // namespace fast
+// Compile-time shape of one fast-kernel variant.
+template <int TILE_, int WGM_, int WGN_, int BK_, int NS_>
+struct FastCfg {
+  static constexpr int TILE = TILE_;  // square workgroup tile (rows of P == rows of Q per tile)
+  static constexpr int WGM = WGM_, WGN = WGN_, NW = WGM * WGN, NT = NW * 64;
+  static constexpr int TM = TILE / WGM, TN = TILE / WGN, FM = TM / 32, FN = TN / 32;
+  static constexpr int BK = BK_;                       // k extent of one ring slot
+  static constexpr int NS = NS_;                       // ring slots
+  static constexpr int TILE_BYTES = TILE * BK * 2;     // one operand tile
+  static constexpr int SLOT_BYTES = 2 * TILE_BYTES;
+  static constexpr int LPT = TILE_BYTES / 1024 / NW;   // direct-to-LDS loads per wavefront per operand tile
+  static constexpr int CPR = BK / 8;                   // 16-byte chunks per K-contiguous LDS row
+  static constexpr int ROWS_PER_KB = 1024 / (BK * 2);  // K-contiguous rows covered by one 1 KB load
+  static constexpr int KS_ROW_BYTES = TILE * 2;        // K-strided layout: one k-row
+  static_assert(BK == 32 || BK == 64, "ring slot depth");
+  static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of the 32 x 32 MFMA");
+  static_assert(TILE_BYTES % (1024 * NW) == 0, "tile must split evenly over the wavefronts' 1 KB loads");
+  static_assert(NS * SLOT_BYTES <= 160 * 1024 - 256, "ring exceeds the 160 KB LDS");
+};
+// MFMA-bound default: 256 x 256 tile, 8 wavefronts (2 per SIMD) of 128 x 64, two 64 KB slots.
+#ifndef MI_BIG_WGN
+#define MI_BIG_WGN 4
+#endif
+using CfgBig = FastCfg<256, 2, MI_BIG_WGN, 64, 2>;
+// SYRK on ~4096-row Gram matrices: 192 x 192 tiles give 22 * 23 / 2 = 253 lower-triangle tiles, one per
+// CU in a single round (256 x 256 tiles would give 136 and leave 47 % of the CUs idle).
+// 4 wavefronts of 96 x 96, three 48 KB slots (two K tiles in flight).
+using CfgSyrk192 = FastCfg<192, 2, 2, 64, 3>;
 
+// Direct-to-LDS load: every lane fetches 16 bytes from its own global address; the wavefront's 1 KB lands
+// at LDS byte address `lds_wave_base` + 16 * lane (the base travels in M0).  Written as inline assembly so
+// that completion is tracked only by the explicit s_waitcnt vmcnt(..) in the kernel: the compiler's own
+// bookkeeping would make every later LDS read wait for all outstanding loads, i.e. no prefetching.
 __device__ __forceinline__ void dma16(const uint16_t* g, char* lds_wave_base) {
-  __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)g,
-                                   (void __attribute__((address_space(3)))*)lds_wave_base, 16, 0, 0);
+  const uint32_t lds_addr = __builtin_amdgcn_readfirstlane(
+      (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_wave_base);  // wave-uniform by construction
+#ifndef MI_ABLATE_LOADS
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(g) : "memory", "m0");
+#endif
 }
 
-// Per-thread global pointers of the direct-to-LDS loads of one operand tile.
-template <bool KS>
+// XOR swizzle of the K-contiguous LDS tile: chunk c of row r is stored at slot kc_slot(r, c) of its row, so
+// that the 16 rows a quarter-wave reads (same chunk) cover all 64 banks.
+template <int BK>
+__device__ __forceinline__ int kc_slot(int row, int c) {
+  return BK == 64 ? (c ^ ((row >> 1) & 7)) : (c ^ ((row >> 2) & 3));
+}
+
+// Per-thread global pointers of the direct-to-LDS loads of one operand tile.  Rows beyond `rows_valid` are
+// redirected to the last valid row: they only feed output rows that the epilogue never stores.
+template <class C, bool KS>
 struct FastLoader {
-  const uint16_t* gp[fast::LPT];
+  const uint16_t* gp[C::LPT];
   int64_t step;  // elements to advance per K tile
 
-  __device__ __forceinline__ void init(const uint16_t* base, int64_t ld, int row0, int wave, int lane) {
+  __device__ __forceinline__ void init(const uint16_t* base, int64_t ld, int row0, int rows_valid, int wave, int lane) {
 #pragma unroll
-    for (int i = 0; i < fast::LPT; ++i) {
-      const int b = wave * fast::LPT + i;  // 1 KB block index inside the tile
+    for (int i = 0; i < C::LPT; ++i) {
+      const int b = wave * C::LPT + i;  // 1 KB block index inside the tile
       if (!KS) {
-        const int row = 8 * b + (lane >> 3);
-        const int c = (lane & 7) ^ ((row >> 1) & 7);
-        gp[i] = base + (int64_t)(row0 + row) * ld + c * 8;
+        const int row = C::ROWS_PER_KB * b + lane / C::CPR;
+        const int c = kc_slot<C::BK>(row, lane % C::CPR);  // the swizzle is an involution: slot -> chunk
+        int gr = row0 + row;
+        gr = gr < rows_valid ? gr : rows_valid - 1;
+        gp[i] = base + (int64_t)gr * ld + c * 8;
       } else {
+        static_assert(!KS || C::TILE == 256, "K-strided LDS layout is laid out for 256-wide tiles");
         const int k = 2 * b + (lane >> 5);
         const int c = ((lane & 31) - 4 * k) & 31;
         gp[i] = base + (int64_t)k * ld + row0 + c * 8;
       }
     }
-    step = KS ? (int64_t)fast::BK * ld : fast::BK;
+    step = KS ? (int64_t)C::BK * ld : C::BK;
   }
   __device__ __forceinline__ void issue(char* tile, int wave) {
 #pragma unroll
-    for (int i = 0; i < fast::LPT; ++i) {
-      dma16(gp[i], tile + (wave * fast::LPT + i) * 1024);
+    for (int i = 0; i < C::LPT; ++i) {
+      dma16(gp[i], tile + (wave * C::LPT + i) * 1024);
       gp[i] += step;
     }
   }
 };
 
 // MFMA fragment (8 bf16 along k) for 32 consecutive rows starting at `row_base`, k-step q (16 k each).
-template <bool KS>
+template <class C, bool KS>
 __device__ __forceinline__ bf16x8_t fast_frag(const char* tile, int row_base, int q, int lane) {
   if (!KS) {
     const int row = row_base + (lane & 31);
-    const int c = (2 * q + (lane >> 5)) ^ ((row >> 1) & 7);
-    return *reinterpret_cast<const bf16x8_t*>(tile + row * 128 + c * 16);
+    const int c = kc_slot<C::BK>(row, 2 * q + (lane >> 5));
+    return *reinterpret_cast<const bf16x8_t*>(tile + row * (C::BK * 2) + c * 16);
   } else {
     const int i16 = lane & 15;
     const int col = row_base + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
@@ -96,15 +131,21 @@ __device__ __forceinline__ bf16x8_t fast_frag(const char* tile, int row_base, in
   }
 }
 
-template <bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
-__global__ void __launch_bounds__(fast::NT) gemm_fast_kernel(GemmParams p) {
-  using namespace fast;
-  __shared__ __align__(1024) char stage0[STAGE_BYTES];
-  __shared__ __align__(1024) char stage1[STAGE_BYTES];
+// s_waitcnt immediate for gfx9: vmcnt in bits [3:0] and [15:14], expcnt [6:4] = 7 (no wait), lgkmcnt [11:8].
+constexpr int waitcnt_imm(int vmcnt, int lgkmcnt) {
+  return (vmcnt & 15) | ((vmcnt >> 4) << 14) | 0x70 | ((lgkmcnt & 15) << 8);
+}
+
+template <class C, bool P_KS, bool Q_KS, int MODE, bool OUT_F32, bool EDGE>
+__global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
+  constexpr int NS = C::NS, FM = C::FM, FN = C::FN, TILE_BYTES = C::TILE_BYTES, NT = C::NT;
+  // One array per ring slot: every LDS access below names its slot statically.
+  __shared__ __align__(1024) char ring[NS][C::SLOT_BYTES];
   __shared__ float red[NT / 64];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave % WGM, wn = wave / WGM;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: everything derived from it stays in SGPRs
+  const int wm = wave % C::WGM, wn = wave / C::WGM;
   const int64_t batch = blockIdx.y;
   int tm, tn;
   if (MODE == MODE_SYRK) {
@@ -113,12 +154,12 @@ __global__ void __launch_bounds__(fast::NT) gemm_fast_kernel(GemmParams p) {
     tm = (int)blockIdx.x % p.tiles_m;
     tn = (int)blockIdx.x / p.tiles_m;
   }
-  const int m0 = tm * BM, n0 = tn * BN;
+  const int m0 = tm * C::TILE, n0 = tn * C::TILE;
 
-  FastLoader<P_KS> lp;
-  FastLoader<Q_KS> lq;
-  lp.init(p.P + batch * p.p_bs, p.ldp, m0, wave, lane);
-  lq.init(p.Q + batch * p.q_bs, p.ldq, n0, wave, lane);
+  FastLoader<C, P_KS> lp;
+  FastLoader<C, Q_KS> lq;
+  lp.init(p.P + batch * p.p_bs, p.ldp, m0, p.M, wave, lane);
+  lq.init(p.Q + batch * p.q_bs, p.ldq, n0, p.N, wave, lane);
 
   f32x16_t acc[FM][FN];
 #pragma unroll
@@ -128,51 +169,76 @@ __global__ void __launch_bounds__(fast::NT) gemm_fast_kernel(GemmParams p) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-  const int nk = p.K / BK;
+  const int nk = p.K / C::BK;
+  constexpr int NQ = C::BK / 16;
+  constexpr int LOADS_PER_TILE = 2 * C::LPT;  // per thread, both operands
+  static_assert(NQ % 2 == 0, "fragment buffer parity assumes an even number of k-steps per tile");
+  static_assert((NS - 2) * LOADS_PER_TILE < 64, "vmcnt is a 6-bit counter");
 
-  auto compute = [&](const char* st) {
+  // Pipeline.  Ring slot kt % NS holds K tile kt.  While tile kt is multiplied, tiles kt+1 .. kt+NS-1 are in
+  // flight; the slot refilled at the top of tile kt is the one tile kt-1 occupied, which every wavefront left
+  // before the previous barrier.  Fragment registers are double buffered (the LDS reads of k-step q+1 run
+  // under the MFMAs of k-step q), and the barrier that publishes tile kt+1 sits before the last k-step of
+  // tile kt so that its skew and the first fragment reads of tile kt+1 are covered by that k-step's MFMAs.
+  bf16x8_t fp[2][FM], fq[2][FN];
+  auto fetch = [&](const char* st, int q, int buf) {
 #pragma unroll
-    for (int q = 0; q < BK / 16; ++q) {
-      bf16x8_t fp[FM], fq[FN];
+    for (int i = 0; i < FM; ++i) fp[buf][i] = fast_frag<C, P_KS>(st, wm * C::TM + i * 32, q, lane);
 #pragma unroll
-      for (int i = 0; i < FM; ++i) fp[i] = fast_frag<P_KS>(st, wm * TM + i * 32, q, lane);
+    for (int j = 0; j < FN; ++j) fq[buf][j] = fast_frag<C, Q_KS>(st + TILE_BYTES, wn * C::TN + j * 32, q, lane);
+  };
+  auto mma = [&](int buf) {
 #pragma unroll
-      for (int j = 0; j < FN; ++j) fq[j] = fast_frag<Q_KS>(st + TILE_BYTES, wn * TN + j * 32, q, lane);
+    for (int i = 0; i < FM; ++i)
 #pragma unroll
-      for (int i = 0; i < FM; ++i)
+      for (int j = 0; j < FN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fq[buf][j], fp[buf][i], acc[i][j], 0, 0, 0);
+  };
+  auto issue = [&](char* slot) {
+    lp.issue(slot, wave);
+    lq.issue(slot + TILE_BYTES, wave);
+  };
+  auto k_tile = [&](int kt, char* cur, char* nxt, char* refill) {
+    const bool refilled = kt + NS - 1 < nk;
+    if (refilled) issue(refill);  // tile kt+NS-1 -> slot (kt-1) % NS
 #pragma unroll
-        for (int j = 0; j < FN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fq[j], fp[i], acc[i][j], 0, 0, 0);
+    for (int q = 0; q + 1 < NQ; ++q) {
+      fetch(cur, q + 1, (q + 1) & 1);
+      mma(q & 1);
     }
+    // own loads of tile kt+1 have landed (younger tiles may stay in flight); own reads of `cur` are done
+    if (refilled)
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm((NS - 2) * LOADS_PER_TILE, 0));
+    else
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+#ifndef MI_ABLATE_BARRIER
+    __syncthreads();
+#endif
+    if (kt + 1 < nk) fetch(nxt, 0, 0);
+    mma((NQ - 1) & 1);
   };
 
-  lp.issue(stage0, wave);
-  lq.issue(stage0 + TILE_BYTES, wave);
-  // Two K tiles per trip so that each stage is a distinct LDS object in every statement.
-  for (int kt = 0; kt < nk; kt += 2) {
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's part of tile kt has landed
-    __syncthreads();
-    if (kt + 1 < nk) {
-      lp.issue(stage1, wave);
-      lq.issue(stage1 + TILE_BYTES, wave);
-    }
-    compute(stage0);
-    if (kt + 1 < nk) {
-      __builtin_amdgcn_s_waitcnt(0x0f70);
-      __syncthreads();
-      if (kt + 2 < nk) {
-        lp.issue(stage0, wave);
-        lq.issue(stage0 + TILE_BYTES, wave);
-      }
-      compute(stage1);
-    }
+  // prologue: tiles 0 .. NS-2 in flight, wait for tile 0
+#pragma unroll
+  for (int t = 0; t < NS - 1; ++t)
+    if (t < nk) issue(ring[t]);
+  if (nk >= NS - 1)
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm((NS - 2) * LOADS_PER_TILE, 15));
+  else
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+  __syncthreads();
+  fetch(ring[0], 0, 0);
+  for (int kt = 0; kt < nk; kt += NS) {
+#pragma unroll
+    for (int u = 0; u < NS; ++u)
+      if (kt + u < nk) k_tile(kt + u, ring[u], ring[(u + 1) % NS], ring[(u + NS - 1) % NS]);
   }
 
   float beta = p.beta;
   const float shift = resolve_shift<NT>(p, batch, red, beta);
   const bool diag = (MODE == MODE_SYRK) && (tm == tn);
-  tile_epilogue<MODE, OUT_F32, false, FM, FN, NT>(p, acc, m0 + wm * TM, n0 + wn * TN, lane, batch, diag, p.alpha, beta,
-                                                  shift, red);
+  tile_epilogue<MODE, OUT_F32, EDGE, FM, FN, NT>(p, acc, m0 + wm * C::TM, n0 + wn * C::TN, lane, batch, diag, p.alpha,
+                                                 beta, shift, red);
 }
 
 }  // namespace mi

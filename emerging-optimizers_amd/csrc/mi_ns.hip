@@ -100,28 +100,62 @@ static int launch_one(const GemmParams& p, int64_t batch, hipStream_t stream) {
   return MI_OK;
 }
 
-template <bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
+template <class C, bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
 static int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream) {
   GemmParams q = p;
-  q.tiles_m = p.M / fast::BM;
-  q.tiles_n = p.N / fast::BN;
+  q.tiles_m = (p.M + C::TILE - 1) / C::TILE;
+  q.tiles_n = (p.N + C::TILE - 1) / C::TILE;
   const int64_t tiles = (MODE == MODE_SYRK) ? (int64_t)q.tiles_m * (q.tiles_m + 1) / 2 : (int64_t)q.tiles_m * q.tiles_n;
   if (batch > 65535) return fail(MI_ERR_UNSUPPORTED_SHAPE, "batch %lld exceeds the grid limit 65535", (long long)batch);
   g_last_tiles = (int)tiles;
-  dim3 grid((unsigned)tiles, (unsigned)batch, 1), block(fast::NT, 1, 1);
-  hipLaunchKernelGGL((gemm_fast_kernel<P_KS, Q_KS, MODE, OUT_F32>), grid, block, 0, stream, q);
+  dim3 grid((unsigned)tiles, (unsigned)batch, 1), block(C::NT, 1, 1);
+  const bool edge = (p.M % C::TILE) != 0 || (p.N % C::TILE) != 0;
+  if (edge)
+    hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, true>), grid, block, 0, stream, q);
+  else
+    hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, false>), grid, block, 0, stream, q);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
   return MI_OK;
 }
 
-static bool fast_eligible(const GemmParams& p) {
-  return p.M >= 1024 && p.N >= 1024 && p.M % fast::BM == 0 && p.N % fast::BN == 0 && p.K % fast::BK == 0 && p.K >= fast::BK;
+static int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Device-wide compute units (workgroups that run concurrently at one fast-kernel workgroup per CU).
+static int num_cus() {
+  static int cached = 0;
+  if (!cached) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      cached = n;
+    else
+      cached = 256;
+  }
+  return cached;
+}
+
+// Picks the SYRK tile by modelled time: rounds of workgroups over the CUs times the work of one tile.
+// 4096 rows: 256-tiles -> 136 workgroups (1 round at full cost); 192-tiles -> 253 (1 round at 56 % of the cost).
+static bool syrk_prefers_192(int64_t n, int64_t batch) {
+  const int cus = num_cus();
+  auto cost = [&](int64_t tile, double per_tile) {
+    const int64_t t = ceil_div(n, tile);
+    return (double)ceil_div(t * (t + 1) / 2 * batch, cus) * per_tile;
+  };
+  // per-tile cost ~ tile^2, with a penalty for the 4-wavefront variant's lower MFMA duty cycle
+  return cost(192, 192.0 * 192.0 * 1.15) < cost(256, 256.0 * 256.0);
 }
 
 template <bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
 static int launch_class(TileClass tc, const GemmParams& p, int64_t batch, hipStream_t stream) {
-  if (fast_eligible(p)) return launch_fast<P_KS, Q_KS, MODE, OUT_F32>(p, batch, stream);
+  const bool k_ok = p.K % 64 == 0 && p.K >= 64;
+  if (k_ok && p.M >= 1024 && p.N >= 1024) {
+    if constexpr (MODE == MODE_SYRK && !P_KS && !Q_KS) {
+      if (syrk_prefers_192(p.M, batch)) return launch_fast<CfgSyrk192, false, false, MODE, OUT_F32>(p, batch, stream);
+    }
+    if (p.M % 256 == 0 && p.N % 256 == 0) return launch_fast<CfgBig, P_KS, Q_KS, MODE, OUT_F32>(p, batch, stream);
+  }
   switch (tc) {
     case TILE_BIG:
       return launch_one<256, 256, 64, 2, 2, P_KS, Q_KS, MODE, OUT_F32>(p, batch, stream);
