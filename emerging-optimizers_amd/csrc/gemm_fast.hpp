@@ -131,6 +131,112 @@ __device__ __forceinline__ bf16x8_t fast_frag(const char* tile, int row_base, in
   }
 }
 
+// Workgroup id -> GEMM tile.  Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its
+// own L2, so id % 8 names the XCD and id / 8 the position in that XCD's queue.  Each XCD gets a contiguous
+// range of tile columns (all tile rows), walked in blocks of XCD_BLOCK_M tile rows: the ~32 tiles an XCD
+// works on at one time then form a compact block that shares P row-panels and Q column-panels in L2.
+#ifndef MI_XCD_BLOCK_M
+#define MI_XCD_BLOCK_M 8
+#endif
+__device__ __forceinline__ void gemm_tile_of(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+  constexpr int XCDS = 8;
+  const int total = tiles_m * tiles_n;
+  if (MI_XCD_BLOCK_M == 0 || tiles_n % XCDS != 0 || tiles_m % MI_XCD_BLOCK_M != 0) {
+    tm = pid % tiles_m;
+    tn = pid / tiles_m;
+    return;
+  }
+  (void)total;
+  const int xcd = pid % XCDS, local = pid / XCDS;
+  const int cols_per_xcd = tiles_n / XCDS;
+  const int block = MI_XCD_BLOCK_M * cols_per_xcd;  // tiles in one row-block of this XCD's column range
+  const int rb = local / block, r = local % block;
+  tm = rb * MI_XCD_BLOCK_M + r % MI_XCD_BLOCK_M;
+  tn = xcd * cols_per_xcd + r / MI_XCD_BLOCK_M;
+}
+
+// GEMM-mode epilogue through LDS.  In the MFMA accumulator layout a lane owns one output row and scattered
+// 4-column groups, so direct global accesses touch 32 rows per instruction.  Here every wavefront parks one
+// 32-row block of its accumulators in its own LDS region (float32, rows padded by 16 bytes against bank
+// conflicts), then re-reads it so that 8 consecutive lanes cover 64 consecutive columns of one row: the
+// Cin loads and the stores become 16-byte-per-lane, 128-byte-per-row accesses.  No workgroup barrier is
+// needed between the passes: a wavefront only touches its own region and LDS operations of one wavefront
+// complete in order.
+template <class C, bool OUT_F32, bool GUARD>
+__device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16_t (&acc)[C::FM][C::FN], char* lds, int wave,
+                                                  int lane, int m_base, int n_base, int64_t batch, float alpha,
+                                                  float beta, float* red) {
+  constexpr int TN = C::TN, ROWB = TN * 4 + 16;
+  constexpr int LPR = TN / 8;    // lanes per output row (8 columns each)
+  constexpr int RPI = 64 / LPR;  // rows per read iteration
+  static_assert(32 % RPI == 0 && 64 % LPR == 0, "wave tile width must be 32, 64 or 128");
+  static_assert(C::NW * 32 * ROWB <= C::NS * C::SLOT_BYTES, "epilogue staging exceeds the ring");
+  char* reg = lds + wave * (32 * ROWB);
+  const int frow = lane & 31, fk = lane >> 5;
+  const int rr = lane / LPR, cc = (lane % LPR) * 8;
+  const uint16_t* __restrict__ Cb = p.Cin ? p.Cin + batch * p.c_bs : nullptr;
+  const bool use_c = beta != 0.0f && Cb != nullptr;
+  constexpr int NIT = 32 / RPI;
+  // All Cin pieces of this lane are requested up front (the fragment registers of the main loop are dead by
+  // now), so the global-load latency is paid once instead of once per piece.
+  uint4 cin[C::FM][NIT];
+#pragma unroll
+  for (int i = 0; i < C::FM; ++i)
+#pragma unroll
+    for (int t = 0; t < NIT; ++t) {
+      const int m = m_base + i * 32 + t * RPI + rr, n = n_base + cc;
+      cin[i][t] = make_uint4(0u, 0u, 0u, 0u);
+      if (use_c && (!GUARD || (m < p.M && n < p.N))) cin[i][t] = *reinterpret_cast<const uint4*>(Cb + (int64_t)m * p.ldc + n);
+    }
+  float ssq = 0.0f;
+#pragma unroll
+  for (int i = 0; i < C::FM; ++i) {
+#pragma unroll
+    for (int j = 0; j < C::FN; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4_t v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+        *reinterpret_cast<f32x4_t*>(reg + frow * ROWB + (j * 32 + 8 * g + 4 * fk) * 4) = v;
+      }
+#pragma unroll
+    for (int t = 0; t < NIT; ++t) {
+      const int row = t * RPI + rr;
+      const int m = m_base + i * 32 + row, n = n_base + cc;
+      f32x4_t lo = *reinterpret_cast<const f32x4_t*>(reg + row * ROWB + cc * 4);
+      f32x4_t hi = *reinterpret_cast<const f32x4_t*>(reg + row * ROWB + cc * 4 + 16);
+      if (GUARD && (m >= p.M || n >= p.N)) continue;
+      lo *= alpha;
+      hi *= alpha;
+      if (use_c) {
+        const uint32_t w[4] = {cin[i][t].x, cin[i][t].y, cin[i][t].z, cin[i][t].w};
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          lo[2 * e] = __builtin_fmaf(beta, __uint_as_float(w[e] << 16), lo[2 * e]);
+          lo[2 * e + 1] = __builtin_fmaf(beta, __uint_as_float(w[e] & 0xffff0000u), lo[2 * e + 1]);
+          hi[2 * e] = __builtin_fmaf(beta, __uint_as_float(w[2 + e] << 16), hi[2 * e]);
+          hi[2 * e + 1] = __builtin_fmaf(beta, __uint_as_float(w[2 + e] & 0xffff0000u), hi[2 * e + 1]);
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ssq = __builtin_fmaf(lo[e], lo[e], __builtin_fmaf(hi[e], hi[e], ssq));
+      if (OUT_F32) {
+        float* o = reinterpret_cast<float*>(p.Out) + batch * p.o_bs + (int64_t)m * p.ldo + n;
+        *reinterpret_cast<f32x4_t*>(o) = lo * p.out_scale;
+        *reinterpret_cast<f32x4_t*>(o + 4) = hi * p.out_scale;
+      } else {
+        uint16_t* o = reinterpret_cast<uint16_t*>(p.Out) + batch * p.o_bs + (int64_t)m * p.ldo + n;
+        const uint2 a = __builtin_bit_cast(uint2, __builtin_convertvector(lo, bf16x4_t));
+        const uint2 b = __builtin_bit_cast(uint2, __builtin_convertvector(hi, bf16x4_t));
+        *reinterpret_cast<uint4*>(o) = make_uint4(a.x, a.y, b.x, b.y);
+      }
+    }
+  }
+  if (p.slots_out != nullptr) {
+    const float total = block_sum_f32<C::NT>(ssq, red);
+    if (threadIdx.x == 0) p.slots_out[batch * gridDim.x + blockIdx.x] = total;
+  }
+}
+
 // s_waitcnt immediate for gfx9: vmcnt in bits [3:0] and [15:14], expcnt [6:4] = 7 (no wait), lgkmcnt [11:8].
 constexpr int waitcnt_imm(int vmcnt, int lgkmcnt) {
   return (vmcnt & 15) | ((vmcnt >> 4) << 14) | 0x70 | ((lgkmcnt & 15) << 8);
@@ -151,8 +257,7 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   if (MODE == MODE_SYRK) {
     tri_decode((int)blockIdx.x, tm, tn);
   } else {
-    tm = (int)blockIdx.x % p.tiles_m;
-    tn = (int)blockIdx.x / p.tiles_m;
+    gemm_tile_of((int)blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
   }
   const int m0 = tm * C::TILE, n0 = tn * C::TILE;
 
@@ -180,6 +285,9 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   // before the previous barrier.  Fragment registers are double buffered (the LDS reads of k-step q+1 run
   // under the MFMAs of k-step q), and the barrier that publishes tile kt+1 sits before the last k-step of
   // tile kt so that its skew and the first fragment reads of tile kt+1 are covered by that k-step's MFMAs.
+#ifdef MI_TIMING
+  long long t_load = 0, t_bar = 0;
+#endif
   bf16x8_t fp[2][FM], fq[2][FN];
   auto fetch = [&](const char* st, int q, int buf) {
 #pragma unroll
@@ -188,11 +296,17 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
     for (int j = 0; j < FN; ++j) fq[buf][j] = fast_frag<C, Q_KS>(st + TILE_BYTES, wn * C::TN + j * 32, q, lane);
   };
   auto mma = [&](int buf) {
+#ifdef MI_SETPRIO
+    __builtin_amdgcn_s_setprio(MI_SETPRIO);
+#endif
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
       for (int j = 0; j < FN; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fq[buf][j], fp[buf][i], acc[i][j], 0, 0, 0);
+#ifdef MI_SETPRIO
+    __builtin_amdgcn_s_setprio(0);
+#endif
   };
   auto issue = [&](char* slot) {
     lp.issue(slot, wave);
@@ -207,17 +321,32 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
       mma(q & 1);
     }
     // own loads of tile kt+1 have landed (younger tiles may stay in flight); own reads of `cur` are done
+#ifdef MI_TIMING
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
+    const long long tw0 = __builtin_readcyclecounter();
+#endif
     if (refilled)
       __builtin_amdgcn_s_waitcnt(waitcnt_imm((NS - 2) * LOADS_PER_TILE, 0));
     else
       __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+#ifdef MI_TIMING
+    const long long tw1 = __builtin_readcyclecounter();
+#endif
 #ifndef MI_ABLATE_BARRIER
     __syncthreads();
+#endif
+#ifdef MI_TIMING
+    const long long tw2 = __builtin_readcyclecounter();
+    t_load += tw1 - tw0;
+    t_bar += tw2 - tw1;
 #endif
     if (kt + 1 < nk) fetch(nxt, 0, 0);
     mma((NQ - 1) & 1);
   };
 
+#ifdef MI_TIMING
+  const long long t_start = __builtin_readcyclecounter();
+#endif
   // prologue: tiles 0 .. NS-2 in flight, wait for tile 0
 #pragma unroll
   for (int t = 0; t < NS - 1; ++t)
@@ -234,11 +363,31 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
       if (kt + u < nk) k_tile(kt + u, ring[u], ring[(u + 1) % NS], ring[(u + NS - 1) % NS]);
   }
 
+#ifdef MI_TIMING
+  const long long t_loop = __builtin_readcyclecounter();
+#endif
   float beta = p.beta;
   const float shift = resolve_shift<NT>(p, batch, red, beta);
   const bool diag = (MODE == MODE_SYRK) && (tm == tn);
-  tile_epilogue<MODE, OUT_F32, EDGE, FM, FN, NT>(p, acc, m0 + wm * C::TM, n0 + wn * C::TN, lane, batch, diag, p.alpha,
-                                                 beta, shift, red);
+  if constexpr (MODE == MODE_GEMM && (C::TN == 32 || C::TN == 64 || C::TN == 128)) {
+    __syncthreads();  // every wavefront has finished reading the ring: it can be reused as staging space
+    gemm_epilogue_lds<C, OUT_F32, EDGE>(p, acc, &ring[0][0], wave, lane, m0 + wm * C::TM, n0 + wn * C::TN, batch, p.alpha,
+                                        beta, red);
+  } else {
+    tile_epilogue<MODE, OUT_F32, EDGE, FM, FN, NT>(p, acc, m0 + wm * C::TM, n0 + wn * C::TN, lane, batch, diag, p.alpha,
+                                                   beta, shift, red);
+  }
+#ifdef MI_TIMING
+  if (p.slots_in && lane == 0) {  // debug build only: slots_in doubles as the timing dump
+    __builtin_amdgcn_s_waitcnt(0);
+    const long long t_end = __builtin_readcyclecounter();
+    long long* dump = (long long*)p.slots_in + ((long long)blockIdx.x * C::NW + wave) * 4;
+    dump[0] = t_load;
+    dump[1] = t_bar;
+    dump[2] = t_loop - t_start;
+    dump[3] = t_end - t_loop;
+  }
+#endif
 }
 
 }  // namespace mi

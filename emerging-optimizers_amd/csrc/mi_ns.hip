@@ -5,6 +5,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -252,6 +253,9 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
   p.beta = beta;
   p.out_scale = out_scale;
   if (sh) sh->apply(p);
+#ifdef MI_TIMING
+  p.slots_in = reinterpret_cast<const float*>(getenv("MI_TIMING_PTR") ? strtoull(getenv("MI_TIMING_PTR"), nullptr, 0) : 0ull);
+#endif
   TileClass tc = pick_class(m);
   if (!x_trans) {
     // OUT (m x n): P = Bm rows (K-contiguous), Q[j][k] = X[k][j] (K-strided).
