@@ -71,6 +71,40 @@ __device__ __forceinline__ void tri_decode(int pid, int& ti, int& tj) {
   tj = pid - t * (t + 1) / 2;
 }
 
+// Locality-preserving enumeration of the lower-triangle tiles for the XCD-aware SYRK launch.
+// The triangle is cut into block-rows of TRI_BLOCK tile rows; inside a block-row the full
+// TRI_BLOCK-wide rectangles come first (row-major inside each), then the triangular block on the
+// diagonal.  Consecutive sequence numbers therefore stay inside a ~TRI_BLOCK x TRI_BLOCK block that
+// touches only ~2 TRI_BLOCK operand panels.  `s` must be < T (T + 1) / 2.
+constexpr int TRI_BLOCK = 6;
+__device__ __host__ inline void tri_block_decode(int s, int T, int& ti, int& tj) {
+  // block-row: the plain row-major row of s tells which band of TRI_BLOCK rows s falls into
+  int r = 0;
+#if defined(__HIP_DEVICE_COMPILE__)
+  r = (int)((sqrtf(8.0f * (float)s + 1.0f) - 1.0f) * 0.5f);
+#else
+  while ((r + 1) * (r + 2) / 2 <= s) ++r;
+#endif
+  while ((r + 1) * (r + 2) / 2 <= s) ++r;
+  while (r * (r + 1) / 2 > s) --r;
+  const int bi = r / TRI_BLOCK;
+  const int row0 = bi * TRI_BLOCK;
+  const int h = (T - row0) < TRI_BLOCK ? (T - row0) : TRI_BLOCK;  // rows in this block-row
+  int u = s - row0 * (row0 + 1) / 2;                               // index inside the block-row
+  const int rect = h * TRI_BLOCK;                                  // tiles per full rectangle
+  if (u < bi * rect) {
+    const int bj = u / rect, v = u % rect;
+    ti = row0 + v / TRI_BLOCK;
+    tj = bj * TRI_BLOCK + v % TRI_BLOCK;
+    return;
+  }
+  u -= bi * rect;  // triangular block on the diagonal: plain row-major triangle
+  int lr = 0;
+  while ((lr + 1) * (lr + 2) / 2 <= u) ++lr;
+  ti = row0 + lr;
+  tj = row0 + (u - lr * (lr + 1) / 2);
+}
+
 __device__ __forceinline__ uint32_t dword_of(const uint4& v, int c) {
   return c == 0 ? v.x : (c == 1 ? v.y : (c == 2 ? v.z : v.w));
 }

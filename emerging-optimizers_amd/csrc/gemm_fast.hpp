@@ -19,10 +19,13 @@ namespace mi {
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 
 // Compile-time shape of one fast-kernel variant.
-template <int TILE_, int WGM_, int WGN_, int BK_, int NS_>
+template <int TILE_, int WGM_, int WGN_, int BK_, int NS_, int KSPLIT_ = 1>
 struct FastCfg {
   static constexpr int TILE = TILE_;  // square workgroup tile (rows of P == rows of Q per tile)
-  static constexpr int WGM = WGM_, WGN = WGN_, NW = WGM * WGN, NT = NW * 64;
+  // KSPLIT groups of WGM x WGN wavefronts each cover the whole tile and take alternate 16-wide k-steps; their
+  // accumulators are added through LDS after the K loop (two wavefronts per SIMD with large wave tiles).
+  static constexpr int KSPLIT = KSPLIT_;
+  static constexpr int WGM = WGM_, WGN = WGN_, NWG = WGM * WGN, NW = NWG * KSPLIT, NT = NW * 64;
   static constexpr int TM = TILE / WGM, TN = TILE / WGN, FM = TM / 32, FN = TN / 32;
   static constexpr int BK = BK_;                       // k extent of one ring slot
   static constexpr int NS = NS_;                       // ring slots
@@ -33,6 +36,8 @@ struct FastCfg {
   static constexpr int ROWS_PER_KB = 1024 / (BK * 2);  // K-contiguous rows covered by one 1 KB load
   static constexpr int KS_ROW_BYTES = TILE * 2;        // K-strided layout: one k-row
   static_assert(BK == 32 || BK == 64, "ring slot depth");
+  static_assert(KSPLIT == 1 || KSPLIT == 2, "at most two K groups");
+  static_assert((BK / 16) % (2 * KSPLIT) == 0 || KSPLIT == 1, "each K group needs an even number of k-steps per tile");
   static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of the 32 x 32 MFMA");
   static_assert(TILE_BYTES % (1024 * NW) == 0, "tile must split evenly over the wavefronts' 1 KB loads");
   static_assert(NS * SLOT_BYTES <= 160 * 1024 - 256, "ring exceeds the 160 KB LDS");
@@ -44,8 +49,11 @@ struct FastCfg {
 using CfgBig = FastCfg<256, 2, MI_BIG_WGN, 64, 2>;
 // SYRK on ~4096-row Gram matrices: 192 x 192 tiles give 22 * 23 / 2 = 253 lower-triangle tiles, one per
 // CU in a single round (256 x 256 tiles would give 136 and leave 47 % of the CUs idle).
-// 4 wavefronts of 96 x 96, three 48 KB slots (two K tiles in flight).
-using CfgSyrk192 = FastCfg<192, 2, 2, 64, 3>;
+// 2 K-groups x 4 wavefronts of 96 x 96, three 48 KB slots (two K tiles in flight).
+#ifndef MI_SYRK192_KSPLIT
+#define MI_SYRK192_KSPLIT 2
+#endif
+using CfgSyrk192 = FastCfg<192, 2, 2, 64, 3, MI_SYRK192_KSPLIT>;
 
 // Direct-to-LDS load: every lane fetches 16 bytes from its own global address; the wavefront's 1 KB lands
 // at LDS byte address `lds_wave_base` + 16 * lane (the base travels in M0).  Written as inline assembly so
@@ -179,18 +187,24 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16_t 
   constexpr int NIT = 32 / RPI;
   // All Cin pieces of this lane are requested up front (the fragment registers of the main loop are dead by
   // now), so the global-load latency is paid once instead of once per piece.
+  constexpr bool PREFETCH_ALL = C::FM * NIT * 4 <= 64;  // else one 32-row block at a time (register budget)
   uint4 cin[C::FM][NIT];
-#pragma unroll
-  for (int i = 0; i < C::FM; ++i)
+  auto load_cin = [&](int i) {
 #pragma unroll
     for (int t = 0; t < NIT; ++t) {
       const int m = m_base + i * 32 + t * RPI + rr, n = n_base + cc;
       cin[i][t] = make_uint4(0u, 0u, 0u, 0u);
       if (use_c && (!GUARD || (m < p.M && n < p.N))) cin[i][t] = *reinterpret_cast<const uint4*>(Cb + (int64_t)m * p.ldc + n);
     }
+  };
+  if (PREFETCH_ALL) {
+#pragma unroll
+    for (int i = 0; i < C::FM; ++i) load_cin(i);
+  }
   float ssq = 0.0f;
 #pragma unroll
   for (int i = 0; i < C::FM; ++i) {
+    if (!PREFETCH_ALL) load_cin(i);
 #pragma unroll
     for (int j = 0; j < C::FN; ++j)
 #pragma unroll
@@ -251,11 +265,18 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: everything derived from it stays in SGPRs
-  const int wm = wave % C::WGM, wn = wave / C::WGM;
+  const int kgroup = wave / C::NWG, wig = wave % C::NWG;  // K group and position inside it
+  const int wm = wig % C::WGM, wn = wig / C::WGM;
   const int64_t batch = blockIdx.y;
   int tm, tn;
   if (MODE == MODE_SYRK) {
-    tri_decode((int)blockIdx.x, tm, tn);
+    // The grid is padded to a multiple of 8 workgroups: id % 8 names the XCD (round-robin dispatch), and
+    // each XCD takes one contiguous chunk of the blocked triangular enumeration.
+    const int total = p.tiles_m * (p.tiles_m + 1) / 2;
+    const int per_xcd = (int)gridDim.x / 8;
+    const int s = ((int)blockIdx.x % 8) * per_xcd + (int)blockIdx.x / 8;
+    if (s >= total) return;  // padding workgroup (whole workgroup leaves before any barrier)
+    tri_block_decode(s, p.tiles_m, tm, tn);
   } else {
     gemm_tile_of((int)blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
   }
@@ -275,7 +296,7 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   const int nk = p.K / C::BK;
-  constexpr int NQ = C::BK / 16;
+  constexpr int NQ = C::BK / 16 / C::KSPLIT;  // k-steps of one tile that this wavefront multiplies
   constexpr int LOADS_PER_TILE = 2 * C::LPT;  // per thread, both operands
   static_assert(NQ % 2 == 0, "fragment buffer parity assumes an even number of k-steps per tile");
   static_assert((NS - 2) * LOADS_PER_TILE < 64, "vmcnt is a 6-bit counter");
@@ -291,9 +312,10 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   bf16x8_t fp[2][FM], fq[2][FN];
   auto fetch = [&](const char* st, int q, int buf) {
 #pragma unroll
-    for (int i = 0; i < FM; ++i) fp[buf][i] = fast_frag<C, P_KS>(st, wm * C::TM + i * 32, q, lane);
+    for (int i = 0; i < FM; ++i) fp[buf][i] = fast_frag<C, P_KS>(st, wm * C::TM + i * 32, q * C::KSPLIT + kgroup, lane);
 #pragma unroll
-    for (int j = 0; j < FN; ++j) fq[buf][j] = fast_frag<C, Q_KS>(st + TILE_BYTES, wn * C::TN + j * 32, q, lane);
+    for (int j = 0; j < FN; ++j)
+      fq[buf][j] = fast_frag<C, Q_KS>(st + TILE_BYTES, wn * C::TN + j * 32, q * C::KSPLIT + kgroup, lane);
   };
   auto mma = [&](int buf) {
 #ifdef MI_SETPRIO
@@ -319,6 +341,16 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
     for (int q = 0; q + 1 < NQ; ++q) {
       fetch(cur, q + 1, (q + 1) & 1);
       mma(q & 1);
+#ifndef MI_NO_SCHED_INTERLEAVE
+      // one LDS read issued in the shadow of every MFMA
+      constexpr int READS = FM * (P_KS ? 2 : 1) + FN * (Q_KS ? 2 : 1);
+      constexpr int MMAS = FM * FN;
+#pragma unroll
+      for (int x = 0; x < MMAS; ++x) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, (READS + MMAS - 1) / MMAS, 0);
+      }
+#endif
     }
     // own loads of tile kt+1 have landed (younger tiles may stay in flight); own reads of `cur` are done
 #ifdef MI_TIMING
@@ -363,6 +395,37 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
       if (kt + u < nk) k_tile(kt + u, ring[u], ring[(u + 1) % NS], ring[(u + NS - 1) % NS]);
   }
 
+  if constexpr (C::KSPLIT == 2) {
+    // Sum the two K groups: group 1 parks its accumulators in the ring (lane-linear, conflict free),
+    // group 0 adds them and carries on with the epilogue alone.
+    static_assert(C::KSPLIT == 1 || C::NWG * FM * FN * 4096 <= NS * C::SLOT_BYTES, "accumulators exceed the ring");
+    __syncthreads();  // all fragment reads of the ring are done
+    char* park = &ring[0][0] + wig * (FM * FN * 4096);
+    if (kgroup == 1) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            f32x4_t v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+            *reinterpret_cast<f32x4_t*>(park + ((i * FN + j) * 4 + g) * 1024 + lane * 16) = v;
+          }
+    }
+    __syncthreads();
+    if (kgroup == 0) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const f32x4_t v = *reinterpret_cast<const f32x4_t*>(park + ((i * FN + j) * 4 + g) * 1024 + lane * 16);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[i][j][4 * g + r] += v[r];
+          }
+    }
+  }
 #ifdef MI_TIMING
   const long long t_loop = __builtin_readcyclecounter();
 #endif
@@ -374,8 +437,11 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
     gemm_epilogue_lds<C, OUT_F32, EDGE>(p, acc, &ring[0][0], wave, lane, m0 + wm * C::TM, n0 + wn * C::TN, batch, p.alpha,
                                         beta, red);
   } else {
-    tile_epilogue<MODE, OUT_F32, EDGE, FM, FN, NT>(p, acc, m0 + wm * C::TM, n0 + wn * C::TN, lane, batch, diag, p.alpha,
-                                                   beta, shift, red);
+    static_assert(C::KSPLIT == 1 || MODE == MODE_SYRK, "the K-group variant is wired for SYRK only");
+    // (SYRK never takes the per-workgroup sum at the end of tile_epilogue, so group 1 may simply skip it)
+    if (C::KSPLIT == 1 || kgroup == 0)
+      tile_epilogue<MODE, OUT_F32, EDGE, FM, FN, NT>(p, acc, m0 + wm * C::TM, n0 + wn * C::TN, lane, batch, diag, p.alpha,
+                                                     beta, shift, red);
   }
 #ifdef MI_TIMING
   if (p.slots_in && lane == 0) {  // debug build only: slots_in doubles as the timing dump

@@ -106,7 +106,8 @@ static int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream) {
   GemmParams q = p;
   q.tiles_m = (p.M + C::TILE - 1) / C::TILE;
   q.tiles_n = (p.N + C::TILE - 1) / C::TILE;
-  const int64_t tiles = (MODE == MODE_SYRK) ? (int64_t)q.tiles_m * (q.tiles_m + 1) / 2 : (int64_t)q.tiles_m * q.tiles_n;
+  int64_t tiles = (MODE == MODE_SYRK) ? (int64_t)q.tiles_m * (q.tiles_m + 1) / 2 : (int64_t)q.tiles_m * q.tiles_n;
+  if (MODE == MODE_SYRK) tiles = (tiles + 7) / 8 * 8;  // XCD-chunked enumeration: grid padded to a multiple of 8
   if (batch > 65535) return fail(MI_ERR_UNSUPPORTED_SHAPE, "batch %lld exceeds the grid limit 65535", (long long)batch);
   g_last_tiles = (int)tiles;
   dim3 grid((unsigned)tiles, (unsigned)batch, 1), block(C::NT, 1, 1);
@@ -219,6 +220,9 @@ static int syrk_impl(const void* A, int64_t batch, int64_t n, int64_t k, int64_t
   p.out_scale = 1.0f;
   p.skip_upper = skip_upper ? 1 : 0;
   if (sh) sh->apply(p);
+#ifdef MI_TIMING
+  p.slots_in = reinterpret_cast<const float*>(getenv("MI_TIMING_PTR") ? strtoull(getenv("MI_TIMING_PTR"), nullptr, 0) : 0ull);
+#endif
   TileClass tc = pick_class(n);
   return a_trans ? launch_class<true, true, MODE_SYRK, false>(tc, p, batch, stream)
                  : launch_class<false, false, MODE_SYRK, false>(tc, p, batch, stream);

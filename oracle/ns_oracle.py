@@ -358,3 +358,21 @@ def flops_sym(m: int, n: int, steps: int, batch: int = 1) -> int:
 
 
 __all__ = [name for name in dir() if not name.startswith("_") and name not in ("itertools", "math", "np")]
+
+
+def tri_block_decode(s: int, T: int, block: int = 6) -> tuple[int, int]:
+    """Blocked enumeration of the lower-triangle tiles used by the XCD-aware SYRK launch (build-specific, no
+    counterpart in the reference): block-rows of ``block`` tile rows; inside a block-row the full
+    ``block``-wide rectangles first (row-major), then the triangular block on the diagonal."""
+    r = (math.isqrt(8 * s + 1) - 1) // 2
+    bi = r // block
+    row0 = bi * block
+    h = min(block, T - row0)
+    u = s - row0 * (row0 + 1) // 2
+    rect = h * block
+    if u < bi * rect:
+        bj, v = divmod(u, rect)
+        return row0 + v // block, bj * block + v % block
+    u -= bi * rect
+    lr = (math.isqrt(8 * u + 1) - 1) // 2
+    return row0 + lr, row0 + (u - lr * (lr + 1) // 2)

@@ -282,3 +282,9 @@ def test_torch_cpu_restatement_matches_oracle():
         np.testing.assert_allclose(got, O.newton_schulz(x.numpy(), 5, "simple"), atol=2e-6)
     cub = ns_torch_cpu.newton_schulz_cpu(x, O.expand_coefficients(5, "cubic5")).numpy()
     np.testing.assert_allclose(cub, O.newton_schulz(x.numpy(), 5, "cubic5"), atol=2e-6)
+
+
+def test_tri_block_decode_bijection():
+    for T in [1, 2, 5, 6, 7, 11, 12, 13, 16, 22, 23, 40]:
+        seen = {O.tri_block_decode(s, T) for s in range(T * (T + 1) // 2)}
+        assert seen == {(i, j) for i in range(T) for j in range(i + 1)}, T
