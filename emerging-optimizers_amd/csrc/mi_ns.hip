@@ -406,9 +406,89 @@ __global__ void __launch_bounds__(NORM_THREADS) scale_cast_kernel(const float* _
   }
 }
 
+// Tall inputs (rows > cols): the divide + bf16 cast also transposes, so that the iteration can run on the
+// (cols x rows) orientation with K-contiguous operands (the fastest kernels), and the float32 result is
+// transposed back once at the end.  64 x 64 tiles through LDS, 16-byte global accesses on both sides.
+__global__ void __launch_bounds__(256) scale_cast_transpose_kernel(const float* __restrict__ x, int64_t rows, int64_t cols,
+                                                                   const double* __restrict__ partials, int nparts,
+                                                                   float eps, int f64, uint16_t* __restrict__ out,
+                                                                   float* __restrict__ dev_norm,
+                                                                   float* __restrict__ sumsq_out) {
+  const int64_t b = blockIdx.z;
+  __shared__ double scratch_d[NORM_THREADS / 64];
+  __shared__ float tile[64][65];
+  double s = 0;
+  for (int i = threadIdx.x; i < nparts; i += NORM_THREADS) s += partials[b * nparts + i];
+  s = block_sum<double>(s, scratch_d);
+  const float divisor = f64 ? (float)sqrt(s) : fmaxf(sqrtf((float)s), eps);
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+    if (dev_norm) dev_norm[b] = divisor;
+    if (sumsq_out) {
+      const float ratio = sqrtf((float)s) / divisor;
+      sumsq_out[b] = (divisor > 0.0f && ratio == ratio) ? ratio * ratio : 0.0f;
+    }
+  }
+  const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+  const float* __restrict__ xb = x + b * rows * cols;
+  // read 64 rows x 64 cols: thread t handles row t/4 (+ 16 per pass... 4 passes), 16 columns... use float4 x 4 passes
+#pragma unroll
+  for (int pass = 0; pass < 4; ++pass) {
+    const int r = pass * 16 + (threadIdx.x >> 4), c = (threadIdx.x & 15) * 4;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (r0 + r < rows && c0 + c < cols) v = *reinterpret_cast<const float4*>(xb + (r0 + r) * cols + c0 + c);
+    tile[r][c] = v.x / divisor;
+    tile[r][c + 1] = v.y / divisor;
+    tile[r][c + 2] = v.z / divisor;
+    tile[r][c + 3] = v.w / divisor;
+  }
+  __syncthreads();
+  // write transposed: out[(c0 + c)][r0 + r], 8 consecutive r per thread (16 bytes of bf16)
+  uint16_t* __restrict__ ob = out + b * rows * cols;
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int c = pass * 32 + (threadIdx.x >> 3), r = (threadIdx.x & 7) * 8;
+    if (c0 + c < cols && r0 + r < rows) {
+      f32x4_t lo = {tile[r][c], tile[r + 1][c], tile[r + 2][c], tile[r + 3][c]};
+      f32x4_t hi = {tile[r + 4][c], tile[r + 5][c], tile[r + 6][c], tile[r + 7][c]};
+      const uint2 a = __builtin_bit_cast(uint2, __builtin_convertvector(lo, bf16x4_t));
+      const uint2 d = __builtin_bit_cast(uint2, __builtin_convertvector(hi, bf16x4_t));
+      *reinterpret_cast<uint4*>(ob + (c0 + c) * rows + r0 + r) = make_uint4(a.x, a.y, d.x, d.y);
+    }
+  }
+}
+
+// out[b][c][r] = in[b][r][c] for float32 (rows x cols) -> (cols x rows); 64 x 64 tiles through LDS.
+__global__ void __launch_bounds__(256) transpose_f32_kernel(const float* __restrict__ in, int64_t rows, int64_t cols,
+                                                            float* __restrict__ out) {
+  const int64_t b = blockIdx.z;
+  __shared__ float tile[64][65];
+  const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+  const float* __restrict__ ib = in + b * rows * cols;
+  float* __restrict__ ob = out + b * rows * cols;
+#pragma unroll
+  for (int pass = 0; pass < 4; ++pass) {
+    const int r = pass * 16 + (threadIdx.x >> 4), c = (threadIdx.x & 15) * 4;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (r0 + r < rows && c0 + c < cols) v = *reinterpret_cast<const float4*>(ib + (r0 + r) * cols + c0 + c);
+    tile[r][c] = v.x;
+    tile[r][c + 1] = v.y;
+    tile[r][c + 2] = v.z;
+    tile[r][c + 3] = v.w;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int pass = 0; pass < 4; ++pass) {
+    const int c = pass * 16 + (threadIdx.x >> 4), r = (threadIdx.x & 15) * 4;
+    if (c0 + c < cols && r0 + r < rows) {
+      f32x4_t v = {tile[r][c], tile[r + 1][c], tile[r + 2][c], tile[r + 3][c]};
+      *reinterpret_cast<f32x4_t*>(ob + (c0 + c) * rows + r0 + r) = v;
+    }
+  }
+}
+
 static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, int f64, void* out, int out_bf16,
                      float post_scale, double* partials, float* dev_norm, hipStream_t stream,
-                     float* sumsq_out = nullptr) {
+                     float* sumsq_out = nullptr, int64_t t_rows = 0, int64_t t_cols = 0) {
   if (!x || !out || !partials) return fail(MI_ERR_BAD_ARG, "mi_frob_normalize: null pointer");
   if (batch < 0 || numel < 0) return fail(MI_ERR_BAD_ARG, "mi_frob_normalize: negative extent");
   if (numel % 8) return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_frob_normalize: numel must be a multiple of 8, got %lld", (long long)numel);
@@ -421,6 +501,15 @@ static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, in
     hipLaunchKernelGGL(sumsq_kernel<true>, grid1, block, 0, stream, x, numel, partials);
   else
     hipLaunchKernelGGL(sumsq_kernel<false>, grid1, block, 0, stream, x, numel, partials);
+  if (t_rows > 0) {
+    // bf16 output transposed to (t_cols x t_rows)
+    dim3 gridt((unsigned)((t_cols + 63) / 64), (unsigned)((t_rows + 63) / 64), (unsigned)batch);
+    hipLaunchKernelGGL(scale_cast_transpose_kernel, gridt, block, 0, stream, x, t_rows, t_cols, partials, nb, eps, f64,
+                       static_cast<uint16_t*>(out), dev_norm, sumsq_out);
+    hipError_t et = hipGetLastError();
+    if (et != hipSuccess) return fail(MI_ERR_LAUNCH, "mi_frob_normalize launch failed: %s", hipGetErrorString(et));
+    return MI_OK;
+  }
   int64_t want = (numel / 8 + (int64_t)NORM_THREADS * 4 - 1) / ((int64_t)NORM_THREADS * 4);
   if (want < 1) want = 1;
   if (want > 4096) want = 4096;
@@ -440,7 +529,7 @@ static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, in
 static size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct NsWorkspace {
-  size_t x0, x1, a, b, partials, norm, slots, shift, total;
+  size_t x0, x1, a, b, partials, norm, slots, shift, result, total;
   int64_t max_slots;
 };
 
@@ -460,6 +549,10 @@ static NsWorkspace ns_layout(int64_t batch, int64_t rows, int64_t cols) {
   w.max_slots = ((rows + 63) / 64) * ((cols + 63) / 64);
   w.slots = off; off += align_up((size_t)batch * w.max_slots * sizeof(float), 256);
   w.shift = off; off += align_up((size_t)batch * sizeof(float), 256);
+  // tall inputs iterate on the transposed orientation; their float32 result is staged here before the
+  // final transpose into `out`
+  w.result = off;
+  if (rows > cols) off += align_up((size_t)batch * rows * cols * sizeof(float), 256);
   w.total = off;
   return w;
 }
@@ -568,19 +661,22 @@ int mi_newton_schulz_bf16(const float* x, float* out, int64_t batch, int64_t row
 
   float* slots = reinterpret_cast<float*>(ws + w.slots);
   float* shift = reinterpret_cast<float*>(ws + w.shift);
+  // The iteration runs on the (m x n) orientation with m <= n, K-contiguous in memory.  A tall input is
+  // transposed while it is cast to bf16, and its float32 result is transposed back at the end.
+  const int tall = rows > cols;
+  const int trans = 0;
+  const int64_t m = tall ? cols : rows, n = tall ? rows : cols;
+  const int64_t ld = n;
+  const int64_t x_bs = numel, g_bs = m * m;
+  float* result = tall ? reinterpret_cast<float*>(ws + w.result) : out;
   int rc;
   {
     ProfScope prof(PROF_NORMALIZE, stream);
-    rc = frob_impl(x, batch, numel, eps, accumulate_fp64, xbuf[0], /*out_bf16=*/1, 1.0f, partials, norm, stream, slots);
+    rc = frob_impl(x, batch, numel, eps, accumulate_fp64, xbuf[0], /*out_bf16=*/1, 1.0f, partials, norm, stream, slots,
+                   tall ? rows : 0, tall ? cols : 0);
   }
   if (rc != MI_OK) return rc;
 
-  // The iteration runs on the (m x n) orientation with m <= n.  When rows > cols that orientation is
-  // the transpose of what memory holds, which the kernels read in place (a_trans / x_trans).
-  const int trans = rows > cols;
-  const int64_t m = trans ? cols : rows, n = trans ? rows : cols;
-  const int64_t ld = cols;  // row-major (rows x cols) in memory either way
-  const int64_t x_bs = numel, g_bs = m * m;
   int cur = 0;
   int nslots = 1;  // the normalisation kernel left one value per matrix
   for (int s = 0; s < steps; ++s) {
@@ -607,7 +703,7 @@ int mi_newton_schulz_bf16(const float* x, float* out, int64_t batch, int64_t row
       alpha = 1.0f;
     }
     // X' = (a + b s + c s^2) X + B' X      (cubic: (a + b s) X + b A' X)
-    void* dst = last ? static_cast<void*>(out) : static_cast<void*>(xbuf[cur ^ 1]);
+    void* dst = last ? static_cast<void*>(result) : static_cast<void*>(xbuf[cur ^ 1]);
     ShiftArgs sh_apply{SHIFT_APPLY, b, c, nullptr, 0, shift, last ? nullptr : slots};
     {
       ProfScope prof(PROF_APPLY, stream);
@@ -618,6 +714,13 @@ int mi_newton_schulz_bf16(const float* x, float* out, int64_t batch, int64_t row
     nslots = g_last_tiles;
     if (nslots > w.max_slots) return fail(MI_ERR_WORKSPACE, "internal: %d partial-sum slots exceed the %lld reserved", nslots, (long long)w.max_slots);
     cur ^= 1;
+  }
+  if (tall) {
+    ProfScope prof(PROF_NORMALIZE, stream);
+    dim3 gridt((unsigned)((n + 63) / 64), (unsigned)((m + 63) / 64), (unsigned)batch), blockt(256);
+    hipLaunchKernelGGL(transpose_f32_kernel, gridt, blockt, 0, stream, result, m, n, out);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "transpose launch failed: %s", hipGetErrorString(e));
   }
   return MI_OK;
 }
