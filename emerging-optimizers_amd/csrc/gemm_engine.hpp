@@ -47,7 +47,8 @@ struct GemmParams {
   const float* slots_in;     // SHIFT_GRAM: per-tile partial sums of squares of X, [batch][nslots_in]
   int nslots_in;
   float* shift_io;           // [batch]: written by SHIFT_GRAM, read by SHIFT_POLY / SHIFT_APPLY
-  float* slots_out;          // GEMM mode: per-tile sum of squares of the output, [batch][gridDim.x]
+  float* slots_out;          // GEMM mode: per-workgroup sum of squares of the output,
+  int slot_stride, slot_base;  //   at slots_out[batch * slot_stride + slot_base + blockIdx.x]
 };
 
 enum { SHIFT_NONE = 0, SHIFT_GRAM = 1, SHIFT_POLY = 2, SHIFT_APPLY = 3 };
@@ -324,7 +325,7 @@ __device__ __forceinline__ void tile_epilogue(const GemmParams& p, f32x16_t (&ac
   }
   if (MODE == MODE_GEMM && p.slots_out != nullptr) {
     const float total = block_sum_f32<NT>(ssq, red);
-    if (threadIdx.x == 0) p.slots_out[batch * gridDim.x + blockIdx.x] = total;
+    if (threadIdx.x == 0) p.slots_out[batch * p.slot_stride + p.slot_base + blockIdx.x] = total;
   }
 }
 

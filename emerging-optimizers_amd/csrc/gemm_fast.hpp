@@ -19,27 +19,29 @@ namespace mi {
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 
 // Compile-time shape of one fast-kernel variant.
-template <int TILE_, int WGM_, int WGN_, int BK_, int NS_, int KSPLIT_ = 1>
+template <int TILE_M_, int WGM_, int WGN_, int BK_, int NS_, int KSPLIT_ = 1, int TILE_N_ = TILE_M_>
 struct FastCfg {
-  static constexpr int TILE = TILE_;  // square workgroup tile (rows of P == rows of Q per tile)
+  static constexpr int TILE_M = TILE_M_, TILE_N = TILE_N_;  // workgroup tile: rows of P x rows of Q
+  static constexpr int TILE = TILE_M_;                      // (SYRK uses square tiles)
   // KSPLIT groups of WGM x WGN wavefronts each cover the whole tile and take alternate 16-wide k-steps; their
   // accumulators are added through LDS after the K loop (two wavefronts per SIMD with large wave tiles).
   static constexpr int KSPLIT = KSPLIT_;
   static constexpr int WGM = WGM_, WGN = WGN_, NWG = WGM * WGN, NW = NWG * KSPLIT, NT = NW * 64;
-  static constexpr int TM = TILE / WGM, TN = TILE / WGN, FM = TM / 32, FN = TN / 32;
+  static constexpr int TM = TILE_M / WGM, TN = TILE_N / WGN, FM = TM / 32, FN = TN / 32;
   static constexpr int BK = BK_;                       // k extent of one ring slot
   static constexpr int NS = NS_;                       // ring slots
-  static constexpr int TILE_BYTES = TILE * BK * 2;     // one operand tile
-  static constexpr int SLOT_BYTES = 2 * TILE_BYTES;
-  static constexpr int LPT = TILE_BYTES / 1024 / NW;   // direct-to-LDS loads per wavefront per operand tile
+  static constexpr int P_BYTES = TILE_M * BK * 2, Q_BYTES = TILE_N * BK * 2;  // operand tiles
+  static constexpr int SLOT_BYTES = P_BYTES + Q_BYTES;
+  static constexpr int LPT_P = P_BYTES / 1024 / NW;    // direct-to-LDS loads per wavefront per K tile
+  static constexpr int LPT_Q = Q_BYTES / 1024 / NW;
   static constexpr int CPR = BK / 8;                   // 16-byte chunks per K-contiguous LDS row
   static constexpr int ROWS_PER_KB = 1024 / (BK * 2);  // K-contiguous rows covered by one 1 KB load
-  static constexpr int KS_ROW_BYTES = TILE * 2;        // K-strided layout: one k-row
   static_assert(BK == 32 || BK == 64, "ring slot depth");
   static_assert(KSPLIT == 1 || KSPLIT == 2, "at most two K groups");
   static_assert((BK / 16) % (2 * KSPLIT) == 0 || KSPLIT == 1, "each K group needs an even number of k-steps per tile");
   static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of the 32 x 32 MFMA");
-  static_assert(TILE_BYTES % (1024 * NW) == 0, "tile must split evenly over the wavefronts' 1 KB loads");
+  static_assert(P_BYTES % (1024 * NW) == 0 && Q_BYTES % (1024 * NW) == 0,
+                "tiles must split evenly over the wavefronts' 1 KB loads");
   static_assert(NS * SLOT_BYTES <= 160 * 1024 - 256, "ring exceeds the 160 KB LDS");
 };
 // MFMA-bound default: 256 x 256 tile, 8 wavefronts (2 per SIMD) of 128 x 64, two 64 KB slots.
@@ -47,6 +49,8 @@ struct FastCfg {
 #define MI_BIG_WGN 4
 #endif
 using CfgBig = FastCfg<256, 2, MI_BIG_WGN, 64, 2>;
+// Half-width tile for the last partial round of a GEMM: 256 x 128, wavefronts of 128 x 32.
+using CfgHalfN = FastCfg<256, 2, 4, 64, 2, 1, 128>;
 // SYRK on ~4096-row Gram matrices: 192 x 192 tiles give 22 * 23 / 2 = 253 lower-triangle tiles, one per
 // CU in a single round (256 x 256 tiles would give 136 and leave 47 % of the CUs idle).
 // 2 K-groups x 4 wavefronts of 96 x 96, three 48 KB slots (two K tiles in flight).
@@ -76,15 +80,18 @@ __device__ __forceinline__ int kc_slot(int row, int c) {
 
 // Per-thread global pointers of the direct-to-LDS loads of one operand tile.  Rows beyond `rows_valid` are
 // redirected to the last valid row: they only feed output rows that the epilogue never stores.
-template <class C, bool KS>
+template <class C, bool KS, int ROWS>
 struct FastLoader {
-  const uint16_t* gp[C::LPT];
+  static constexpr int LPT = ROWS * C::BK * 2 / 1024 / C::NW;
+  static constexpr int KS_CHUNKS = ROWS / 8;          // 16-byte chunks per k-row of the K-strided layout
+  static constexpr int KS_ROWS_PER_KB = 512 / ROWS;   // k-rows covered by one 1 KB load
+  const uint16_t* gp[LPT];
   int64_t step;  // elements to advance per K tile
 
   __device__ __forceinline__ void init(const uint16_t* base, int64_t ld, int row0, int rows_valid, int wave, int lane) {
 #pragma unroll
-    for (int i = 0; i < C::LPT; ++i) {
-      const int b = wave * C::LPT + i;  // 1 KB block index inside the tile
+    for (int i = 0; i < LPT; ++i) {
+      const int b = wave * LPT + i;  // 1 KB block index inside the tile
       if (!KS) {
         const int row = C::ROWS_PER_KB * b + lane / C::CPR;
         const int c = kc_slot<C::BK>(row, lane % C::CPR);  // the swizzle is an involution: slot -> chunk
@@ -92,9 +99,9 @@ struct FastLoader {
         gr = gr < rows_valid ? gr : rows_valid - 1;
         gp[i] = base + (int64_t)gr * ld + c * 8;
       } else {
-        static_assert(!KS || C::TILE == 256, "K-strided LDS layout is laid out for 256-wide tiles");
-        const int k = 2 * b + (lane >> 5);
-        const int c = ((lane & 31) - 4 * k) & 31;
+        static_assert(!KS || ROWS == 256 || ROWS == 128, "K-strided LDS layout is laid out for 128/256-wide tiles");
+        const int k = KS_ROWS_PER_KB * b + lane / KS_CHUNKS;
+        const int c = ((lane % KS_CHUNKS) - 4 * k) & (KS_CHUNKS - 1);
         gp[i] = base + (int64_t)k * ld + row0 + c * 8;
       }
     }
@@ -102,16 +109,17 @@ struct FastLoader {
   }
   __device__ __forceinline__ void issue(char* tile, int wave) {
 #pragma unroll
-    for (int i = 0; i < C::LPT; ++i) {
-      dma16(gp[i], tile + (wave * C::LPT + i) * 1024);
+    for (int i = 0; i < LPT; ++i) {
+      dma16(gp[i], tile + (wave * LPT + i) * 1024);
       gp[i] += step;
     }
   }
 };
 
 // MFMA fragment (8 bf16 along k) for 32 consecutive rows starting at `row_base`, k-step q (16 k each).
-template <class C, bool KS>
+template <class C, bool KS, int ROWS>
 __device__ __forceinline__ bf16x8_t fast_frag(const char* tile, int row_base, int q, int lane) {
+  constexpr int KS_CHUNKS = ROWS / 8, KS_ROW_BYTES = ROWS * 2;
   if (!KS) {
     const int row = row_base + (lane & 31);
     const int c = kc_slot<C::BK>(row, 2 * q + (lane >> 5));
@@ -123,15 +131,15 @@ __device__ __forceinline__ bf16x8_t fast_frag(const char* tile, int row_base, in
     s16x4_t lo, hi;
     {
       const int k = kb;
-      const int slot = ((col >> 3) + 4 * k) & 31;
+      const int slot = ((col >> 3) + 4 * k) & (KS_CHUNKS - 1);
       lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (s16x4_t __attribute__((address_space(3)))*)(tile + k * 512 + slot * 16 + (col & 7) * 2));
+          (s16x4_t __attribute__((address_space(3)))*)(tile + k * KS_ROW_BYTES + slot * 16 + (col & 7) * 2));
     }
     {
       const int k = kb + 4;
-      const int slot = ((col >> 3) + 4 * k) & 31;
+      const int slot = ((col >> 3) + 4 * k) & (KS_CHUNKS - 1);
       hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (s16x4_t __attribute__((address_space(3)))*)(tile + k * 512 + slot * 16 + (col & 7) * 2));
+          (s16x4_t __attribute__((address_space(3)))*)(tile + k * KS_ROW_BYTES + slot * 16 + (col & 7) * 2));
     }
     typedef short s16x8_t __attribute__((ext_vector_type(8)));
     s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -247,7 +255,7 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16_t 
   }
   if (p.slots_out != nullptr) {
     const float total = block_sum_f32<C::NT>(ssq, red);
-    if (threadIdx.x == 0) p.slots_out[batch * gridDim.x + blockIdx.x] = total;
+    if (threadIdx.x == 0) p.slots_out[batch * p.slot_stride + p.slot_base + blockIdx.x] = total;
   }
 }
 
@@ -258,7 +266,7 @@ constexpr int waitcnt_imm(int vmcnt, int lgkmcnt) {
 
 template <class C, bool P_KS, bool Q_KS, int MODE, bool OUT_F32, bool EDGE>
 __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
-  constexpr int NS = C::NS, FM = C::FM, FN = C::FN, TILE_BYTES = C::TILE_BYTES, NT = C::NT;
+  constexpr int NS = C::NS, FM = C::FM, FN = C::FN, P_BYTES = C::P_BYTES, NT = C::NT;
   // One array per ring slot: every LDS access below names its slot statically.
   __shared__ __align__(1024) char ring[NS][C::SLOT_BYTES];
   __shared__ float red[NT / 64];
@@ -280,10 +288,10 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   } else {
     gemm_tile_of((int)blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
   }
-  const int m0 = tm * C::TILE, n0 = tn * C::TILE;
+  const int m0 = tm * C::TILE_M, n0 = tn * C::TILE_N;
 
-  FastLoader<C, P_KS> lp;
-  FastLoader<C, Q_KS> lq;
+  FastLoader<C, P_KS, C::TILE_M> lp;
+  FastLoader<C, Q_KS, C::TILE_N> lq;
   lp.init(p.P + batch * p.p_bs, p.ldp, m0, p.M, wave, lane);
   lq.init(p.Q + batch * p.q_bs, p.ldq, n0, p.N, wave, lane);
 
@@ -297,7 +305,7 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
 
   const int nk = p.K / C::BK;
   constexpr int NQ = C::BK / 16 / C::KSPLIT;  // k-steps of one tile that this wavefront multiplies
-  constexpr int LOADS_PER_TILE = 2 * C::LPT;  // per thread, both operands
+  constexpr int LOADS_PER_TILE = C::LPT_P + C::LPT_Q;  // per thread, both operands
   static_assert(NQ % 2 == 0, "fragment buffer parity assumes an even number of k-steps per tile");
   static_assert((NS - 2) * LOADS_PER_TILE < 64, "vmcnt is a 6-bit counter");
 
@@ -312,10 +320,11 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   bf16x8_t fp[2][FM], fq[2][FN];
   auto fetch = [&](const char* st, int q, int buf) {
 #pragma unroll
-    for (int i = 0; i < FM; ++i) fp[buf][i] = fast_frag<C, P_KS>(st, wm * C::TM + i * 32, q * C::KSPLIT + kgroup, lane);
+    for (int i = 0; i < FM; ++i)
+      fp[buf][i] = fast_frag<C, P_KS, C::TILE_M>(st, wm * C::TM + i * 32, q * C::KSPLIT + kgroup, lane);
 #pragma unroll
     for (int j = 0; j < FN; ++j)
-      fq[buf][j] = fast_frag<C, Q_KS>(st + TILE_BYTES, wn * C::TN + j * 32, q * C::KSPLIT + kgroup, lane);
+      fq[buf][j] = fast_frag<C, Q_KS, C::TILE_N>(st + P_BYTES, wn * C::TN + j * 32, q * C::KSPLIT + kgroup, lane);
   };
   auto mma = [&](int buf) {
 #ifdef MI_SETPRIO
@@ -332,7 +341,7 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   };
   auto issue = [&](char* slot) {
     lp.issue(slot, wave);
-    lq.issue(slot + TILE_BYTES, wave);
+    lq.issue(slot + P_BYTES, wave);
   };
   auto k_tile = [&](int kt, char* cur, char* nxt, char* refill) {
     const bool refilled = kt + NS - 1 < nk;

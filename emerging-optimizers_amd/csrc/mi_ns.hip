@@ -94,6 +94,7 @@ static int launch_one(const GemmParams& p, int64_t batch, hipStream_t stream) {
   if (tiles <= 0 || batch <= 0) return MI_OK;
   if (batch > 65535) return fail(MI_ERR_UNSUPPORTED_SHAPE, "batch %lld exceeds the grid limit 65535", (long long)batch);
   g_last_tiles = (int)tiles;
+  if (q.slot_stride == 0) q.slot_stride = (int)tiles;
   dim3 grid((unsigned)tiles, (unsigned)batch, 1), block(WGM * WGN * 64, 1, 1);
   hipLaunchKernelGGL(kern, grid, block, LDS_BYTES, stream, q);
   hipError_t e = hipGetLastError();
@@ -104,14 +105,15 @@ static int launch_one(const GemmParams& p, int64_t batch, hipStream_t stream) {
 template <class C, bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
 static int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream) {
   GemmParams q = p;
-  q.tiles_m = (p.M + C::TILE - 1) / C::TILE;
-  q.tiles_n = (p.N + C::TILE - 1) / C::TILE;
+  q.tiles_m = (p.M + C::TILE_M - 1) / C::TILE_M;
+  q.tiles_n = (p.N + C::TILE_N - 1) / C::TILE_N;
   int64_t tiles = (MODE == MODE_SYRK) ? (int64_t)q.tiles_m * (q.tiles_m + 1) / 2 : (int64_t)q.tiles_m * q.tiles_n;
   if (MODE == MODE_SYRK) tiles = (tiles + 7) / 8 * 8;  // XCD-chunked enumeration: grid padded to a multiple of 8
   if (batch > 65535) return fail(MI_ERR_UNSUPPORTED_SHAPE, "batch %lld exceeds the grid limit 65535", (long long)batch);
   g_last_tiles = (int)tiles;
+  if (q.slot_stride == 0) q.slot_stride = (int)tiles;
   dim3 grid((unsigned)tiles, (unsigned)batch, 1), block(C::NT, 1, 1);
-  const bool edge = (p.M % C::TILE) != 0 || (p.N % C::TILE) != 0;
+  const bool edge = (p.M % C::TILE_M) != 0 || (p.N % C::TILE_N) != 0;
   if (edge)
     hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, true>), grid, block, 0, stream, q);
   else
@@ -184,6 +186,8 @@ struct ShiftArgs {
     p.nslots_in = nslots_in;
     p.shift_io = shift_io;
     p.slots_out = slots_out;
+    p.slot_stride = 0;  // filled in by the launcher
+    p.slot_base = 0;
   }
 };
 
@@ -271,6 +275,36 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
     p.q_bs = x_bs;
     p.M = (int)m;
     p.N = (int)n;
+    // Tile-count quantisation: T full 256 x 256 tiles over C compute units leave a last round that is at
+    // most half full when 0 < T mod C <= C/2.  If that remainder is a whole number of tile columns, those
+    // columns are computed as 256 x 128 tiles instead (twice as many workgroups, one short round).
+#ifndef MI_NO_GEMM_SPLIT
+    if (batch == 1 && m % 256 == 0 && n % 256 == 0 && m >= 1024 && n >= 1024 && m % 64 == 0) {
+      const int64_t tm = m / 256, tn = n / 256, cus = num_cus();
+      const int64_t rem = (tm * tn) % cus;
+      if (rem > 0 && rem * 2 <= cus && rem % tm == 0 && tn > rem / tm) {
+        const int64_t tail_cols = (rem / tm) * 256, main_cols = n - tail_cols;
+        const int tiles_main = (int)(tm * (main_cols / 256)), tiles_tail = (int)(tm * (tail_cols / 128));
+        GemmParams pm = p, pt = p;
+        pm.N = (int)main_cols;
+        pm.slot_stride = pt.slot_stride = tiles_main + tiles_tail;
+        pm.slot_base = 0;
+        pt.slot_base = tiles_main;
+        pt.N = (int)tail_cols;
+        pt.Q = p.Q + main_cols;  // K-strided operand: column offset
+        if (pt.Cin) pt.Cin = p.Cin + main_cols;
+        pt.Out = out_fp32 ? static_cast<void*>(static_cast<float*>(p.Out) + main_cols)
+                          : static_cast<void*>(static_cast<uint16_t*>(p.Out) + main_cols);
+        int rc = out_fp32 ? launch_fast<CfgBig, false, true, MODE_GEMM, true>(pm, batch, stream)
+                          : launch_fast<CfgBig, false, true, MODE_GEMM, false>(pm, batch, stream);
+        if (rc != MI_OK) return rc;
+        rc = out_fp32 ? launch_fast<CfgHalfN, false, true, MODE_GEMM, true>(pt, batch, stream)
+                      : launch_fast<CfgHalfN, false, true, MODE_GEMM, false>(pt, batch, stream);
+        g_last_tiles = tiles_main + tiles_tail;
+        return rc;
+      }
+    }
+#endif
     return out_fp32 ? launch_class<false, true, MODE_GEMM, true>(tc, p, batch, stream)
                     : launch_class<false, true, MODE_GEMM, false>(tc, p, batch, stream);
   }
