@@ -251,23 +251,26 @@ __device__ __forceinline__ float resolve_shift(const GemmParams& p, int64_t batc
   return s;
 }
 
-// Epilogue shared by both kernels.  A lane owns output row m = m_base + 32 i + (lane & 31) and, for each
-// (j, g), the four columns n .. n+3 with n = n_base + 32 j + 8 g + 4 (lane >> 5).
-template <int MODE, bool OUT_F32, bool GUARD, int FM, int FN, int NT>
-__device__ __forceinline__ void tile_epilogue(const GemmParams& p, f32x16_t (&acc)[FM][FN], int m_base, int n_base,
+// Epilogue shared by both kernels.  MI names the MFMA tile the accumulators come from:
+//   MI = 32 (f32x16): a lane owns output row m = m_base + 32 i + (lane & 31) and, for each (j, g), the four
+//                     columns n .. n+3 with n = n_base + 32 j + 8 g + 4 (lane >> 5)
+//   MI = 16 (f32x4):  row m = m_base + 16 i + (lane & 15), columns n .. n+3 with n = n_base + 16 j + 4 (lane >> 4)
+template <int MODE, bool OUT_F32, bool GUARD, int FM, int FN, int NT, int MI = 32, class ACC = f32x16_t>
+__device__ __forceinline__ void tile_epilogue(const GemmParams& p, ACC (&acc)[FM][FN], int m_base, int n_base,
                                               int lane, int64_t batch, bool diag, float alpha, float beta, float shift,
                                               float* red) {
-  const int frow = lane & 31, fk = lane >> 5;
+  constexpr int G = MI == 32 ? 4 : 1;
+  const int frow = lane & (MI - 1), fk = lane / MI;
   const uint16_t* __restrict__ Cb = p.Cin ? p.Cin + batch * p.c_bs : nullptr;
   float ssq = 0.0f;
 #pragma unroll
   for (int i = 0; i < FM; ++i) {
-    const int m = m_base + i * 32 + frow;
+    const int m = m_base + i * MI + frow;
 #pragma unroll
     for (int j = 0; j < FN; ++j) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int n = n_base + j * 32 + 8 * g + 4 * fk;
+      for (int g = 0; g < G; ++g) {
+        const int n = n_base + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
         if (GUARD && (m >= p.M || n >= p.N)) continue;
         f32x4_t v;
 #pragma unroll

@@ -12,22 +12,41 @@
 //     (c + 4 k) mod 32; fragments are fetched with the LDS transpose read ds_read_b64_tr_b16, which
 //     returns to lane i of a 16-lane group the four k-values of column i from four consecutive k-rows.
 #pragma once
+#include <type_traits>
+#include <utility>
+
 #include "gemm_engine.hpp"
 
 namespace mi {
 
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 
+// Compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{}).  Used where a
+// body must be unrolled whatever its size (register arrays indexed by the loop variable must never become
+// runtime-indexed, i.e. scratch memory).
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
 // Compile-time shape of one fast-kernel variant.
-template <int TILE_M_, int WGM_, int WGN_, int BK_, int NS_, int KSPLIT_ = 1, int TILE_N_ = TILE_M_>
+template <int TILE_M_, int WGM_, int WGN_, int BK_, int NS_, int KSPLIT_ = 1, int TILE_N_ = TILE_M_, int MI_ = 32>
 struct FastCfg {
+  // MFMA shape: MI = 32 -> v_mfma_f32_32x32x16_bf16, MI = 16 -> v_mfma_f32_16x16x32_bf16 (KI = k per MFMA).
+  // Both do 16 K FLOP per pass; on random operands the 16 x 16 shape draws less power per FLOP (it moves a
+  // quarter of the accumulator registers per instruction), which is what bounds the clock on this part.
+  static constexpr int MI = MI_, KI = MI_ == 32 ? 16 : 32;
   static constexpr int TILE_M = TILE_M_, TILE_N = TILE_N_;  // workgroup tile: rows of P x rows of Q
   static constexpr int TILE = TILE_M_;                      // (SYRK uses square tiles)
   // KSPLIT groups of WGM x WGN wavefronts each cover the whole tile and take alternate 16-wide k-steps; their
   // accumulators are added through LDS after the K loop (two wavefronts per SIMD with large wave tiles).
   static constexpr int KSPLIT = KSPLIT_;
   static constexpr int WGM = WGM_, WGN = WGN_, NWG = WGM * WGN, NW = NWG * KSPLIT, NT = NW * 64;
-  static constexpr int TM = TILE_M / WGM, TN = TILE_N / WGN, FM = TM / 32, FN = TN / 32;
+  static constexpr int TM = TILE_M / WGM, TN = TILE_N / WGN, FM = TM / MI, FN = TN / MI;
   static constexpr int BK = BK_;                       // k extent of one ring slot
   static constexpr int NS = NS_;                       // ring slots
   static constexpr int P_BYTES = TILE_M * BK * 2, Q_BYTES = TILE_N * BK * 2;  // operand tiles
@@ -38,17 +57,26 @@ struct FastCfg {
   static constexpr int ROWS_PER_KB = 1024 / (BK * 2);  // K-contiguous rows covered by one 1 KB load
   static_assert(BK == 32 || BK == 64, "ring slot depth");
   static_assert(KSPLIT == 1 || KSPLIT == 2, "at most two K groups");
-  static_assert((BK / 16) % (2 * KSPLIT) == 0 || KSPLIT == 1, "each K group needs an even number of k-steps per tile");
-  static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of the 32 x 32 MFMA");
+  static_assert(MI == 32 || MI == 16, "MFMA shape");
+  static_assert((BK / KI) % (2 * KSPLIT) == 0, "each K group needs an even number of k-steps per tile");
+  static_assert(TM % MI == 0 && TN % MI == 0, "wave tile must be a multiple of the MFMA tile");
   static_assert(P_BYTES % (1024 * NW) == 0 && Q_BYTES % (1024 * NW) == 0,
                 "tiles must split evenly over the wavefronts' 1 KB loads");
   static_assert(NS * SLOT_BYTES <= 160 * 1024 - 256, "ring exceeds the 160 KB LDS");
 };
+#ifndef MI_SHAPE
+#define MI_SHAPE 16
+#endif
+#if MI_SHAPE == 32
 // MFMA-bound default: 256 x 256 tile, 8 wavefronts (2 per SIMD) of 128 x 64, two 64 KB slots.
 #ifndef MI_BIG_WGN
 #define MI_BIG_WGN 4
 #endif
-using CfgBig = FastCfg<256, 2, MI_BIG_WGN, 64, 2>;
+#ifndef MI_BIG_BK
+#define MI_BIG_BK 64
+#define MI_BIG_NS 2
+#endif
+using CfgBig = FastCfg<256, 2, MI_BIG_WGN, MI_BIG_BK, MI_BIG_NS>;
 // Half-width tile for the last partial round of a GEMM: 256 x 128, wavefronts of 128 x 32.
 using CfgHalfN = FastCfg<256, 2, 4, 64, 2, 1, 128>;
 // SYRK on ~4096-row Gram matrices: 192 x 192 tiles give 22 * 23 / 2 = 253 lower-triangle tiles, one per
@@ -58,16 +86,37 @@ using CfgHalfN = FastCfg<256, 2, 4, 64, 2, 1, 128>;
 #define MI_SYRK192_KSPLIT 2
 #endif
 using CfgSyrk192 = FastCfg<192, 2, 2, 64, 3, MI_SYRK192_KSPLIT>;
+#else
+// 16 x 16 x 32 MFMA variants: one wavefront per SIMD (4 per workgroup), accumulators in 256 / 128 / 144 registers.
+using CfgBig = FastCfg<256, 2, 2, 64, 2, 1, 256, 16>;     // wavefronts of 128 x 128
+#ifndef MI_HALFN_NS
+#define MI_HALFN_NS 3
+#endif
+using CfgHalfN = FastCfg<256, 2, 2, 64, MI_HALFN_NS, 1, 128, 16>;   // wavefronts of 128 x 64
+using CfgSyrk192 = FastCfg<192, 2, 2, 64, 3, 1, 192, 16>;  // wavefronts of 96 x 96
+#endif
+
+template <int MI> struct AccVec { typedef f32x16_t type; };
+template <> struct AccVec<16> { typedef f32x4_t type; };
+
+// Rotation (in 16-byte chunks) of k-row k of a K-strided LDS tile.  It is chosen per MFMA shape so that the
+// k-rows which one pass of the transpose read touches (32 lanes) fall on disjoint banks:
+//   MI = 32: a pass reads 4 k-rows x 64 B  -> 64 B per k
+//   MI = 16: a pass reads 4 k-rows x 32 B at k and at k + 8 -> 32 B per k inside an 8-row group, 128 B per group
+template <int MI>
+__device__ __forceinline__ int ks_rot(int k) {
+  return MI == 32 ? 4 * k : 2 * (k & 7) + 8 * (k >> 3);
+}
 
 // Direct-to-LDS load: every lane fetches 16 bytes from its own global address; the wavefront's 1 KB lands
-// at LDS byte address `lds_wave_base` + 16 * lane (the base travels in M0).  Written as inline assembly so
+// at LDS byte address `lds_addr` + 16 * lane (`lds_addr` is wave-uniform and travels in M0).  Written as inline assembly so
 // that completion is tracked only by the explicit s_waitcnt vmcnt(..) in the kernel: the compiler's own
 // bookkeeping would make every later LDS read wait for all outstanding loads, i.e. no prefetching.
-__device__ __forceinline__ void dma16(const uint16_t* g, char* lds_wave_base) {
-  const uint32_t lds_addr = __builtin_amdgcn_readfirstlane(
-      (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_wave_base);  // wave-uniform by construction
+// (M0 is a reserved register: the compiler never keeps a value in it across statements, so it is not
+// listed as clobbered.)
+__device__ __forceinline__ void dma16(const uint16_t* g, uint32_t lds_addr) {
 #ifndef MI_ABLATE_LOADS
-  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(g) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(g) : "memory");
 #endif
 }
 
@@ -78,66 +127,127 @@ __device__ __forceinline__ int kc_slot(int row, int c) {
   return BK == 64 ? (c ^ ((row >> 1) & 7)) : (c ^ ((row >> 2) & 3));
 }
 
-// Per-thread global pointers of the direct-to-LDS loads of one operand tile.  Rows beyond `rows_valid` are
-// redirected to the last valid row: they only feed output rows that the epilogue never stores.
-template <class C, bool KS, int ROWS>
+// Same load with the address split into a wave-uniform 64-bit base (SGPR pair) and a per-lane 32-bit byte
+// offset: the blocks of one tile differ only in the base, so a handful of offset registers serve all loads
+// of an operand and the per-load address arithmetic runs on the scalar unit.
+__device__ __forceinline__ void dma16_sv(uint64_t sbase, uint32_t voff, uint32_t lds_addr) {
+#ifndef MI_ABLATE_LOADS
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
+#endif
+}
+
+// Direct-to-LDS loads of one operand tile (ROWS rows of the operand x BK along k).  The tile is cut into
+// 1 KB blocks, LPT per wavefront; block b = wave * LPT + i lands at tile + 1024 * b.
+//   CLAMP = false: the tile lies wholly inside the operand.  Block b starts at a wave-uniform address and the
+//     lanes' offsets inside a block repeat with a short period in b (the swizzle phase), so the loader keeps
+//     one scalar base plus NV lane-offset registers.
+//   CLAMP = true: rows beyond `rows_valid` are redirected to the last valid row (they only feed output rows
+//     that the epilogue never stores); every load keeps its own per-lane pointer.
+template <class C, bool KS, int ROWS, bool CLAMP>
 struct FastLoader {
   static constexpr int LPT = ROWS * C::BK * 2 / 1024 / C::NW;
   static constexpr int KS_CHUNKS = ROWS / 8;          // 16-byte chunks per k-row of the K-strided layout
   static constexpr int KS_ROWS_PER_KB = 512 / ROWS;   // k-rows covered by one 1 KB load
-  const uint16_t* gp[LPT];
-  int64_t step;  // elements to advance per K tile
+  // period of the swizzle phase in the block index
+  static constexpr int PERIOD = KS ? (C::MI == 32 ? (KS_CHUNKS / (4 * KS_ROWS_PER_KB) > 0 ? KS_CHUNKS / (4 * KS_ROWS_PER_KB) : 1)
+                                                  : (KS_CHUNKS / KS_ROWS_PER_KB > 0 ? KS_CHUNKS / KS_ROWS_PER_KB : 1))
+                                   : (C::BK == 64 ? 2 : 1);
+  static constexpr bool PERIODIC = LPT % PERIOD == 0;  // then the phase of load i is i % PERIOD for every wavefront
+  static constexpr int NV = CLAMP ? 1 : (PERIODIC ? (PERIOD < LPT ? PERIOD : LPT) : LPT);
+  static_assert(!KS || ROWS == 256 || ROWS == 128, "K-strided LDS layout is laid out for 128/256-wide tiles");
 
-  __device__ __forceinline__ void init(const uint16_t* base, int64_t ld, int row0, int rows_valid, int wave, int lane) {
-#pragma unroll
-    for (int i = 0; i < LPT; ++i) {
-      const int b = wave * LPT + i;  // 1 KB block index inside the tile
-      if (!KS) {
-        const int row = C::ROWS_PER_KB * b + lane / C::CPR;
-        const int c = kc_slot<C::BK>(row, lane % C::CPR);  // the swizzle is an involution: slot -> chunk
-        int gr = row0 + row;
-        gr = gr < rows_valid ? gr : rows_valid - 1;
-        gp[i] = base + (int64_t)gr * ld + c * 8;
-      } else {
-        static_assert(!KS || ROWS == 256 || ROWS == 128, "K-strided LDS layout is laid out for 128/256-wide tiles");
-        const int k = KS_ROWS_PER_KB * b + lane / KS_CHUNKS;
-        const int c = ((lane % KS_CHUNKS) - 4 * k) & (KS_CHUNKS - 1);
-        gp[i] = base + (int64_t)k * ld + row0 + c * 8;
-      }
+  const uint16_t* gp[CLAMP ? LPT : 1];  // CLAMP: per-load pointers
+  uint32_t voff[NV];                    // !CLAMP: per-lane byte offsets inside a block
+  uint64_t base;                        // !CLAMP: byte address of this wavefront's first block (uniform)
+  int64_t block_step;                   // !CLAMP: bytes between consecutive blocks (uniform)
+  int64_t step;                         // advance per K tile: elements (CLAMP) or bytes (!CLAMP)
+
+  // lane's element offset inside block b, relative to the block's first element
+  static __device__ __forceinline__ int64_t lane_part(int b, int64_t ld, int lane) {
+    if (!KS) {
+      const int lr = lane / C::CPR;
+      const int c = kc_slot<C::BK>(C::ROWS_PER_KB * b + lr, lane % C::CPR);  // the swizzle is an involution
+      return (int64_t)lr * ld + c * 8;
+    } else {
+      const int kr = lane / KS_CHUNKS;
+      const int c = ((lane % KS_CHUNKS) - ks_rot<C::MI>(KS_ROWS_PER_KB * b + kr)) & (KS_CHUNKS - 1);
+      return (int64_t)kr * ld + c * 8;
     }
-    step = KS ? (int64_t)C::BK * ld : C::BK;
   }
-  __device__ __forceinline__ void issue(char* tile, int wave) {
+
+  __device__ __forceinline__ void init(const uint16_t* opbase, int64_t ld, int row0, int rows_valid, int wave, int lane) {
+    if constexpr (CLAMP) {
 #pragma unroll
-    for (int i = 0; i < LPT; ++i) {
-      dma16(gp[i], tile + (wave * LPT + i) * 1024);
-      gp[i] += step;
+      for (int i = 0; i < LPT; ++i) {
+        const int b = wave * LPT + i;  // 1 KB block index inside the tile
+        if (!KS) {
+          const int row = C::ROWS_PER_KB * b + lane / C::CPR;
+          const int c = kc_slot<C::BK>(row, lane % C::CPR);
+          int gr = row0 + row;
+          gr = gr < rows_valid ? gr : rows_valid - 1;
+          gp[i] = opbase + (int64_t)gr * ld + c * 8;
+        } else {
+          const int k = KS_ROWS_PER_KB * b + lane / KS_CHUNKS;
+          const int c = ((lane % KS_CHUNKS) - ks_rot<C::MI>(k)) & (KS_CHUNKS - 1);
+          gp[i] = opbase + (int64_t)k * ld + row0 + c * 8;
+        }
+      }
+      step = KS ? (int64_t)C::BK * ld : C::BK;
+    } else {
+      const int b0 = wave * LPT;
+#pragma unroll
+      for (int v = 0; v < NV; ++v) voff[v] = (uint32_t)(2 * lane_part(PERIODIC ? v : b0 + v, ld, lane));
+      const int64_t first = KS ? (int64_t)(KS_ROWS_PER_KB * b0) * ld + row0 : (int64_t)(row0 + C::ROWS_PER_KB * b0) * ld;
+      base = (uint64_t)(uintptr_t)(opbase + first);
+      block_step = 2 * (int64_t)(KS ? KS_ROWS_PER_KB : C::ROWS_PER_KB) * ld;
+      step = 2 * (KS ? (int64_t)C::BK * ld : (int64_t)C::BK);
+    }
+  }
+  // Issues load i (0 .. LPT-1) of the current K tile; `lds_tile` is the LDS byte address of the operand tile
+  // in the target ring slot.  advance() moves on to the next K tile once all LPT loads are out.
+  __device__ __forceinline__ void issue_one(uint32_t lds_tile, int wave, int i) {
+    if constexpr (CLAMP)
+      dma16(gp[i], lds_tile + (wave * LPT + i) * 1024);
+    else
+      dma16_sv(base + (uint64_t)(i * block_step), voff[PERIODIC ? i % NV : i], lds_tile + (wave * LPT + i) * 1024);
+  }
+  __device__ __forceinline__ void advance() {
+    if constexpr (CLAMP) {
+#pragma unroll
+      for (int i = 0; i < LPT; ++i) gp[i] += step;
+    } else {
+      base += step;
     }
   }
 };
 
-// MFMA fragment (8 bf16 along k) for 32 consecutive rows starting at `row_base`, k-step q (16 k each).
+// MFMA fragment (8 bf16 along k per lane) for MI consecutive rows starting at `row_base`, k-step q (KI k each).
+//   MI = 32: lane l -> row l % 32, k = 16 q + 8 (l / 32) .. +7
+//   MI = 16: lane l -> row l % 16, k = 32 q + 8 (l / 16) .. +7
+// K-strided tiles are read with the LDS transpose read: its 16 lanes fetch 4 k-rows x 16 rows (8 bytes per
+// lane: 4 consecutive rows at one k) and every lane receives the 4 k-values of its own row.
 template <class C, bool KS, int ROWS>
 __device__ __forceinline__ bf16x8_t fast_frag(const char* tile, int row_base, int q, int lane) {
-  constexpr int KS_CHUNKS = ROWS / 8, KS_ROW_BYTES = ROWS * 2;
+  constexpr int KS_CHUNKS = ROWS / 8, KS_ROW_BYTES = ROWS * 2, MI = C::MI;
+  const int kgrp = MI == 32 ? (lane >> 5) : (lane >> 4);  // which 8-wide k group of the k-step this lane feeds
   if (!KS) {
-    const int row = row_base + (lane & 31);
-    const int c = kc_slot<C::BK>(row, 2 * q + (lane >> 5));
+    const int row = row_base + (lane & (MI - 1));
+    const int c = kc_slot<C::BK>(row, (C::KI / 8) * q + kgrp);
     return *reinterpret_cast<const bf16x8_t*>(tile + row * (C::BK * 2) + c * 16);
   } else {
     const int i16 = lane & 15;
-    const int col = row_base + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
-    const int kb = 16 * q + 8 * (lane >> 5) + (i16 >> 2);
+    const int col = row_base + (MI == 32 ? 16 * ((lane >> 4) & 1) : 0) + 4 * (i16 & 3);
+    const int kb = C::KI * q + 8 * kgrp + (i16 >> 2);
     s16x4_t lo, hi;
     {
       const int k = kb;
-      const int slot = ((col >> 3) + 4 * k) & (KS_CHUNKS - 1);
+      const int slot = ((col >> 3) + ks_rot<MI>(k)) & (KS_CHUNKS - 1);
       lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
           (s16x4_t __attribute__((address_space(3)))*)(tile + k * KS_ROW_BYTES + slot * 16 + (col & 7) * 2));
     }
     {
       const int k = kb + 4;
-      const int slot = ((col >> 3) + 4 * k) & (KS_CHUNKS - 1);
+      const int slot = ((col >> 3) + ks_rot<MI>(k)) & (KS_CHUNKS - 1);
       hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
           (s16x4_t __attribute__((address_space(3)))*)(tile + k * KS_ROW_BYTES + slot * 16 + (col & 7) * 2));
     }
@@ -146,6 +256,37 @@ __device__ __forceinline__ bf16x8_t fast_frag(const char* tile, int row_base, in
     return __builtin_bit_cast(bf16x8_t, both);
   }
 }
+
+// K-strided fragment of the 16 x 16 x 32 shape from two per-lane constants (see ks16_consts): the LDS address of
+// every transpose read is ((S + c) & rowmask | R) + constant, i.e. two VALU operations next to the read instead
+// of one address register per (fragment, k-half, k-step, ring slot) kept alive across the whole K loop.
+template <int ROWS>
+__device__ __forceinline__ void ks16_consts(int lane, int wave_row_base, uint32_t& S, uint32_t& R) {
+  const int g = lane >> 4, i16 = lane & 15, kk = i16 >> 2, cq = i16 & 3;
+  S = (uint32_t)((wave_row_base / 8 + (cq >> 1) + 2 * kk + 8 * g) * 16 + (cq & 1) * 8);
+  R = (uint32_t)((8 * g + kk) * (ROWS * 2));
+}
+template <int ROWS>
+__device__ __forceinline__ bf16x8_t fast_frag16_ks(uint32_t tile_lds, uint32_t S, uint32_t R, int r, int q) {
+  constexpr int ROWB = ROWS * 2;  // bytes per k-row = 16 * chunks per k-row (a power of two)
+  static_assert((ROWB & (ROWB - 1)) == 0, "row mask");
+  typedef s16x4_t __attribute__((address_space(3))) * lds_ptr;
+  const uint32_t a0 = (((S + (uint32_t)(2 * r) * 16u) & (ROWB - 1)) | R) + tile_lds + (uint32_t)(32 * q) * ROWB;
+  const uint32_t a1 = (((S + (uint32_t)(2 * r + 8) * 16u) & (ROWB - 1)) | R) + tile_lds + (uint32_t)(32 * q + 4) * ROWB;
+  const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(uintptr_t)a0);
+  const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(uintptr_t)a1);
+  typedef short s16x8_t __attribute__((ext_vector_type(8)));
+  return __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+// acc += A B with the accumulator tied in place (AGPRs).  With the builtin the register allocator is free to
+// give the result other registers than the addend and then restores the loop-carried layout with copies.
+// The compiler does not see an MFMA here: code that reads the accumulators with VALU instructions must be
+// separated from the last of these by mfma_drain().
+__device__ __forceinline__ void mfma16_inplace(f32x4_t& c, const bf16x8_t& a, const bf16x8_t& b) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_drain() { asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory"); }
 
 // Workgroup id -> GEMM tile.  Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its
 // own L2, so id % 8 names the XCD and id / 8 the position in that XCD's queue.  Each XCD gets a contiguous
@@ -175,32 +316,33 @@ __device__ __forceinline__ void gemm_tile_of(int pid, int tiles_m, int tiles_n, 
 // 4-column groups, so direct global accesses touch 32 rows per instruction.  Here every wavefront parks one
 // 32-row block of its accumulators in its own LDS region (float32, rows padded by 16 bytes against bank
 // conflicts), then re-reads it so that 8 consecutive lanes cover 64 consecutive columns of one row: the
-// Cin loads and the stores become 16-byte-per-lane, 128-byte-per-row accesses.  No workgroup barrier is
+// Cin loads and the stores become 16-byte-per-lane, 128-byte-per-row accesses.  (MI = rows of one MFMA tile,
+// G = 4-column groups a lane holds per MFMA tile: 4 for the 32 x 32 shape, 1 for 16 x 16.)  No workgroup barrier is
 // needed between the passes: a wavefront only touches its own region and LDS operations of one wavefront
 // complete in order.
 template <class C, bool OUT_F32, bool GUARD>
-__device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16_t (&acc)[C::FM][C::FN], char* lds, int wave,
+__device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, typename AccVec<C::MI>::type (&acc)[C::FM][C::FN], char* lds, int wave,
                                                   int lane, int m_base, int n_base, int64_t batch, float alpha,
                                                   float beta, float* red) {
-  constexpr int TN = C::TN, ROWB = TN * 4 + 16;
+  constexpr int TN = C::TN, ROWB = TN * 4 + 16, MI = C::MI, G = MI == 32 ? 4 : 1;
   constexpr int LPR = TN / 8;    // lanes per output row (8 columns each)
   constexpr int RPI = 64 / LPR;  // rows per read iteration
-  static_assert(32 % RPI == 0 && 64 % LPR == 0, "wave tile width must be 32, 64 or 128");
-  static_assert(C::NW * 32 * ROWB <= C::NS * C::SLOT_BYTES, "epilogue staging exceeds the ring");
-  char* reg = lds + wave * (32 * ROWB);
-  const int frow = lane & 31, fk = lane >> 5;
+  static_assert(MI % RPI == 0 && 64 % LPR == 0, "wave tile width must be 32, 64 or 128");
+  static_assert(C::NW * MI * ROWB <= C::NS * C::SLOT_BYTES, "epilogue staging exceeds the ring");
+  char* reg = lds + wave * (MI * ROWB);
+  const int frow = lane & (MI - 1), fk = lane / MI;
   const int rr = lane / LPR, cc = (lane % LPR) * 8;
   const uint16_t* __restrict__ Cb = p.Cin ? p.Cin + batch * p.c_bs : nullptr;
   const bool use_c = beta != 0.0f && Cb != nullptr;
-  constexpr int NIT = 32 / RPI;
+  constexpr int NIT = MI / RPI;
   // All Cin pieces of this lane are requested up front (the fragment registers of the main loop are dead by
   // now), so the global-load latency is paid once instead of once per piece.
-  constexpr bool PREFETCH_ALL = C::FM * NIT * 4 <= 64;  // else one 32-row block at a time (register budget)
+  constexpr bool PREFETCH_ALL = C::FM * NIT * 4 <= 64;  // else one MI-row block at a time (register budget)
   uint4 cin[C::FM][NIT];
   auto load_cin = [&](int i) {
 #pragma unroll
     for (int t = 0; t < NIT; ++t) {
-      const int m = m_base + i * 32 + t * RPI + rr, n = n_base + cc;
+      const int m = m_base + i * MI + t * RPI + rr, n = n_base + cc;
       cin[i][t] = make_uint4(0u, 0u, 0u, 0u);
       if (use_c && (!GUARD || (m < p.M && n < p.N))) cin[i][t] = *reinterpret_cast<const uint4*>(Cb + (int64_t)m * p.ldc + n);
     }
@@ -216,14 +358,14 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x16_t 
 #pragma unroll
     for (int j = 0; j < C::FN; ++j)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
+      for (int g = 0; g < G; ++g) {
         f32x4_t v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-        *reinterpret_cast<f32x4_t*>(reg + frow * ROWB + (j * 32 + 8 * g + 4 * fk) * 4) = v;
+        *reinterpret_cast<f32x4_t*>(reg + frow * ROWB + (j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk) * 4) = v;
       }
 #pragma unroll
     for (int t = 0; t < NIT; ++t) {
       const int row = t * RPI + rr;
-      const int m = m_base + i * 32 + row, n = n_base + cc;
+      const int m = m_base + i * MI + row, n = n_base + cc;
       f32x4_t lo = *reinterpret_cast<const f32x4_t*>(reg + row * ROWB + cc * 4);
       f32x4_t hi = *reinterpret_cast<const f32x4_t*>(reg + row * ROWB + cc * 4 + 16);
       if (GUARD && (m >= p.M || n >= p.N)) continue;
@@ -290,86 +432,155 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   }
   const int m0 = tm * C::TILE_M, n0 = tn * C::TILE_N;
 
-  FastLoader<C, P_KS, C::TILE_M> lp;
-  FastLoader<C, Q_KS, C::TILE_N> lq;
+  FastLoader<C, P_KS, C::TILE_M, EDGE> lp;
+  FastLoader<C, Q_KS, C::TILE_N, EDGE> lq;
   lp.init(p.P + batch * p.p_bs, p.ldp, m0, p.M, wave, lane);
   lq.init(p.Q + batch * p.q_bs, p.ldq, n0, p.N, wave, lane);
 
-  f32x16_t acc[FM][FN];
+  constexpr int MI = C::MI, ACC_N = MI == 32 ? 16 : 4;
+  typename AccVec<MI>::type acc[FM][FN];
 #pragma unroll
   for (int i = 0; i < FM; ++i)
 #pragma unroll
     for (int j = 0; j < FN; ++j)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+      for (int e = 0; e < ACC_N; ++e) acc[i][j][e] = 0.0f;
 
   const int nk = p.K / C::BK;
-  constexpr int NQ = C::BK / 16 / C::KSPLIT;  // k-steps of one tile that this wavefront multiplies
+  constexpr int NQ = C::BK / C::KI / C::KSPLIT;  // k-steps of one tile that this wavefront multiplies
   constexpr int LOADS_PER_TILE = C::LPT_P + C::LPT_Q;  // per thread, both operands
   static_assert(NQ % 2 == 0, "fragment buffer parity assumes an even number of k-steps per tile");
-  static_assert((NS - 2) * LOADS_PER_TILE < 64, "vmcnt is a 6-bit counter");
+  static_assert((NS - 1) * LOADS_PER_TILE < 64, "vmcnt is a 6-bit counter");
 
-  // Pipeline.  Ring slot kt % NS holds K tile kt.  While tile kt is multiplied, tiles kt+1 .. kt+NS-1 are in
-  // flight; the slot refilled at the top of tile kt is the one tile kt-1 occupied, which every wavefront left
-  // before the previous barrier.  Fragment registers are double buffered (the LDS reads of k-step q+1 run
-  // under the MFMAs of k-step q), and the barrier that publishes tile kt+1 sits before the last k-step of
-  // tile kt so that its skew and the first fragment reads of tile kt+1 are covered by that k-step's MFMAs.
+  // Pipeline.  Ring slot kt % NS holds K tile kt; while tile kt is multiplied, tiles kt+1 .. kt+NS-1 are in
+  // flight.  Per tile: k-steps 0 .. NQ-2 (each fetches the fragments of the next k-step into the other
+  // register buffer), then wait for this wavefront's loads of tile kt+1 and its own LDS reads, one barrier
+  // (tile kt+1 is published; nobody reads slot kt % NS any more), then the last k-step, which also fetches
+  // the first fragments of tile kt+1 and starts the loads of tile kt+NS into the slot just vacated.
+  // Every k-step is written as MFMA "slots": one MFMA followed by its share of the LDS reads and of the
+  // direct-to-LDS loads, pinned in that order, so that a wavefront that has the SIMD to itself never stops
+  // issuing MFMAs while it feeds the memory pipes.
+  // The loads of a tile are cut into PARTS equal parts.  With three or more ring slots the parts go out one
+  // per k-step (part 0 right after the barrier that vacates the slot, the rest in the k-steps of the next
+  // tile before its barrier): the CU's single address unit then sees an even stream instead of a burst from
+  // all wavefronts at once, and the tile still has NS-2 whole tile times to land.  With two slots there is no
+  // slack for that and the whole tile goes out in the k-step after the barrier.
 #ifdef MI_TIMING
   long long t_load = 0, t_bar = 0;
 #endif
+  constexpr int UNITS = FM + FN, MMAS = FM * FN;  // fragment reads / MFMAs per k-step
+  constexpr int UPS = (UNITS + MMAS - 1) / MMAS;  // fragment reads per slot
+  constexpr int PARTS = (NS >= 3 && LOADS_PER_TILE % NQ == 0) ? NQ : 1;
+  constexpr int PL = LOADS_PER_TILE / PARTS;      // loads per part
+  constexpr int DPS = (PL + MMAS - 1) / MMAS;     // loads per slot (1 unless a part outnumbers the MFMAs)
   bf16x8_t fp[2][FM], fq[2][FN];
+  uint32_t ks_sp = 0, ks_rp = 0, ks_sq = 0, ks_rq = 0;  // 16 x 16 shape: lane constants of the K-strided reads
+  if constexpr (MI == 16 && P_KS) ks16_consts<C::TILE_M>(lane, wm * C::TM, ks_sp, ks_rp);
+  if constexpr (MI == 16 && Q_KS) ks16_consts<C::TILE_N>(lane, wn * C::TN, ks_sq, ks_rq);
+  auto lds_of = [&](const char* ptr) { return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)ptr; };
+  auto read_unit = [&](const char* st, int q, int buf, int r) {
+#ifdef MI_ABLATE_READS
+    if (q >= 0) return;  // debug build: fragments keep their start-up contents
+#endif
+    if (r < FM) {
+      if constexpr (MI == 16 && P_KS)
+        fp[buf][r] = fast_frag16_ks<C::TILE_M>(lds_of(st), ks_sp, ks_rp, r, q * C::KSPLIT + kgroup);
+      else
+        fp[buf][r] = fast_frag<C, P_KS, C::TILE_M>(st, wm * C::TM + r * MI, q * C::KSPLIT + kgroup, lane);
+    } else {
+      if constexpr (MI == 16 && Q_KS)
+        fq[buf][r - FM] = fast_frag16_ks<C::TILE_N>(lds_of(st + P_BYTES), ks_sq, ks_rq, r - FM, q * C::KSPLIT + kgroup);
+      else
+        fq[buf][r - FM] = fast_frag<C, Q_KS, C::TILE_N>(st + P_BYTES, wn * C::TN + (r - FM) * MI, q * C::KSPLIT + kgroup, lane);
+    }
+  };
   auto fetch = [&](const char* st, int q, int buf) {
 #pragma unroll
-    for (int i = 0; i < FM; ++i)
-      fp[buf][i] = fast_frag<C, P_KS, C::TILE_M>(st, wm * C::TM + i * 32, q * C::KSPLIT + kgroup, lane);
-#pragma unroll
-    for (int j = 0; j < FN; ++j)
-      fq[buf][j] = fast_frag<C, Q_KS, C::TILE_N>(st + P_BYTES, wn * C::TN + j * 32, q * C::KSPLIT + kgroup, lane);
+    for (int r = 0; r < UNITS; ++r) read_unit(st, q, buf, r);
   };
-  auto mma = [&](int buf) {
+  const uint32_t ring_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)&ring[0][0];
+  auto issue_one = [&](int slot, int d) {  // d-th load of this wavefront for a tile: P blocks first, then Q
+    if (d < C::LPT_P)
+      lp.issue_one(ring_lds + slot * C::SLOT_BYTES, wave, d);
+    else
+      lq.issue_one(ring_lds + slot * C::SLOT_BYTES + P_BYTES, wave, d - C::LPT_P);
+  };
+  // parts [p0, p1) of the current tile of the loaders in one go; the loaders move on after the last part
+  auto issue_parts = [&](int slot, int p0, int p1) {
+#pragma unroll
+    for (int d = p0 * PL; d < p1 * PL; ++d) issue_one(slot, d);
+    if (p1 == PARTS) {
+      lp.advance();
+      lq.advance();
+    }
+  };
+  // One k-step on register buffer `buf`.  READ: fetch the fragments of k-step rd_q of tile rd_tile into the
+  // other buffer.  PART >= 0: issue that part of the loaders' current tile into slot ld_slot.
+  auto k_step = [&](auto read_flag, auto part, int buf, const char* rd_tile, int rd_q, int ld_slot) {
+    constexpr bool READ = decltype(read_flag)::value;
+    constexpr int PART = decltype(part)::value;
+    if constexpr (MI == 16 && (P_KS || Q_KS)) {
+      // keep the address arithmetic of the transpose reads next to them (it would otherwise be hoisted out of
+      // the K loop, one register per read)
+      asm volatile("" : "+v"(ks_sp), "+v"(ks_rp), "+v"(ks_sq), "+v"(ks_rq));
+    }
 #ifdef MI_SETPRIO
     __builtin_amdgcn_s_setprio(MI_SETPRIO);
 #endif
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-      for (int j = 0; j < FN; ++j)
+    static_for<MMAS>([&](auto xc) {
+      constexpr int x = decltype(xc)::value, i = x / FN, j = x % FN;
+      if constexpr (MI == 32)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fq[buf][j], fp[buf][i], acc[i][j], 0, 0, 0);
+      else
+        mfma16_inplace(acc[i][j], fq[buf][j], fp[buf][i]);
+      if constexpr (READ) {
+        static_for<UPS>([&](auto uc) {
+          constexpr int u = decltype(uc)::value;
+          if constexpr (x * UPS + u < UNITS) read_unit(rd_tile, rd_q, buf ^ 1, x * UPS + u);
+        });
+      }
+      if constexpr (PART >= 0) {
+        // load e of the part goes into slot e * MMAS / PL when the part has fewer loads than the k-step has
+        // MFMAs (an even spread), else DPS loads per slot
+        static_for<PL>([&](auto ec) {
+          constexpr int e = decltype(ec)::value;
+          if constexpr ((PL <= MMAS ? e * MMAS / PL : e / DPS) == x) issue_one(ld_slot, PART * PL + e);
+        });
+      }
+#ifndef MI_NO_SCHED_INTERLEAVE
+      __builtin_amdgcn_sched_barrier(0);
+#endif
+    });
+    if (PART == PARTS - 1) {
+      lp.advance();
+      lq.advance();
+    }
 #ifdef MI_SETPRIO
     __builtin_amdgcn_s_setprio(0);
 #endif
   };
-  auto issue = [&](char* slot) {
-    lp.issue(slot, wave);
-    lq.issue(slot + P_BYTES, wave);
-  };
-  auto k_tile = [&](int kt, char* cur, char* nxt, char* refill) {
-    const bool refilled = kt + NS - 1 < nk;
-    if (refilled) issue(refill);  // tile kt+NS-1 -> slot (kt-1) % NS
+  // `steady` (a compile-time flag) marks tiles in the middle of the K loop: tile kt+NS exists (so the vacated
+  // slot is refilled and NS-2 younger tiles stay in flight at the wait), and the tile body is branch free.
+  auto k_tile = [&](auto steady, int kt, int cur_slot, const char* cur, const char* nxt) {
+    constexpr bool STEADY = decltype(steady)::value;
+    const int prev_slot = (cur_slot + NS - 1) % NS;  // receives the later parts of tile kt-1+NS
+    if (!STEADY && PARTS > 1 && kt + NS - 1 < nk) issue_parts(prev_slot, 1, PARTS);
 #pragma unroll
     for (int q = 0; q + 1 < NQ; ++q) {
-      fetch(cur, q + 1, (q + 1) & 1);
-      mma(q & 1);
-#ifndef MI_NO_SCHED_INTERLEAVE
-      // one LDS read issued in the shadow of every MFMA
-      constexpr int READS = FM * (P_KS ? 2 : 1) + FN * (Q_KS ? 2 : 1);
-      constexpr int MMAS = FM * FN;
-#pragma unroll
-      for (int x = 0; x < MMAS; ++x) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, (READS + MMAS - 1) / MMAS, 0);
+      if (STEADY && PARTS > 1) {
+        if (q == 0) k_step(std::true_type{}, std::integral_constant<int, (PARTS > 1 ? 1 : -1)>{}, q & 1, cur, q + 1, prev_slot);
+        if (q == 1) k_step(std::true_type{}, std::integral_constant<int, (PARTS > 2 ? 2 : -1)>{}, q & 1, cur, q + 1, prev_slot);
+        if (q == 2) k_step(std::true_type{}, std::integral_constant<int, (PARTS > 3 ? 3 : -1)>{}, q & 1, cur, q + 1, prev_slot);
+      } else {
+        k_step(std::true_type{}, std::integral_constant<int, -1>{}, q & 1, cur, q + 1, 0);
       }
-#endif
     }
-    // own loads of tile kt+1 have landed (younger tiles may stay in flight); own reads of `cur` are done
 #ifdef MI_TIMING
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
     const long long tw0 = __builtin_readcyclecounter();
 #endif
-    if (refilled)
-      __builtin_amdgcn_s_waitcnt(waitcnt_imm((NS - 2) * LOADS_PER_TILE, 0));
-    else
-      __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+    // own loads of tile kt+1 have landed; own reads of `cur` are done
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(STEADY ? (NS - 2) * LOADS_PER_TILE : 0, 0));
 #ifdef MI_TIMING
     const long long tw1 = __builtin_readcyclecounter();
 #endif
@@ -381,44 +592,64 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
     t_load += tw1 - tw0;
     t_bar += tw2 - tw1;
 #endif
-    if (kt + 1 < nk) fetch(nxt, 0, 0);
-    mma((NQ - 1) & 1);
+    if (STEADY) {
+      k_step(std::true_type{}, std::integral_constant<int, 0>{}, (NQ - 1) & 1, nxt, 0, cur_slot);
+    } else {
+      if (kt + NS < nk) issue_parts(cur_slot, 0, 1);
+      if (kt + 1 < nk) fetch(nxt, 0, 0);
+      k_step(std::false_type{}, std::integral_constant<int, -1>{}, (NQ - 1) & 1, nxt, 0, 0);
+    }
   };
+  static_assert(NQ <= 4, "k_tile spells out at most three k-steps before the barrier");
 
 #ifdef MI_TIMING
   const long long t_start = __builtin_readcyclecounter();
 #endif
-  // prologue: tiles 0 .. NS-2 in flight, wait for tile 0
+  // prologue: tiles 0 .. NS-2 and part 0 of tile NS-1 in flight, wait for tile 0
 #pragma unroll
   for (int t = 0; t < NS - 1; ++t)
-    if (t < nk) issue(ring[t]);
-  if (nk >= NS - 1)
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm((NS - 2) * LOADS_PER_TILE, 15));
+    if (t < nk) issue_parts(t, 0, PARTS);
+  if (NS - 1 < nk) issue_parts(NS - 1, 0, 1);
+  if (nk >= NS)
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm((NS - 2) * LOADS_PER_TILE + PL, 15));
   else
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
   __syncthreads();
+#ifdef MI_ABLATE_READS
+#pragma unroll
+  for (int r = 0; r < UNITS; ++r) {
+    if (r < FM) fp[0][r] = fp[1][r] = fast_frag<C, P_KS, C::TILE_M>(ring[0], wm * C::TM + r * MI, kgroup, lane);
+    else fq[0][r - FM] = fq[1][r - FM] = fast_frag<C, Q_KS, C::TILE_N>(ring[0] + P_BYTES, wn * C::TN + (r - FM) * MI, kgroup, lane);
+  }
+#endif
   fetch(ring[0], 0, 0);
-  for (int kt = 0; kt < nk; kt += NS) {
+  int kt = 0;
+  for (; kt + 2 * NS - 1 < nk; kt += NS) {  // every tile of this round is a steady one
+#pragma unroll
+    for (int u = 0; u < NS; ++u) k_tile(std::true_type{}, kt + u, u, ring[u], ring[(u + 1) % NS]);
+  }
+  for (; kt < nk; kt += NS) {
 #pragma unroll
     for (int u = 0; u < NS; ++u)
-      if (kt + u < nk) k_tile(kt + u, ring[u], ring[(u + 1) % NS], ring[(u + NS - 1) % NS]);
+      if (kt + u < nk) k_tile(std::false_type{}, kt + u, u, ring[u], ring[(u + 1) % NS]);
   }
 
+  if constexpr (MI == 16) mfma_drain();
   if constexpr (C::KSPLIT == 2) {
     // Sum the two K groups: group 1 parks its accumulators in the ring (lane-linear, conflict free),
     // group 0 adds them and carries on with the epilogue alone.
-    static_assert(C::KSPLIT == 1 || C::NWG * FM * FN * 4096 <= NS * C::SLOT_BYTES, "accumulators exceed the ring");
+    static_assert(C::KSPLIT == 1 || C::NWG * FM * FN * ACC_N * 256 <= NS * C::SLOT_BYTES, "accumulators exceed the ring");
     __syncthreads();  // all fragment reads of the ring are done
-    char* park = &ring[0][0] + wig * (FM * FN * 4096);
+    char* park = &ring[0][0] + wig * (FM * FN * ACC_N * 256);
     if (kgroup == 1) {
 #pragma unroll
       for (int i = 0; i < FM; ++i)
 #pragma unroll
         for (int j = 0; j < FN; ++j)
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
+          for (int g = 0; g < ACC_N / 4; ++g) {
             f32x4_t v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-            *reinterpret_cast<f32x4_t*>(park + ((i * FN + j) * 4 + g) * 1024 + lane * 16) = v;
+            *reinterpret_cast<f32x4_t*>(park + ((i * FN + j) * (ACC_N / 4) + g) * 1024 + lane * 16) = v;
           }
     }
     __syncthreads();
@@ -428,8 +659,8 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
 #pragma unroll
         for (int j = 0; j < FN; ++j)
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const f32x4_t v = *reinterpret_cast<const f32x4_t*>(park + ((i * FN + j) * 4 + g) * 1024 + lane * 16);
+          for (int g = 0; g < ACC_N / 4; ++g) {
+            const f32x4_t v = *reinterpret_cast<const f32x4_t*>(park + ((i * FN + j) * (ACC_N / 4) + g) * 1024 + lane * 16);
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[i][j][4 * g + r] += v[r];
           }
@@ -449,7 +680,7 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
     static_assert(C::KSPLIT == 1 || MODE == MODE_SYRK, "the K-group variant is wired for SYRK only");
     // (SYRK never takes the per-workgroup sum at the end of tile_epilogue, so group 1 may simply skip it)
     if (C::KSPLIT == 1 || kgroup == 0)
-      tile_epilogue<MODE, OUT_F32, EDGE, FM, FN, NT>(p, acc, m0 + wm * C::TM, n0 + wn * C::TN, lane, batch, diag, p.alpha,
+      tile_epilogue<MODE, OUT_F32, EDGE, FM, FN, NT, MI>(p, acc, m0 + wm * C::TM, n0 + wn * C::TN, lane, batch, diag, p.alpha,
                                                      beta, shift, red);
   }
 #ifdef MI_TIMING
