@@ -262,6 +262,23 @@ __device__ __forceinline__ void tile_epilogue(const GemmParams& p, ACC (&acc)[FM
   constexpr int G = MI == 32 ? 4 : 1;
   const int frow = lane & (MI - 1), fk = lane / MI;
   const uint16_t* __restrict__ Cb = p.Cin ? p.Cin + batch * p.c_bs : nullptr;
+  const bool use_c = beta != 0.0f && Cb != nullptr;
+  // All Cin pieces are requested before the first store (stores may alias Cin as far as the compiler knows, so
+  // loads left between them would each wait out a full memory latency).
+  constexpr bool HOIST_C = FM * FN * G * 2 <= 96;  // register budget
+  uint2 cpre[HOIST_C ? FM : 1][HOIST_C ? FN : 1][G];
+  if (HOIST_C && use_c) {
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          const int m = m_base + i * MI + frow, n = n_base + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
+          cpre[i][j][g] = make_uint2(0u, 0u);
+          if (!GUARD || (m < p.M && n < p.N)) cpre[i][j][g] = *reinterpret_cast<const uint2*>(Cb + (int64_t)m * p.ldc + n);
+        }
+  }
   float ssq = 0.0f;
 #pragma unroll
   for (int i = 0; i < FM; ++i) {
@@ -275,8 +292,17 @@ __device__ __forceinline__ void tile_epilogue(const GemmParams& p, ACC (&acc)[FM
         f32x4_t v;
 #pragma unroll
         for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][4 * g + r];
-        if (beta != 0.0f && Cb != nullptr) {
-          f32x4_t c = load_bf16x4_as_f32(Cb + (int64_t)m * p.ldc + n);
+        if (use_c) {
+          f32x4_t c;
+          if (HOIST_C) {
+            const uint2 raw = cpre[i][j][g];
+            c[0] = __uint_as_float(raw.x << 16);
+            c[1] = __uint_as_float(raw.x & 0xffff0000u);
+            c[2] = __uint_as_float(raw.y << 16);
+            c[3] = __uint_as_float(raw.y & 0xffff0000u);
+          } else {
+            c = load_bf16x4_as_f32(Cb + (int64_t)m * p.ldc + n);
+          }
 #pragma unroll
           for (int r = 0; r < 4; ++r) v[r] = __builtin_fmaf(beta, c[r], v[r]);
         }

@@ -329,7 +329,9 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, typename 
   constexpr int RPI = 64 / LPR;  // rows per read iteration
   static_assert(MI % RPI == 0 && 64 % LPR == 0, "wave tile width must be 32, 64 or 128");
   static_assert(C::NW * MI * ROWB <= C::NS * C::SLOT_BYTES, "epilogue staging exceeds the ring");
-  char* reg = lds + wave * (MI * ROWB);
+  // two staging regions per wavefront when the ring has room: block i+1 is parked while block i is still being
+  // re-read and stored
+  constexpr int NREG = 2 * C::NW * MI * ROWB <= C::NS * C::SLOT_BYTES ? 2 : 1;
   const int frow = lane & (MI - 1), fk = lane / MI;
   const int rr = lane / LPR, cc = (lane % LPR) * 8;
   const uint16_t* __restrict__ Cb = p.Cin ? p.Cin + batch * p.c_bs : nullptr;
@@ -337,7 +339,8 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, typename 
   constexpr int NIT = MI / RPI;
   // All Cin pieces of this lane are requested up front (the fragment registers of the main loop are dead by
   // now), so the global-load latency is paid once instead of once per piece.
-  constexpr bool PREFETCH_ALL = C::FM * NIT * 4 <= 64;  // else one MI-row block at a time (register budget)
+  // (register budget: a workgroup of four wavefronts leaves each lane 512 registers, 256 of them free here)
+  constexpr bool PREFETCH_ALL = C::FM * NIT * 4 <= (C::NW <= 4 ? 160 : 64);  // else one MI-row block at a time
   uint4 cin[C::FM][NIT];
   auto load_cin = [&](int i) {
 #pragma unroll
@@ -355,6 +358,7 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, typename 
 #pragma unroll
   for (int i = 0; i < C::FM; ++i) {
     if (!PREFETCH_ALL) load_cin(i);
+    char* reg = lds + (wave * NREG + i % NREG) * (MI * ROWB);
 #pragma unroll
     for (int j = 0; j < C::FN; ++j)
 #pragma unroll
@@ -398,6 +402,141 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, typename 
   if (p.slots_out != nullptr) {
     const float total = block_sum_f32<C::NT>(ssq, red);
     if (threadIdx.x == 0) p.slots_out[batch * p.slot_stride + p.slot_base + blockIdx.x] = total;
+  }
+}
+
+// SYRK-mode epilogue through LDS.  The accumulator layout gives a lane one output row and 4-column groups, i.e.
+// 8-byte pieces of 16 different rows per store instruction, and the mirrored tile would go out as single bf16
+// values.  Here the finished bf16 tile is assembled in LDS (row-major, rows padded by 16 bytes) and written
+// with 16 bytes per lane along rows; then the transposed tile is assembled the same way (2-byte LDS writes) and
+// written to the mirrored position.  A diagonal tile is assembled once from its lower half (value and mirror
+// image), so the stored result is symmetric bit for bit.  Tiles too large for the ring go in passes of RP rows.
+// Cin (the beta term) is fetched with the same row-wise 16-byte accesses into LDS first and picked up from
+// there in accumulator layout.  Every wavefront of the workgroup must call this (it contains barriers).
+template <class C, bool GUARD>
+__device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename AccVec<C::MI>::type (&acc)[C::FM][C::FN],
+                                                  char* lds, int lane, int wm, int wn, int m0, int n0, int64_t batch,
+                                                  bool diag, float alpha, float beta, float shift) {
+  constexpr int TILE = C::TILE_M, LDT = TILE + 8, MI = C::MI, G = MI == 32 ? 4 : 1, FM = C::FM, FN = C::FN;
+  constexpr int RING = C::NS * C::SLOT_BYTES;
+  constexpr int RP = (TILE * LDT * 2 <= RING) ? TILE : TILE / 2;  // rows per pass
+  constexpr int NPASS = TILE / RP;
+  static_assert(RP * LDT * 2 <= RING, "staging pass exceeds the ring");
+  static_assert(RP % C::TM == 0 && RP % C::TN == 0, "a wavefront's block must fall into one pass");
+  static_assert(C::KSPLIT == 1 && C::TILE_M == C::TILE_N, "square tiles, one K group");
+  constexpr int CPRW = TILE / 8;                        // 16-byte chunks per tile row
+  constexpr int NCH = RP * CPRW / C::NT;                // chunks per thread and pass
+  static_assert(RP * CPRW % C::NT == 0, "write-out must divide evenly");
+  const int tid = threadIdx.x;
+  const int frow = lane & (MI - 1), fk = lane / MI;
+  const int mw = wm * C::TM, nw = wn * C::TN;           // this wavefront's block inside the tile
+  uint16_t* __restrict__ ob = reinterpret_cast<uint16_t*>(p.Out) + batch * p.o_bs;
+  const uint16_t* __restrict__ Cb = p.Cin ? p.Cin + batch * p.c_bs : nullptr;
+  const bool use_c = beta != 0.0f && Cb != nullptr;
+
+  uint2 val[FM][FN][G];  // finished bf16 quads of this lane
+  // ---- values: alpha * acc (+ beta * Cin) (- shift on the diagonal), rounded to bf16 ----
+#pragma unroll
+  for (int h = 0; h < NPASS; ++h) {
+    if (use_c) {
+      __syncthreads();  // the ring (or the previous pass) is no longer read
+#pragma unroll
+      for (int it = 0; it < NCH; ++it) {
+        const int c = tid + it * C::NT, row = c / CPRW, c8 = c % CPRW;
+        const int m = m0 + h * RP + row, n = n0 + c8 * 8;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (!GUARD || (m < p.M && n < p.N)) v = *reinterpret_cast<const uint4*>(Cb + (int64_t)m * p.ldc + n);
+        *reinterpret_cast<uint4*>(lds + (row * LDT + c8 * 8) * 2) = v;
+      }
+      __syncthreads();
+    }
+    if (mw / RP == h) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int g = 0; g < G; ++g) {
+            const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
+            f32x4_t v;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][4 * g + r];
+            if (use_c) {
+              const uint2 raw = *reinterpret_cast<const uint2*>(lds + ((ml - h * RP) * LDT + nl) * 2);
+              v[0] = __builtin_fmaf(beta, __uint_as_float(raw.x << 16), v[0]);
+              v[1] = __builtin_fmaf(beta, __uint_as_float(raw.x & 0xffff0000u), v[1]);
+              v[2] = __builtin_fmaf(beta, __uint_as_float(raw.y << 16), v[2]);
+              v[3] = __builtin_fmaf(beta, __uint_as_float(raw.y & 0xffff0000u), v[3]);
+            }
+            if (p.shift_mode == SHIFT_GRAM && diag) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r)
+                if (nl + r == ml) v[r] -= shift;
+            }
+            val[i][j][g] = __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));
+          }
+    }
+  }
+  auto elem = [&](const uint2& q, int r) -> uint16_t {
+    return (uint16_t)(r == 0 ? (q.x & 0xffffu) : r == 1 ? (q.x >> 16) : r == 2 ? (q.y & 0xffffu) : (q.y >> 16));
+  };
+  // row-wise write-out of one assembled pass: LDS rows [0, RP) -> global rows grow0 + row, columns gcol0 ..
+  auto write_out = [&](int grow0, int gcol0, int row_limit, int col_limit) {
+#pragma unroll
+    for (int it = 0; it < NCH; ++it) {
+      const int c = tid + it * C::NT, row = c / CPRW, c8 = c % CPRW;
+      const int gr = grow0 + row, gc = gcol0 + c8 * 8;
+      const uint4 v = *reinterpret_cast<const uint4*>(lds + (row * LDT + c8 * 8) * 2);
+      if (!GUARD || (gr < row_limit && gc < col_limit)) *reinterpret_cast<uint4*>(ob + (int64_t)gr * p.ldo + gc) = v;
+    }
+  };
+  const bool mirror_in_tile = diag && !p.skip_upper;  // diagonal tile: lower half + its mirror image make the tile
+  // ---- the tile itself ----
+#pragma unroll
+  for (int h = 0; h < NPASS; ++h) {
+    __syncthreads();  // previous readers of the staging area are done
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
+          if (!mirror_in_tile) {
+            if (mw / RP == h) *reinterpret_cast<uint2*>(lds + ((ml - h * RP) * LDT + nl) * 2) = val[i][j][g];
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const uint16_t e = elem(val[i][j][g], r);
+              if (mw / RP == h && nl + r <= ml) *reinterpret_cast<uint16_t*>(lds + ((ml - h * RP) * LDT + nl + r) * 2) = e;
+              if (nw / RP == h && nl + r < ml) *reinterpret_cast<uint16_t*>(lds + ((nl + r - h * RP) * LDT + ml) * 2) = e;
+            }
+          }
+        }
+    __syncthreads();
+    write_out(m0 + h * RP, n0, p.M, p.N);
+  }
+  // ---- the mirrored tile ----
+  if (!diag && !p.skip_upper) {
+#pragma unroll
+    for (int h = 0; h < NPASS; ++h) {
+      __syncthreads();
+      if (nw / RP == h) {
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+          for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+              const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
+#pragma unroll
+              for (int r = 0; r < 4; ++r)
+                *reinterpret_cast<uint16_t*>(lds + ((nl + r - h * RP) * LDT + ml) * 2) = elem(val[i][j][g], r);
+            }
+      }
+      __syncthreads();
+      write_out(n0 + h * RP, m0, p.N, p.M);
+    }
   }
 }
 
@@ -528,7 +667,9 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
     __builtin_amdgcn_s_setprio(MI_SETPRIO);
 #endif
     static_for<MMAS>([&](auto xc) {
-      constexpr int x = decltype(xc)::value, i = x / FN, j = x % FN;
+      // P fragment i stays for FN MFMAs in a row; the Q fragments are walked forth and back, so that one of the
+      // two operands is always the same as in the previous MFMA (measurably less power than changing both)
+      constexpr int x = decltype(xc)::value, i = x / FN, j = (i & 1) ? FN - 1 - x % FN : x % FN;
       if constexpr (MI == 32)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fq[buf][j], fp[buf][i], acc[i][j], 0, 0, 0);
       else
@@ -622,16 +763,34 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
     else fq[0][r - FM] = fq[1][r - FM] = fast_frag<C, Q_KS, C::TILE_N>(ring[0] + P_BYTES, wn * C::TN + (r - FM) * MI, kgroup, lane);
   }
 #endif
-  fetch(ring[0], 0, 0);
-  int kt = 0;
-  for (; kt + 2 * NS - 1 < nk; kt += NS) {  // every tile of this round is a steady one
+  // A wavefront none of whose outputs is ever stored (its rows or columns lie beyond the matrix, or its block is
+  // strictly above the diagonal of a diagonal SYRK tile) keeps loading its share of the operand tiles and keeps
+  // every barrier, but issues no fragment reads and no MFMAs: on this part the clock follows the power drawn,
+  // so work that is thrown away slows down the work that is kept.
+  const bool idle_wave = (m0 + wm * C::TM >= p.M) || (n0 + wn * C::TN >= p.N) ||
+                         (MODE == MODE_SYRK && tm == tn && wn * C::TN >= (wm + 1) * C::TM);
+  if (idle_wave) {
+    for (int kt = 0; kt < nk; ++kt) {
+      const int cur_slot = kt % NS, prev_slot = (cur_slot + NS - 1) % NS;
+      if (PARTS > 1 && kt + NS - 1 < nk) issue_parts(prev_slot, 1, PARTS);
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+#ifndef MI_ABLATE_BARRIER
+      __syncthreads();
+#endif
+      if (kt + NS < nk) issue_parts(cur_slot, 0, 1);
+    }
+  } else {
+    fetch(ring[0], 0, 0);
+    int kt = 0;
+    for (; kt + 2 * NS - 1 < nk; kt += NS) {  // every tile of this round is a steady one
 #pragma unroll
-    for (int u = 0; u < NS; ++u) k_tile(std::true_type{}, kt + u, u, ring[u], ring[(u + 1) % NS]);
-  }
-  for (; kt < nk; kt += NS) {
+      for (int u = 0; u < NS; ++u) k_tile(std::true_type{}, kt + u, u, ring[u], ring[(u + 1) % NS]);
+    }
+    for (; kt < nk; kt += NS) {
 #pragma unroll
-    for (int u = 0; u < NS; ++u)
-      if (kt + u < nk) k_tile(std::false_type{}, kt + u, u, ring[u], ring[(u + 1) % NS]);
+      for (int u = 0; u < NS; ++u)
+        if (kt + u < nk) k_tile(std::false_type{}, kt + u, u, ring[u], ring[(u + 1) % NS]);
+    }
   }
 
   if constexpr (MI == 16) mfma_drain();
@@ -676,6 +835,8 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
     __syncthreads();  // every wavefront has finished reading the ring: it can be reused as staging space
     gemm_epilogue_lds<C, OUT_F32, EDGE>(p, acc, &ring[0][0], wave, lane, m0 + wm * C::TM, n0 + wn * C::TN, batch, p.alpha,
                                         beta, red);
+  } else if constexpr (MODE == MODE_SYRK && !OUT_F32 && C::KSPLIT == 1 && C::NW == 4) {
+    syrk_epilogue_lds<C, EDGE>(p, acc, &ring[0][0], lane, wm, wn, m0, n0, batch, diag, p.alpha, beta, shift);
   } else {
     static_assert(C::KSPLIT == 1 || MODE == MODE_SYRK, "the K-group variant is wired for SYRK only");
     // (SYRK never takes the per-workgroup sum at the end of tile_epilogue, so group 1 may simply skip it)
