@@ -6,8 +6,8 @@
 One "step" = one full orthogonalisation (normalise, bf16 cast, 5 x {SYRK, SYRK, GEMM+AXPY}, float32 result)
 of a Llama-3-8B MLP-shaped float32 gradient that is already resident in HBM.  Prints ONE JSON line:
   value       TFLOP/s on the symmetric-halved FLOP count 5 (3 m^2 n + m^3)
-  roofline    the dominant kernel (GEMM+AXPY, 2 m^2 n FLOP per launch) against the bf16 dense MFMA peak,
-              its duration taken from HIP events the driver records on the launch stream
+  roofline    the dominant kernel (GEMM+AXPY, 2 m^2 n FLOP, issued as two launches) against the bf16 dense MFMA
+              peak, its duration taken from HIP events the driver records on the launch stream
   cpu_baseline the same operator sequence in float32 torch on the host cores (a baseline, not a target)
 This run uses one GPU; --gpus above 1 is refused.
 """
@@ -26,6 +26,10 @@ for _p in (ROOT, os.path.join(ROOT, "emerging-optimizers_amd")):
         sys.path.insert(0, _p)
 
 PEAK_BF16_TFLOPS = 2516.6  # MI355X dense bf16 MFMA: 256 CU x 2.4 GHz x 4096 FLOP/clk/CU
+# HBM-side bytes of one GEMM+AXPY at the headline shape (both launches), from two `rocprofv3 --pmc` runs of this file
+# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for scale_cast_kernel
+# of the same run, whose traffic is known (229 376 KiB read, 114 688 KiB written): factors 1.995 and 1.000.
+GEMM_AXPY_TRAFFIC_BYTES = int(((405954.4 + 146826.3) * 1.995 + (98328.0 + 16392.0) * 1.000) * 1024)
 M, N, NS_STEPS = 4096, 14336, 5
 # Other BASELINE configurations, timed with --workload (the default and the graded line is "mlp").
 WORKLOADS = {
@@ -226,13 +230,13 @@ def main():
             "kernel_ms": {k: (round(v, 4) if v is not None else None) for k, v in per_kernel.items()},
         },
         "roofline": {
-            "kernel": "gemm_fast_kernel (X' = a X + B X, 2 m^2 n FLOP per launch)",
+            "kernel": "gemm_fast_kernel (X' = a X + B X, 2 m^2 n FLOP; 768 tiles of 256x256 + 256 tiles of 256x128)",
             "bound": "mfma",
             "achieved": round(achieved, 2) if achieved else None,
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_BF16_TFLOPS, 4) if achieved else None,
-            "traffic": None,
+            "traffic": GEMM_AXPY_TRAFFIC_BYTES if (M, N) == (4096, 14336) else None,
         },
     }
     if rel > 1e-2:

@@ -413,19 +413,45 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, typename 
 // image), so the stored result is symmetric bit for bit.  Tiles too large for the ring go in passes of RP rows.
 // Cin (the beta term) is fetched with the same row-wise 16-byte accesses into LDS first and picked up from
 // there in accumulator layout.  Every wavefront of the workgroup must call this (it contains barriers).
+// Geometry of the staged SYRK epilogue.
+template <class C>
+struct SyrkStage {
+  static constexpr int TILE = C::TILE_M, LDT = TILE + 8;  // LDS row pitch in elements
+  static constexpr int RING = C::NS * C::SLOT_BYTES;
+  static constexpr int RP = (TILE * LDT * 2 <= RING) ? TILE : TILE / 2;  // rows per pass
+  static constexpr int NPASS = TILE / RP;
+  static constexpr int CPRW = TILE / 8;            // 16-byte chunks per tile row
+  static constexpr int NCH = RP * CPRW / C::NT;    // chunks per thread and pass
+  // a one-pass tile may fetch its Cin rows into registers before the K loop (NCH x 4 registers per lane)
+  static constexpr bool CIN_EARLY = NPASS == 1 && NCH * 4 <= 80;
+};
+// Row-wise 16-byte loads of this thread's Cin chunks of a one-pass tile (issued before the K loop so that the
+// burst of all workgroups does not sit on the critical path at the end of the kernel).
+template <class C, bool GUARD>
+__device__ __forceinline__ void syrk_cin_prefetch(const GemmParams& p, int m0, int n0, int64_t batch,
+                                                  uint4 (&pre)[SyrkStage<C>::NCH]) {
+  using S = SyrkStage<C>;
+  const uint16_t* __restrict__ Cb = p.Cin + batch * p.c_bs;
+#pragma unroll
+  for (int it = 0; it < S::NCH; ++it) {
+    const int c = threadIdx.x + it * C::NT, row = c / S::CPRW, c8 = c % S::CPRW;
+    const int m = m0 + row, n = n0 + c8 * 8;
+    pre[it] = make_uint4(0u, 0u, 0u, 0u);
+    if (!GUARD || (m < p.M && n < p.N)) pre[it] = *reinterpret_cast<const uint4*>(Cb + (int64_t)m * p.ldc + n);
+  }
+}
+
 template <class C, bool GUARD>
 __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename AccVec<C::MI>::type (&acc)[C::FM][C::FN],
                                                   char* lds, int lane, int wm, int wn, int m0, int n0, int64_t batch,
-                                                  bool diag, float alpha, float beta, float shift) {
-  constexpr int TILE = C::TILE_M, LDT = TILE + 8, MI = C::MI, G = MI == 32 ? 4 : 1, FM = C::FM, FN = C::FN;
-  constexpr int RING = C::NS * C::SLOT_BYTES;
-  constexpr int RP = (TILE * LDT * 2 <= RING) ? TILE : TILE / 2;  // rows per pass
-  constexpr int NPASS = TILE / RP;
-  static_assert(RP * LDT * 2 <= RING, "staging pass exceeds the ring");
+                                                  bool diag, float alpha, float beta, float shift,
+                                                  const uint4 (&cin_pre)[SyrkStage<C>::CIN_EARLY ? SyrkStage<C>::NCH : 1]) {
+  using S = SyrkStage<C>;
+  constexpr int TILE = S::TILE, LDT = S::LDT, MI = C::MI, G = MI == 32 ? 4 : 1, FM = C::FM, FN = C::FN;
+  constexpr int RP = S::RP, NPASS = S::NPASS, CPRW = S::CPRW, NCH = S::NCH;
+  static_assert(RP * LDT * 2 <= S::RING, "staging pass exceeds the ring");
   static_assert(RP % C::TM == 0 && RP % C::TN == 0, "a wavefront's block must fall into one pass");
   static_assert(C::KSPLIT == 1 && C::TILE_M == C::TILE_N, "square tiles, one K group");
-  constexpr int CPRW = TILE / 8;                        // 16-byte chunks per tile row
-  constexpr int NCH = RP * CPRW / C::NT;                // chunks per thread and pass
   static_assert(RP * CPRW % C::NT == 0, "write-out must divide evenly");
   const int tid = threadIdx.x;
   const int frow = lane & (MI - 1), fk = lane / MI;
@@ -445,7 +471,10 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
         const int c = tid + it * C::NT, row = c / CPRW, c8 = c % CPRW;
         const int m = m0 + h * RP + row, n = n0 + c8 * 8;
         uint4 v = make_uint4(0u, 0u, 0u, 0u);
-        if (!GUARD || (m < p.M && n < p.N)) v = *reinterpret_cast<const uint4*>(Cb + (int64_t)m * p.ldc + n);
+        if constexpr (S::CIN_EARLY)
+          v = cin_pre[it];  // fetched before the K loop
+        else if (!GUARD || (m < p.M && n < p.N))
+          v = *reinterpret_cast<const uint4*>(Cb + (int64_t)m * p.ldc + n);
         *reinterpret_cast<uint4*>(lds + (row * LDT + c8 * 8) * 2) = v;
       }
       __syncthreads();
@@ -763,6 +792,14 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
     else fq[0][r - FM] = fq[1][r - FM] = fast_frag<C, Q_KS, C::TILE_N>(ring[0] + P_BYTES, wn * C::TN + (r - FM) * MI, kgroup, lane);
   }
 #endif
+  constexpr bool SYRK_STAGED = MODE == MODE_SYRK && !OUT_F32 && C::KSPLIT == 1 && C::NW == 4;
+  constexpr bool CIN_EARLY = SYRK_STAGED && SyrkStage<C>::CIN_EARLY;
+  uint4 cin_pre[CIN_EARLY ? SyrkStage<C>::NCH : 1];
+  if constexpr (CIN_EARLY) {
+    // these loads are older than every direct-to-LDS load issued from here on, so the vmcnt waits of the K
+    // loop cover them as well
+    if (p.Cin != nullptr) syrk_cin_prefetch<C, EDGE>(p, m0, n0, batch, cin_pre);
+  }
   // A wavefront none of whose outputs is ever stored (its rows or columns lie beyond the matrix, or its block is
   // strictly above the diagonal of a diagonal SYRK tile) keeps loading its share of the operand tiles and keeps
   // every barrier, but issues no fragment reads and no MFMAs: on this part the clock follows the power drawn,
@@ -835,8 +872,8 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
     __syncthreads();  // every wavefront has finished reading the ring: it can be reused as staging space
     gemm_epilogue_lds<C, OUT_F32, EDGE>(p, acc, &ring[0][0], wave, lane, m0 + wm * C::TM, n0 + wn * C::TN, batch, p.alpha,
                                         beta, red);
-  } else if constexpr (MODE == MODE_SYRK && !OUT_F32 && C::KSPLIT == 1 && C::NW == 4) {
-    syrk_epilogue_lds<C, EDGE>(p, acc, &ring[0][0], lane, wm, wn, m0, n0, batch, diag, p.alpha, beta, shift);
+  } else if constexpr (SYRK_STAGED) {
+    syrk_epilogue_lds<C, EDGE>(p, acc, &ring[0][0], lane, wm, wn, m0, n0, batch, diag, p.alpha, beta, shift, cin_pre);
   } else {
     static_assert(C::KSPLIT == 1 || MODE == MODE_SYRK, "the K-group variant is wired for SYRK only");
     // (SYRK never takes the per-workgroup sum at the end of tile_epilogue, so group 1 may simply skip it)

@@ -110,8 +110,9 @@ size_t mi_frob_partials_len(int64_t batch, int64_t numel);
  * plus the scale multiplication of Muon's closure (muon.py:131-132).
  *
  * x, out: float32, batch matrices of (rows, cols) row-major contiguous.  The iteration always runs on
- * the orientation with the smaller leading dimension (muon_utils.py:205-208); no transposed copy is
- * made, kernels for both memory orientations exist.  out must not alias x.
+ * the orientation with the smaller leading dimension (muon_utils.py:205-208): a tall input is transposed
+ * while it is cast to bf16 (into the workspace) and the float32 result is transposed back into `out`, so
+ * the MFMA kernels always see the wide layout.  out must not alias x.
  * abc: HOST array of 3*steps floats (a, b, c per step, already expanded by the coefficient iterator).
  * steps == 0 returns the normalised input.  rows and cols must be multiples of 8.
  * workspace: device scratch of at least mi_newton_schulz_workspace_bytes(batch, rows, cols) bytes,
