@@ -38,6 +38,9 @@ WORKLOADS = {
     "mlp_tall": (14336, 4096),     # same MLP weight stored (out, in): exercises the K-strided kernels
     "per_head": (32, 128, 4096),   # 32 heads in one grouped launch
     "moe_shard": (8, 1792, 4096),  # 8 experts, single-GPU shard shape
+    "moe": (8, 4096, 14336),       # 8 stacked experts at full shape (1.9 GB of float32 gradients)
+    "batched_syrk": (16, 2048, 8192),  # batched SYRK alone (no Newton-Schulz), bf16 in / bf16 out
+    "muon_step": (4096, 14336),    # whole Muon.step() (momentum 0.95, Nesterov, weight decay) on the headline gradient
 }
 COEFFS = [(3.4445, -4.7750, 2.0315)] * NS_STEPS  # "simple" table cycled
 
@@ -96,9 +99,84 @@ def cpu_baseline(x_cpu):
     }
 
 
+def batched_syrk_workload(args):
+    """BASELINE configuration 2: batched_tsyrk_ex alone on 16 x (2048 x 8192) bf16, TFLOP/s on B n^2 k."""
+    import torch
+
+    from emerging_optimizers import _hip
+    from emerging_optimizers.triton_kernels import batched_tsyrk_ex
+
+    _hip.lib()
+    dev = torch.device("cuda:0")
+    b, n, k = WORKLOADS["batched_syrk"]
+    a = (torch.randn(b, n, k, generator=torch.Generator().manual_seed(0)) * 0.02).to(torch.bfloat16).to(dev)
+    out = torch.empty(b, n, n, dtype=torch.bfloat16, device=dev)
+    for _ in range(args.warmup):
+        batched_tsyrk_ex(a, out=out)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        batched_tsyrk_ex(a, out=out)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    ref = torch.bmm(a[:2].float(), a[:2].float().mT)
+    rel = float((out[:2].float() - ref).norm() / ref.norm())
+    sym = bool(torch.equal(out, out.mT))
+    tflops = b * n * n * k / (ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "batched SYRK ms + TFLOP/s (% bf16 MFMA peak)", "value": round(tflops, 2), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"batched_tsyrk_ex on {b}x{n}x{k} bf16 (alpha=1, beta=0), FLOPs counted B n^2 k",
+                   "pct_of_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2), "rel_fro_vs_fp32": round(rel, 6),
+                   "bitwise_symmetric": sym},
+    }))
+
+
+def muon_step_workload(args):
+    """Whole optimizer step around the headline orthogonalisation: Muon(momentum 0.95, Nesterov) on one 4096 x 14336 weight."""
+    import torch
+
+    from emerging_optimizers import _hip
+    from emerging_optimizers.orthogonalized_optimizers.muon import Muon
+
+    _hip.lib()
+    dev = torch.device("cuda:0")
+    shape = WORKLOADS["muon_step"]
+    w = torch.nn.Parameter((torch.randn(*shape, generator=torch.Generator().manual_seed(1)) * 0.02).to(dev))
+    opt = Muon([w], lr=3e-4, momentum=0.95, nesterov=True, weight_decay=0.01, num_ns_steps=NS_STEPS,
+               coefficient_type="simple", use_syrk=True, fp32_matmul_prec="medium")
+    grads = [llama_grad(shape, seed=s).to(dev) for s in range(3)]
+    for i in range(args.warmup):
+        w.grad = grads[i % 3]
+        opt.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        w.grad = grads[i % 3]
+        opt.step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    m, n = shape
+    tflops = NS_STEPS * (3 * m * m * n + m**3) / (ms * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "Muon.step ms (momentum + Nesterov + weight decay + NS orthogonalize + update)", "value": round(ms, 4),
+        "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"Muon.step on one {m}x{n} float32 weight, llama-like gradients, lr 3e-4, momentum 0.95, "
+                               "Nesterov, decoupled weight decay 0.01, 5 'simple' NS steps",
+                   "ns_tflops_if_all_time_were_ns": round(tflops, 1), "finite": bool(torch.isfinite(w).all())},
+    }))
+
+
 def side_workload(args):
     """Times another BASELINE configuration through the same entry point; one JSON line, no roofline legs."""
     import torch
+
+    if args.workload == "batched_syrk":
+        return batched_syrk_workload(args)
+    if args.workload == "muon_step":
+        return muon_step_workload(args)
 
     from emerging_optimizers import _hip, utils
     from emerging_optimizers.orthogonalized_optimizers import muon_utils
@@ -106,7 +184,14 @@ def side_workload(args):
     _hip.lib()
     dev = torch.device("cuda:0")
     shape = WORKLOADS[args.workload]
-    x = (torch.randn(*shape, generator=torch.Generator().manual_seed(0)) * 1e-3).to(dev)
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(*shape, generator=gen)
+    if args.workload in ("moe", "moe_shard"):  # per-expert scales log-uniform in [1e-4, 1e-2]
+        lo, hi = torch.log(torch.tensor(1e-4)), torch.log(torch.tensor(1e-2))
+        x = x * torch.exp(lo + (hi - lo) * torch.rand(shape[0], 1, 1, generator=gen))
+    else:
+        x = x * 1e-3
+    x = x.to(dev)
     run = lambda: muon_utils.newton_schulz(x, steps=NS_STEPS, coefficient_type="simple", use_syrk=True)
     with utils.fp32_matmul_precision("medium"), torch.no_grad():
         for _ in range(args.warmup):
@@ -118,6 +203,9 @@ def side_workload(args):
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t0) / args.steps * 1e3
     torch.set_float32_matmul_precision("highest")
+    nref = min(2, x.shape[0]) if x.dim() == 3 and x.numel() > (1 << 28) else None  # parity on two experts of the big batch
+    if nref is not None:
+        x, out = x[:nref], out[:nref]
     X = x.mT if x.shape[-2] > x.shape[-1] else x
     X = X / X.norm(dim=(-2, -1), keepdim=True)
     for a, b, c in COEFFS:

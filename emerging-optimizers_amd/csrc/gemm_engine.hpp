@@ -36,6 +36,7 @@ struct GemmParams {
   int64_t ldo, o_bs;
   int M, N, K;
   float alpha, beta, out_scale;
+  float out_accum;               // float32 output only: Out = out_accum * Out + out_scale * value (0: plain store)
   int tiles_m, tiles_n;
   int skip_upper;
   // Diagonal-shift bookkeeping of the fused Newton-Schulz driver (all null / 0 for plain calls).
@@ -320,6 +321,11 @@ __device__ __forceinline__ void tile_epilogue(const GemmParams& p, ACC (&acc)[FM
           f32x4_t w;
 #pragma unroll
           for (int r = 0; r < 4; ++r) w[r] = v[r] * p.out_scale;
+          if (p.out_accum != 0.0f) {
+            const f32x4_t old = *reinterpret_cast<const f32x4_t*>(o);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) w[r] = __builtin_fmaf(p.out_accum, old[r], w[r]);
+          }
           *reinterpret_cast<f32x4_t*>(o) = w;
         } else {
           uint16_t* ob = reinterpret_cast<uint16_t*>(p.Out) + batch * p.o_bs;

@@ -389,8 +389,18 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, typename 
       for (int e = 0; e < 4; ++e) ssq = __builtin_fmaf(lo[e], lo[e], __builtin_fmaf(hi[e], hi[e], ssq));
       if (OUT_F32) {
         float* o = reinterpret_cast<float*>(p.Out) + batch * p.o_bs + (int64_t)m * p.ldo + n;
-        *reinterpret_cast<f32x4_t*>(o) = lo * p.out_scale;
-        *reinterpret_cast<f32x4_t*>(o + 4) = hi * p.out_scale;
+        lo *= p.out_scale;
+        hi *= p.out_scale;
+        if (p.out_accum != 0.0f) {  // in-place update of a float32 matrix (optimizer step folded into the epilogue)
+          const f32x4_t olo = *reinterpret_cast<const f32x4_t*>(o), ohi = *reinterpret_cast<const f32x4_t*>(o + 4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            lo[e] = __builtin_fmaf(p.out_accum, olo[e], lo[e]);
+            hi[e] = __builtin_fmaf(p.out_accum, ohi[e], hi[e]);
+          }
+        }
+        *reinterpret_cast<f32x4_t*>(o) = lo;
+        *reinterpret_cast<f32x4_t*>(o + 4) = hi;
       } else {
         uint16_t* o = reinterpret_cast<uint16_t*>(p.Out) + batch * p.o_bs + (int64_t)m * p.ldo + n;
         const uint2 a = __builtin_bit_cast(uint2, __builtin_convertvector(lo, bf16x4_t));

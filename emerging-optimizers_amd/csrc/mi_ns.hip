@@ -139,16 +139,17 @@ static int num_cus() {
   return cached;
 }
 
-// Picks the SYRK tile by modelled time: rounds of workgroups over the CUs times the work of one tile.
-// 4096 rows: 256-tiles -> 136 workgroups (1 round at full cost); 192-tiles -> 253 (1 round at 56 % of the cost).
+// SYRK tile of the fast path.  192 x 192 tiles (253 lower-triangle workgroups at 4096 rows: one round on 256 CUs,
+// where 256 x 256 tiles give 136 and leave 47 % of the CUs idle) were at least as fast as 256 x 256 tiles on every
+// shape measured, batched or not, multiples of 256 included (1024 .. 14336 rows, K 1792 .. 14336): the finer
+// granularity wins back more in partial rounds and diagonal tiles than the smaller tile loses in operand reuse.
 static bool syrk_prefers_192(int64_t n, int64_t batch) {
-  const int cus = num_cus();
-  auto cost = [&](int64_t tile, double per_tile) {
-    const int64_t t = ceil_div(n, tile);
-    return (double)ceil_div(t * (t + 1) / 2 * batch, cus) * per_tile;
-  };
-  // per-tile cost ~ tile^2, with a penalty for the 4-wavefront variant's lower MFMA duty cycle
-  return cost(192, 192.0 * 192.0 * 1.15) < cost(256, 256.0 * 256.0);
+#ifdef MI_FORCE_SYRK192
+  return MI_FORCE_SYRK192 != 0;  // tuning builds only
+#endif
+  (void)n;
+  (void)batch;
+  return true;
 }
 
 template <bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
@@ -236,7 +237,7 @@ static int syrk_impl(const void* A, int64_t batch, int64_t n, int64_t k, int64_t
 static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void* X, int64_t x_bs,
                           int64_t x_ld, int x_trans, void* Xout, int64_t o_bs, int64_t o_ld, int64_t batch,
                           int64_t m, int64_t n, float alpha, float beta, int out_fp32, float out_scale,
-                          hipStream_t stream, const ShiftArgs* sh = nullptr) {
+                          hipStream_t stream, const ShiftArgs* sh = nullptr, float out_accum = 0.0f) {
   if (!Bm || !X || !Xout) return fail(MI_ERR_BAD_ARG, "mi_gemm_axpy_bf16: null pointer");
   if (batch < 0 || m < 0 || n < 0) return fail(MI_ERR_BAD_ARG, "mi_gemm_axpy_bf16: negative extent");
   if (m % 8 || n % 8) return fail(MI_ERR_UNSUPPORTED_SHAPE, "M and N must be multiples of 8, got M=%lld, N=%lld", (long long)m, (long long)n);
@@ -260,6 +261,7 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
   p.alpha = alpha;
   p.beta = beta;
   p.out_scale = out_scale;
+  p.out_accum = out_fp32 ? out_accum : 0.0f;
   if (sh) sh->apply(p);
 #ifdef MI_TIMING
   p.slots_in = reinterpret_cast<const float*>(getenv("MI_TIMING_PTR") ? strtoull(getenv("MI_TIMING_PTR"), nullptr, 0) : 0ull);
@@ -361,19 +363,54 @@ __device__ __forceinline__ T block_sum(T v, T* scratch) {
   return total;
 }
 
+// Momentum source of the fused optimizer step (orthogonalized_optimizer.py:185-192 of the reference):
+//   buf <- buf + (1 - beta) (g - buf)           [buf.lerp_(grad, 1 - beta)]
+//   d    = nesterov ? buf - (buf - g) (1 - beta) [grad.lerp(buf, beta)] : buf
+// lerp follows torch's two-branch formula (weight < 0.5: start + w (end - start); else end - (end - start)(1 - w)).
+struct MomentumSrc {
+  float* buf;     // momentum buffer, updated in place by the sum-of-squares pass; null: plain input
+  float beta;
+  int nesterov;
+};
+__device__ __forceinline__ float torch_lerp(float start, float end, float w) {
+  const float diff = end - start;
+  return w < 0.5f ? start + w * diff : end - diff * (1.0f - w);
+}
+__device__ __forceinline__ float momentum_direction(float g, float buf_new, float beta, int nesterov) {
+  return nesterov ? torch_lerp(g, buf_new, beta) : buf_new;
+}
+
 template <bool F64>
 __global__ void __launch_bounds__(NORM_THREADS) sumsq_kernel(const float* __restrict__ x, int64_t numel,
-                                                             double* __restrict__ partials) {
+                                                             double* __restrict__ partials, MomentumSrc mom) {
   const int64_t b = blockIdx.y;
   const float4* __restrict__ xv = reinterpret_cast<const float4*>(x + b * numel);
+  float4* __restrict__ bv = mom.buf ? reinterpret_cast<float4*>(mom.buf + b * numel) : nullptr;
   const int64_t nvec = numel / 4;
+  // with a momentum source: update the buffer in place and return the direction whose norm is wanted
+  auto fetch = [&](int64_t i) {
+    float4 v = xv[i];
+    if (bv) {
+      float4 m = bv[i];
+      m.x = torch_lerp(m.x, v.x, 1.0f - mom.beta);
+      m.y = torch_lerp(m.y, v.y, 1.0f - mom.beta);
+      m.z = torch_lerp(m.z, v.z, 1.0f - mom.beta);
+      m.w = torch_lerp(m.w, v.w, 1.0f - mom.beta);
+      bv[i] = m;
+      v.x = momentum_direction(v.x, m.x, mom.beta, mom.nesterov);
+      v.y = momentum_direction(v.y, m.y, mom.beta, mom.nesterov);
+      v.z = momentum_direction(v.z, m.z, mom.beta, mom.nesterov);
+      v.w = momentum_direction(v.w, m.w, mom.beta, mom.nesterov);
+    }
+    return v;
+  };
   const int64_t stride = (int64_t)gridDim.x * NORM_THREADS;
   __shared__ double scratch_d[NORM_THREADS / 64];
   double total;
   if (F64) {
     double s0 = 0, s1 = 0, s2 = 0, s3 = 0;
     for (int64_t i = (int64_t)blockIdx.x * NORM_THREADS + threadIdx.x; i < nvec; i += stride) {
-      float4 v = xv[i];
+      float4 v = fetch(i);
       s0 += (double)v.x * (double)v.x;
       s1 += (double)v.y * (double)v.y;
       s2 += (double)v.z * (double)v.z;
@@ -383,7 +420,7 @@ __global__ void __launch_bounds__(NORM_THREADS) sumsq_kernel(const float* __rest
   } else {
     float s0 = 0, s1 = 0, s2 = 0, s3 = 0;
     for (int64_t i = (int64_t)blockIdx.x * NORM_THREADS + threadIdx.x; i < nvec; i += stride) {
-      float4 v = xv[i];
+      float4 v = fetch(i);
       s0 = __builtin_fmaf(v.x, v.x, s0);
       s1 = __builtin_fmaf(v.y, v.y, s1);
       s2 = __builtin_fmaf(v.z, v.z, s2);
@@ -401,7 +438,7 @@ __global__ void __launch_bounds__(NORM_THREADS) scale_cast_kernel(const float* _
                                                                   const double* __restrict__ partials, int nparts,
                                                                   float eps, float post_scale, void* __restrict__ out,
                                                                   float* __restrict__ dev_norm,
-                                                                  float* __restrict__ sumsq_out) {
+                                                                  float* __restrict__ sumsq_out, MomentumSrc mom) {
   const int64_t b = blockIdx.y;
   __shared__ double scratch_d[NORM_THREADS / 64];
   double s = 0;
@@ -422,9 +459,21 @@ __global__ void __launch_bounds__(NORM_THREADS) scale_cast_kernel(const float* _
 
   const int64_t nvec8 = numel / 8;
   const float4* __restrict__ xv = reinterpret_cast<const float4*>(x + b * numel);
+  const float4* __restrict__ bv = mom.buf ? reinterpret_cast<const float4*>(mom.buf + b * numel) : nullptr;
+  auto fetch = [&](int64_t i) {  // the direction again, from the buffer the first pass already updated
+    float4 v = xv[i];
+    if (bv) {
+      const float4 m = bv[i];
+      v.x = momentum_direction(v.x, m.x, mom.beta, mom.nesterov);
+      v.y = momentum_direction(v.y, m.y, mom.beta, mom.nesterov);
+      v.z = momentum_direction(v.z, m.z, mom.beta, mom.nesterov);
+      v.w = momentum_direction(v.w, m.w, mom.beta, mom.nesterov);
+    }
+    return v;
+  };
   const int64_t stride = (int64_t)gridDim.x * NORM_THREADS;
   for (int64_t i = (int64_t)blockIdx.x * NORM_THREADS + threadIdx.x; i < nvec8; i += stride) {
-    float4 a = xv[2 * i], c = xv[2 * i + 1];
+    float4 a = fetch(2 * i), c = fetch(2 * i + 1);
     f32x4_t lo = {a.x / divisor, a.y / divisor, a.z / divisor, a.w / divisor};
     f32x4_t hi = {c.x / divisor, c.y / divisor, c.z / divisor, c.w / divisor};
     if (OUT_BF16) {
@@ -447,7 +496,7 @@ __global__ void __launch_bounds__(256) scale_cast_transpose_kernel(const float* 
                                                                    const double* __restrict__ partials, int nparts,
                                                                    float eps, int f64, uint16_t* __restrict__ out,
                                                                    float* __restrict__ dev_norm,
-                                                                   float* __restrict__ sumsq_out) {
+                                                                   float* __restrict__ sumsq_out, MomentumSrc mom) {
   const int64_t b = blockIdx.z;
   __shared__ double scratch_d[NORM_THREADS / 64];
   __shared__ float tile[64][65];
@@ -469,7 +518,16 @@ __global__ void __launch_bounds__(256) scale_cast_transpose_kernel(const float* 
   for (int pass = 0; pass < 4; ++pass) {
     const int r = pass * 16 + (threadIdx.x >> 4), c = (threadIdx.x & 15) * 4;
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (r0 + r < rows && c0 + c < cols) v = *reinterpret_cast<const float4*>(xb + (r0 + r) * cols + c0 + c);
+    if (r0 + r < rows && c0 + c < cols) {
+      v = *reinterpret_cast<const float4*>(xb + (r0 + r) * cols + c0 + c);
+      if (mom.buf) {
+        const float4 mb = *reinterpret_cast<const float4*>(mom.buf + b * rows * cols + (r0 + r) * cols + c0 + c);
+        v.x = momentum_direction(v.x, mb.x, mom.beta, mom.nesterov);
+        v.y = momentum_direction(v.y, mb.y, mom.beta, mom.nesterov);
+        v.z = momentum_direction(v.z, mb.z, mom.beta, mom.nesterov);
+        v.w = momentum_direction(v.w, mb.w, mom.beta, mom.nesterov);
+      }
+    }
     tile[r][c] = v.x / divisor;
     tile[r][c + 1] = v.y / divisor;
     tile[r][c + 2] = v.z / divisor;
@@ -492,8 +550,9 @@ __global__ void __launch_bounds__(256) scale_cast_transpose_kernel(const float* 
 }
 
 // out[b][c][r] = in[b][r][c] for float32 (rows x cols) -> (cols x rows); 64 x 64 tiles through LDS.
+// With accum != 0 the destination is updated in place: out = accum * out + in^T.
 __global__ void __launch_bounds__(256) transpose_f32_kernel(const float* __restrict__ in, int64_t rows, int64_t cols,
-                                                            float* __restrict__ out) {
+                                                            float* __restrict__ out, float accum) {
   const int64_t b = blockIdx.z;
   __shared__ float tile[64][65];
   const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
@@ -515,14 +574,21 @@ __global__ void __launch_bounds__(256) transpose_f32_kernel(const float* __restr
     const int c = pass * 16 + (threadIdx.x >> 4), r = (threadIdx.x & 15) * 4;
     if (c0 + c < cols && r0 + r < rows) {
       f32x4_t v = {tile[r][c], tile[r + 1][c], tile[r + 2][c], tile[r + 3][c]};
-      *reinterpret_cast<f32x4_t*>(ob + (c0 + c) * rows + r0 + r) = v;
+      f32x4_t* dst = reinterpret_cast<f32x4_t*>(ob + (c0 + c) * rows + r0 + r);
+      if (accum != 0.0f) {
+        const f32x4_t old = *dst;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf(accum, old[e], v[e]);
+      }
+      *dst = v;
     }
   }
 }
 
 static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, int f64, void* out, int out_bf16,
                      float post_scale, double* partials, float* dev_norm, hipStream_t stream,
-                     float* sumsq_out = nullptr, int64_t t_rows = 0, int64_t t_cols = 0) {
+                     float* sumsq_out = nullptr, int64_t t_rows = 0, int64_t t_cols = 0,
+                     MomentumSrc mom = MomentumSrc{nullptr, 0.0f, 0}) {
   if (!x || !out || !partials) return fail(MI_ERR_BAD_ARG, "mi_frob_normalize: null pointer");
   if (batch < 0 || numel < 0) return fail(MI_ERR_BAD_ARG, "mi_frob_normalize: negative extent");
   if (numel % 8) return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_frob_normalize: numel must be a multiple of 8, got %lld", (long long)numel);
@@ -532,14 +598,14 @@ static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, in
   const int nb = norm_blocks(numel);
   dim3 grid1(nb, (unsigned)batch), block(NORM_THREADS);
   if (f64)
-    hipLaunchKernelGGL(sumsq_kernel<true>, grid1, block, 0, stream, x, numel, partials);
+    hipLaunchKernelGGL(sumsq_kernel<true>, grid1, block, 0, stream, x, numel, partials, mom);
   else
-    hipLaunchKernelGGL(sumsq_kernel<false>, grid1, block, 0, stream, x, numel, partials);
+    hipLaunchKernelGGL(sumsq_kernel<false>, grid1, block, 0, stream, x, numel, partials, mom);
   if (t_rows > 0) {
     // bf16 output transposed to (t_cols x t_rows)
     dim3 gridt((unsigned)((t_cols + 63) / 64), (unsigned)((t_rows + 63) / 64), (unsigned)batch);
     hipLaunchKernelGGL(scale_cast_transpose_kernel, gridt, block, 0, stream, x, t_rows, t_cols, partials, nb, eps, f64,
-                       static_cast<uint16_t*>(out), dev_norm, sumsq_out);
+                       static_cast<uint16_t*>(out), dev_norm, sumsq_out, mom);
     hipError_t et = hipGetLastError();
     if (et != hipSuccess) return fail(MI_ERR_LAUNCH, "mi_frob_normalize launch failed: %s", hipGetErrorString(et));
     return MI_OK;
@@ -548,7 +614,7 @@ static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, in
   if (want < 1) want = 1;
   if (want > 4096) want = 4096;
   dim3 grid2((unsigned)want, (unsigned)batch);
-#define MI_SC(F, B) hipLaunchKernelGGL((scale_cast_kernel<F, B>), grid2, block, 0, stream, x, numel, partials, nb, eps, post_scale, out, dev_norm, sumsq_out)
+#define MI_SC(F, B) hipLaunchKernelGGL((scale_cast_kernel<F, B>), grid2, block, 0, stream, x, numel, partials, nb, eps, post_scale, out, dev_norm, sumsq_out, mom)
   if (f64) {
     if (out_bf16) MI_SC(true, true); else MI_SC(true, false);
   } else {
@@ -594,6 +660,103 @@ static NsWorkspace ns_layout(int64_t batch, int64_t rows, int64_t cols) {
 }  // namespace mi
 
 using namespace mi;
+
+// Shared body of mi_newton_schulz_bf16 and mi_muon_update_bf16.  `mom.buf` != null: x is the gradient and the
+// matrix that is orthogonalised is the momentum direction (the buffer is updated in place on the way).
+// `out_accum` != 0: out is updated in place, out = out_accum * out + out_scale * result.
+static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int64_t cols, const float* abc, int steps,
+                   float eps, int accumulate_fp64, float out_scale, void* workspace, size_t workspace_bytes,
+                   hipStream_t stream, MomentumSrc mom, float out_accum) {
+  if (!x || !out) return fail(MI_ERR_BAD_ARG, "mi_newton_schulz_bf16: null tensor pointer");
+  if (batch < 0 || rows < 0 || cols < 0 || steps < 0) return fail(MI_ERR_BAD_ARG, "mi_newton_schulz_bf16: negative argument");
+  if (steps > 0 && !abc) return fail(MI_ERR_BAD_ARG, "mi_newton_schulz_bf16: abc is null");
+  if (rows % 8 || cols % 8)
+    return fail(MI_ERR_UNSUPPORTED_SHAPE, "rows and cols must be multiples of 8, got %lld x %lld", (long long)rows, (long long)cols);
+  if (batch == 0 || rows == 0 || cols == 0) return MI_OK;
+  const NsWorkspace w = ns_layout(batch, rows, cols);
+  if (!workspace || workspace_bytes < w.total)
+    return fail(MI_ERR_WORKSPACE, "workspace too small: need %zu bytes, got %zu", w.total, workspace_bytes);
+  if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(MI_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+
+  char* ws = static_cast<char*>(workspace);
+  uint16_t* xbuf[2] = {reinterpret_cast<uint16_t*>(ws + w.x0), reinterpret_cast<uint16_t*>(ws + w.x1)};
+  uint16_t* gram = reinterpret_cast<uint16_t*>(ws + w.a);
+  uint16_t* poly = reinterpret_cast<uint16_t*>(ws + w.b);
+  double* partials = reinterpret_cast<double*>(ws + w.partials);
+  float* norm = reinterpret_cast<float*>(ws + w.norm);
+
+  const int64_t numel = rows * cols;
+  if (steps == 0) {
+    if (mom.buf || out_accum != 0.0f) return fail(MI_ERR_BAD_ARG, "the fused optimizer update needs at least one step");
+    return frob_impl(x, batch, numel, eps, accumulate_fp64, out, /*out_bf16=*/0, out_scale, partials, norm, stream);
+  }
+
+  float* slots = reinterpret_cast<float*>(ws + w.slots);
+  float* shift = reinterpret_cast<float*>(ws + w.shift);
+  // The iteration runs on the (m x n) orientation with m <= n, K-contiguous in memory.  A tall input is
+  // transposed while it is cast to bf16, and its float32 result is transposed back at the end.
+  const int tall = rows > cols;
+  const int trans = 0;
+  const int64_t m = tall ? cols : rows, n = tall ? rows : cols;
+  const int64_t ld = n;
+  const int64_t x_bs = numel, g_bs = m * m;
+  float* result = tall ? reinterpret_cast<float*>(ws + w.result) : out;
+  int rc;
+  {
+    ProfScope prof(PROF_NORMALIZE, stream);
+    rc = frob_impl(x, batch, numel, eps, accumulate_fp64, xbuf[0], /*out_bf16=*/1, 1.0f, partials, norm, stream, slots,
+                   tall ? rows : 0, tall ? cols : 0, mom);
+  }
+  if (rc != MI_OK) return rc;
+
+  int cur = 0;
+  int nslots = 1;  // the normalisation kernel left one value per matrix
+  for (int s = 0; s < steps; ++s) {
+    const float a = abc[3 * s], b = abc[3 * s + 1], c = abc[3 * s + 2];
+    const bool last = (s + 1 == steps);
+    // A' = X X^T - s I  (s = ||X||_F^2 / m from the partial sums the previous kernel left)
+    ShiftArgs sh_gram{SHIFT_GRAM, b, c, slots, nslots, shift, nullptr};
+    {
+      ProfScope prof(PROF_GRAM, stream);
+      rc = syrk_impl(xbuf[cur], batch, m, n, x_bs, ld, trans, nullptr, 0, m, 1.0f, 0.0f, gram, g_bs, m, 0, stream, &sh_gram);
+    }
+    if (rc != MI_OK) return rc;
+    const uint16_t* mult = gram;
+    float alpha = b;
+    if (c != 0.0f) {
+      // B' = c A'^2 + (b + 2 c s) A'
+      ShiftArgs sh_poly{SHIFT_POLY, b, c, nullptr, 0, shift, nullptr};
+      {
+        ProfScope prof(PROF_POLY, stream);
+        rc = syrk_impl(gram, batch, m, m, g_bs, m, 0, gram, g_bs, m, c, b, poly, g_bs, m, 0, stream, &sh_poly);
+      }
+      if (rc != MI_OK) return rc;
+      mult = poly;
+      alpha = 1.0f;
+    }
+    // X' = (a + b s + c s^2) X + B' X      (cubic: (a + b s) X + b A' X)
+    void* dst = last ? static_cast<void*>(result) : static_cast<void*>(xbuf[cur ^ 1]);
+    ShiftArgs sh_apply{SHIFT_APPLY, b, c, nullptr, 0, shift, last ? nullptr : slots};
+    {
+      ProfScope prof(PROF_APPLY, stream);
+      rc = gemm_axpy_impl(mult, g_bs, m, xbuf[cur], x_bs, ld, trans, dst, x_bs, ld, batch, m, n, alpha, a,
+                          last ? 1 : 0, last ? out_scale : 1.0f, stream, &sh_apply, (last && !tall) ? out_accum : 0.0f);
+    }
+    if (rc != MI_OK) return rc;
+    nslots = g_last_tiles;
+    if (nslots > w.max_slots) return fail(MI_ERR_WORKSPACE, "internal: %d partial-sum slots exceed the %lld reserved", nslots, (long long)w.max_slots);
+    cur ^= 1;
+  }
+  if (tall) {
+    ProfScope prof(PROF_NORMALIZE, stream);
+    dim3 gridt((unsigned)((n + 63) / 64), (unsigned)((m + 63) / 64), (unsigned)batch), blockt(256);
+    hipLaunchKernelGGL(transpose_f32_kernel, gridt, blockt, 0, stream, result, m, n, out, out_accum);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "transpose launch failed: %s", hipGetErrorString(e));
+  }
+  return MI_OK;
+}
+
 
 extern "C" {
 
@@ -669,94 +832,22 @@ size_t mi_newton_schulz_workspace_bytes(int64_t batch, int64_t rows, int64_t col
 
 int mi_newton_schulz_bf16(const float* x, float* out, int64_t batch, int64_t rows, int64_t cols, const float* abc,
                           int steps, float eps, int accumulate_fp64, float out_scale, void* workspace,
-                          size_t workspace_bytes, void* stream_v) {
-  hipStream_t stream = static_cast<hipStream_t>(stream_v);
-  if (!x || !out) return fail(MI_ERR_BAD_ARG, "mi_newton_schulz_bf16: null tensor pointer");
-  if (batch < 0 || rows < 0 || cols < 0 || steps < 0) return fail(MI_ERR_BAD_ARG, "mi_newton_schulz_bf16: negative argument");
-  if (steps > 0 && !abc) return fail(MI_ERR_BAD_ARG, "mi_newton_schulz_bf16: abc is null");
-  if (rows % 8 || cols % 8)
-    return fail(MI_ERR_UNSUPPORTED_SHAPE, "rows and cols must be multiples of 8, got %lld x %lld", (long long)rows, (long long)cols);
-  if (batch == 0 || rows == 0 || cols == 0) return MI_OK;
-  const NsWorkspace w = ns_layout(batch, rows, cols);
-  if (!workspace || workspace_bytes < w.total)
-    return fail(MI_ERR_WORKSPACE, "workspace too small: need %zu bytes, got %zu", w.total, workspace_bytes);
-  if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(MI_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+                          size_t workspace_bytes, void* stream) {
+  return ns_impl(x, out, batch, rows, cols, abc, steps, eps, accumulate_fp64, out_scale, workspace, workspace_bytes,
+                 static_cast<hipStream_t>(stream), MomentumSrc{nullptr, 0.0f, 0}, 0.0f);
+}
 
-  char* ws = static_cast<char*>(workspace);
-  uint16_t* xbuf[2] = {reinterpret_cast<uint16_t*>(ws + w.x0), reinterpret_cast<uint16_t*>(ws + w.x1)};
-  uint16_t* gram = reinterpret_cast<uint16_t*>(ws + w.a);
-  uint16_t* poly = reinterpret_cast<uint16_t*>(ws + w.b);
-  double* partials = reinterpret_cast<double*>(ws + w.partials);
-  float* norm = reinterpret_cast<float*>(ws + w.norm);
-
-  const int64_t numel = rows * cols;
-  if (steps == 0)
-    return frob_impl(x, batch, numel, eps, accumulate_fp64, out, /*out_bf16=*/0, out_scale, partials, norm, stream);
-
-  float* slots = reinterpret_cast<float*>(ws + w.slots);
-  float* shift = reinterpret_cast<float*>(ws + w.shift);
-  // The iteration runs on the (m x n) orientation with m <= n, K-contiguous in memory.  A tall input is
-  // transposed while it is cast to bf16, and its float32 result is transposed back at the end.
-  const int tall = rows > cols;
-  const int trans = 0;
-  const int64_t m = tall ? cols : rows, n = tall ? rows : cols;
-  const int64_t ld = n;
-  const int64_t x_bs = numel, g_bs = m * m;
-  float* result = tall ? reinterpret_cast<float*>(ws + w.result) : out;
-  int rc;
-  {
-    ProfScope prof(PROF_NORMALIZE, stream);
-    rc = frob_impl(x, batch, numel, eps, accumulate_fp64, xbuf[0], /*out_bf16=*/1, 1.0f, partials, norm, stream, slots,
-                   tall ? rows : 0, tall ? cols : 0);
-  }
-  if (rc != MI_OK) return rc;
-
-  int cur = 0;
-  int nslots = 1;  // the normalisation kernel left one value per matrix
-  for (int s = 0; s < steps; ++s) {
-    const float a = abc[3 * s], b = abc[3 * s + 1], c = abc[3 * s + 2];
-    const bool last = (s + 1 == steps);
-    // A' = X X^T - s I  (s = ||X||_F^2 / m from the partial sums the previous kernel left)
-    ShiftArgs sh_gram{SHIFT_GRAM, b, c, slots, nslots, shift, nullptr};
-    {
-      ProfScope prof(PROF_GRAM, stream);
-      rc = syrk_impl(xbuf[cur], batch, m, n, x_bs, ld, trans, nullptr, 0, m, 1.0f, 0.0f, gram, g_bs, m, 0, stream, &sh_gram);
-    }
-    if (rc != MI_OK) return rc;
-    const uint16_t* mult = gram;
-    float alpha = b;
-    if (c != 0.0f) {
-      // B' = c A'^2 + (b + 2 c s) A'
-      ShiftArgs sh_poly{SHIFT_POLY, b, c, nullptr, 0, shift, nullptr};
-      {
-        ProfScope prof(PROF_POLY, stream);
-        rc = syrk_impl(gram, batch, m, m, g_bs, m, 0, gram, g_bs, m, c, b, poly, g_bs, m, 0, stream, &sh_poly);
-      }
-      if (rc != MI_OK) return rc;
-      mult = poly;
-      alpha = 1.0f;
-    }
-    // X' = (a + b s + c s^2) X + B' X      (cubic: (a + b s) X + b A' X)
-    void* dst = last ? static_cast<void*>(result) : static_cast<void*>(xbuf[cur ^ 1]);
-    ShiftArgs sh_apply{SHIFT_APPLY, b, c, nullptr, 0, shift, last ? nullptr : slots};
-    {
-      ProfScope prof(PROF_APPLY, stream);
-      rc = gemm_axpy_impl(mult, g_bs, m, xbuf[cur], x_bs, ld, trans, dst, x_bs, ld, batch, m, n, alpha, a,
-                          last ? 1 : 0, last ? out_scale : 1.0f, stream, &sh_apply);
-    }
-    if (rc != MI_OK) return rc;
-    nslots = g_last_tiles;
-    if (nslots > w.max_slots) return fail(MI_ERR_WORKSPACE, "internal: %d partial-sum slots exceed the %lld reserved", nslots, (long long)w.max_slots);
-    cur ^= 1;
-  }
-  if (tall) {
-    ProfScope prof(PROF_NORMALIZE, stream);
-    dim3 gridt((unsigned)((n + 63) / 64), (unsigned)((m + 63) / 64), (unsigned)batch), blockt(256);
-    hipLaunchKernelGGL(transpose_f32_kernel, gridt, blockt, 0, stream, result, m, n, out);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "transpose launch failed: %s", hipGetErrorString(e));
-  }
-  return MI_OK;
+int mi_muon_update_bf16(float* param, const float* grad, float* momentum, int64_t batch, int64_t rows, int64_t cols,
+                        float beta, int nesterov, float param_decay, float update_scale, const float* abc, int steps,
+                        float eps, int accumulate_fp64, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!param || !grad || !momentum) return fail(MI_ERR_BAD_ARG, "mi_muon_update_bf16: null tensor pointer");
+  if (steps < 1) return fail(MI_ERR_BAD_ARG, "mi_muon_update_bf16: steps must be at least 1");
+  if (param_decay == 0.0f) return fail(MI_ERR_BAD_ARG, "mi_muon_update_bf16: param_decay must not be 0");
+  if (!aligned16(param) || !aligned16(grad) || !aligned16(momentum))
+    return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_muon_update_bf16: pointers must be 16-byte aligned");
+  return ns_impl(grad, param, batch, rows, cols, abc, steps, eps, accumulate_fp64, update_scale, workspace,
+                 workspace_bytes, static_cast<hipStream_t>(stream), MomentumSrc{momentum, beta, nesterov ? 1 : 0},
+                 param_decay);
 }
 
 }  // extern "C"

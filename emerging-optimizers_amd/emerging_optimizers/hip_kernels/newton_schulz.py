@@ -11,7 +11,7 @@ from .. import _hip
 from . import _launch
 
 
-__all__ = ["gemm_axpy", "fused_newton_schulz", "fused_supported"]
+__all__ = ["gemm_axpy", "fused_newton_schulz", "fused_supported", "fused_muon_update"]
 
 
 def gemm_axpy(
@@ -122,3 +122,46 @@ def fused_newton_schulz(
         )  # fmt: skip
     _hip.check(rc)
     return out
+
+
+def fused_muon_update(
+    param: torch.Tensor,
+    grad: torch.Tensor,
+    momentum_buffer: torch.Tensor,
+    coefficients: Sequence[tuple[float, float, float]],
+    *,
+    beta: float,
+    nesterov: bool,
+    param_decay: float,
+    update_scale: float,
+    eps: float = 1e-15,
+) -> None:
+    """One fused Muon update of ``param`` in place (see ``mi_muon_update_bf16``).
+
+    ``momentum_buffer.lerp_(grad, 1 - beta)``; direction = ``grad.lerp(buffer, beta)`` if ``nesterov`` else the
+    buffer; ``param = param_decay * param + update_scale * newton_schulz(direction)``.  The body of the
+    parameter loop of the reference's ``OrthogonalizedOptimizer.step`` (orthogonalized_optimizer.py:185-210)
+    for weight-decay methods that only scale the parameter.  All three tensors: GPU float32, same shape,
+    contiguous, distinct storage.
+    """
+    if not (fused_supported(param) and grad.shape == param.shape and momentum_buffer.shape == param.shape):
+        raise RuntimeError(f"fused_muon_update cannot take tensors of shape {tuple(param.shape)} / {tuple(grad.shape)}")
+    for t, name in ((param, "param"), (grad, "grad"), (momentum_buffer, "momentum_buffer")):
+        if not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.device == param.device):
+            raise RuntimeError(f"fused_muon_update: {name} must be a contiguous float32 tensor on {param.device}")
+    if len(coefficients) < 1:
+        raise ValueError("fused_muon_update needs at least one Newton-Schulz step")
+    batch = param.shape[0] if param.dim() == 3 else 1
+    rows, cols = param.shape[-2], param.shape[-1]
+    lib = _hip.lib()
+    flat = [float(v) for abc in coefficients for v in abc]
+    abc = (ctypes.c_float * len(flat))(*flat)
+    with torch.cuda.device(param.device):
+        nbytes = lib.mi_newton_schulz_workspace_bytes(batch, rows, cols)
+        ws = _workspace(param.device, nbytes)
+        rc = lib.mi_muon_update_bf16(
+            _launch.ptr(param), _launch.ptr(grad), _launch.ptr(momentum_buffer), batch, rows, cols,
+            float(beta), int(bool(nesterov)), float(param_decay), float(update_scale), abc, len(coefficients),
+            float(eps), 0, _launch.ptr(ws), ws.numel(), _hip.current_stream_ptr(param.device),
+        )  # fmt: skip
+    _hip.check(rc)

@@ -30,6 +30,11 @@ _log = logging.getLogger(__name__)
 
 MuonScaleT = Literal["shape_scaling", "spectral", "unit_rms_norm"]
 
+# Switch of the one-call parameter update (momentum + Nesterov + Newton-Schulz + weight update in the library,
+# see hip_kernels.fused_muon_update).  Results agree with the statement-by-statement path to float32 rounding of
+# the elementwise parts; set to False to run the latter.
+FUSED_MUON_STEP = True
+
 
 def get_muon_scale_factor(size_out: int, size_in: int, mode: MuonScaleT = "spectral") -> float:
     """Multiplier applied to the orthogonalised update of a ``(size_out, size_in)`` weight.
@@ -135,6 +140,46 @@ class Muon(OrthogonalizedOptimizer[HookStateT]):
             scaled_orthogonalize_fn=scaled_orthogonalize_fn,
             weight_update_hook=weight_update_hook,
         )
+        self._own_scaled_orthogonalize_fn = scaled_orthogonalize_fn
+
+    def _fused_update(
+        self, p: torch.Tensor, grad: torch.Tensor, buf: torch.Tensor, lr: float, beta: float, weight_decay: float
+    ) -> bool:
+        """Whole update of one 2-D parameter in a single library call, when nothing needs the intermediates.
+
+        Taken for GPU float32 parameters with both dims multiples of 8 under ``use_syrk`` and matmul precision
+        "medium", with the library's own ``newton_schulz``, no subclass or weight-update hooks, and a weight
+        decay that only scales the parameter (every method except ``"l2"``, which modifies the gradient).
+        """
+        if not (FUSED_MUON_STEP and self._use_syrk and self.fp32_matmul_prec == "medium" and p.ndim == 2):
+            return False
+        if self.scaled_orthogonalize_fn is not self._own_scaled_orthogonalize_fn or not self._update_is_plain():
+            return False
+        if muon_utils.newton_schulz is not muon_utils._ORIGINAL_NEWTON_SCHULZ:
+            return False
+        if not muon_utils._fused_path_ok(grad, grad.size(-2) > grad.size(-1), None):
+            return False
+        tensors = (p, grad, buf)
+        if not all(t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.shape == p.shape for t in tensors):
+            return False
+        if len({t.data_ptr() for t in tensors}) != 3 or not isinstance(lr, (int, float)):
+            return False
+        shrink = 0.0
+        if weight_decay != 0.0:
+            shrink = {
+                "decoupled": weight_decay * lr,
+                "independent": weight_decay,
+                "palm": weight_decay * lr * lr,
+            }.get(self.weight_decay_method)
+            if shrink is None or shrink == 1.0:
+                return False  # "l2" changes the gradient; a decay of exactly 1 is left to the generic statements
+        coeffs = muon_utils._schedule(self._num_ns_steps, self._coefficient_type, None)
+        scale = get_muon_scale_factor(p.size(-2), p.size(-1), mode=self._scale_mode) * self._extra_scale_factor
+        hip_kernels.fused_muon_update(
+            p.data, grad, buf, coeffs, beta=beta, nesterov=self.nesterov, param_decay=1.0 - shrink,
+            update_scale=-lr * scale,
+        )  # fmt: skip
+        return True
 
 
 def _read_only(name: str) -> property:

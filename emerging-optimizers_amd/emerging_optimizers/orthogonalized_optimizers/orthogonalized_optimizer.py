@@ -96,6 +96,8 @@ class OrthogonalizedOptimizer(WeightDecayMixin, Optimizer, Generic[HookStateT]):
                 if grad is None:
                     continue
                 buf = self.state[p]["momentum_buffer"]
+                if self._fused_update(p, grad, buf, lr, beta, group["weight_decay"]):
+                    continue
                 self._apply_weight_decay_inplace(p, grad, lr, group["weight_decay"])
                 buf.lerp_(grad, 1 - beta)
                 direction = grad.lerp(buf, beta) if self.nesterov else buf
@@ -107,6 +109,26 @@ class OrthogonalizedOptimizer(WeightDecayMixin, Optimizer, Generic[HookStateT]):
                 self.post_weight_update_fn_inplace(p)
                 self._weight_update_hook.post_weight_update_inplace(p, hook_state)
         return None
+
+    def _fused_update(
+        self, p: torch.Tensor, grad: torch.Tensor, buf: torch.Tensor, lr: float, beta: float, weight_decay: float
+    ) -> bool:
+        """Hook for subclasses that can do the whole update of ``p`` in one library call.
+
+        Return ``True`` after having updated ``buf`` and ``p`` exactly as the statements of :meth:`step` that
+        follow would have; return ``False`` (the default) to let :meth:`step` run them.
+        """
+        return False
+
+    def _update_is_plain(self) -> bool:
+        """No subclass or hook needs to see the update tensor, so it does not have to exist in memory."""
+        cls = type(self)
+        return (
+            cls.orthogonalize is OrthogonalizedOptimizer.orthogonalize
+            and cls.pre_weight_update_fn_inplace is OrthogonalizedOptimizer.pre_weight_update_fn_inplace
+            and cls.post_weight_update_fn_inplace is OrthogonalizedOptimizer.post_weight_update_fn_inplace
+            and type(self._weight_update_hook) is NoOpWeightUpdateHook
+        )
 
     def orthogonalize(self, p: torch.Tensor, grad: torch.Tensor, **kwargs: Any) -> torch.Tensor:
         """Turn the momentum ``grad`` of parameter ``p`` into the update.

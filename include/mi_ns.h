@@ -124,6 +124,28 @@ int mi_newton_schulz_bf16(const float* x, float* out, int64_t batch, int64_t row
 size_t mi_newton_schulz_workspace_bytes(int64_t batch, int64_t rows, int64_t cols);
 
 /*
+ * One fused Muon update of a float32 parameter batch: momentum, Nesterov direction, Newton-Schulz
+ * orthogonalisation and the weight update, without materialising the direction or the update in HBM:
+ *   momentum <- momentum + (1 - beta) (grad - momentum)                 buf.lerp_(grad, 1 - beta)
+ *   d         = nesterov ? lerp(grad, momentum, beta) : momentum        grad.lerp(buf, beta)
+ *   param    <- param_decay * param + update_scale * NewtonSchulz(d)
+ *
+ * Replaces, for the decoupled / independent / palm weight-decay methods (which only scale the parameter,
+ * mixin.py:35-56), the body of the parameter loop of OrthogonalizedOptimizer.step
+ *   emerging_optimizers/orthogonalized_optimizers/orthogonalized_optimizer.py:185-210
+ * together with Muon's closure (muon.py:117-132): param_decay = 1 - wd*lr (decoupled), 1 - wd (independent),
+ * 1 - wd*lr^2 (palm), 1 (no decay); update_scale = -lr * get_muon_scale_factor(...) * extra_scale_factor.
+ * The momentum update and the sum of squares share one pass over grad and momentum, the divide + bf16 cast
+ * recomputes d in a second pass, and the last GEMM epilogue (or the final transpose of a tall parameter)
+ * updates param in place.  param, grad, momentum: float32 (batch, rows, cols) row-major contiguous, distinct
+ * buffers.  Other arguments and the workspace as for mi_newton_schulz_bf16; steps >= 1; param_decay != 0.
+ */
+int mi_muon_update_bf16(float* param, const float* grad, float* momentum, int64_t batch, int64_t rows, int64_t cols,
+                        float beta, int nesterov, float param_decay, float update_scale,
+                        const float* abc, int steps, float eps, int accumulate_fp64,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Per-kernel timing of mi_newton_schulz_bf16 for benchmarks (no counterpart in the reference, whose
  * benchmark brackets whole calls with torch.cuda.profiler.start/stop, benchmarks/newton_schulz_benchmark.py:155-164).
  * Between mi_profile_begin() and mi_profile_end() every kernel group the driver enqueues is bracketed by a

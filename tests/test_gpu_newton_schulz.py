@@ -275,3 +275,75 @@ def test_per_head_muon_equivalence(gpu):
         stacked = fn(g.view(heads, d, n)).reshape(heads * d, n)
         separate = torch.cat([fn(g[i * d:(i + 1) * d]) for i in range(heads)])
     torch.testing.assert_close(stacked, separate, atol=1e-6, rtol=0)
+
+
+# ---------------------------------------------------------------- one-call Muon update
+@pytest.mark.parametrize("shape", [(256, 512), (512, 256), (1024, 1024), (1024, 3584), (3584, 1024)])
+@pytest.mark.parametrize("nesterov", [True, False])
+def test_fused_muon_update_matches_explicit_statements(gpu, shape, nesterov):
+    """mi_muon_update_bf16 against lerp_/lerp + newton_schulz + the two in-place parameter updates."""
+    lr, beta, wd = 0.02, 0.95, 0.1
+    gen = torch.Generator().manual_seed(7)
+    p0 = (torch.randn(shape, generator=gen) * 0.02).to(gpu)
+    buf0 = (torch.randn(shape, generator=gen) * 1e-3).to(gpu)
+    g = llama_grad(shape, seed=3).to(gpu)
+    scale = muon.get_muon_scale_factor(*shape, mode="spectral")
+    # statement by statement, as OrthogonalizedOptimizer.step does it
+    p_ref, buf_ref = p0.clone(), buf0.clone()
+    p_ref.add_(p_ref, alpha=-wd * lr)
+    buf_ref.lerp_(g, 1 - beta)
+    direction = g.lerp(buf_ref, beta) if nesterov else buf_ref
+    with utils.fp32_matmul_precision("medium"):
+        update = muon_utils.newton_schulz(direction, steps=5, coefficient_type="simple", use_syrk=True) * scale
+    p_ref.add_(update, alpha=-lr)
+    # one call
+    p, buf = p0.clone(), buf0.clone()
+    hip_kernels.fused_muon_update(p, g, buf, SIMPLE5, beta=beta, nesterov=nesterov, param_decay=1 - wd * lr,
+                                  update_scale=-lr * scale)
+    torch.testing.assert_close(buf, buf_ref, rtol=2e-6, atol=5e-9)  # one ulp of the largest entries (5e-2)
+    # the parameter differs only through float32 rounding of the elementwise parts and through bf16 rounding flips
+    # of a direction that may differ in the last bit (square matrices amplify those the most): below the 1e-2
+    # budget each of the two results has against float32
+    assert float((p - p_ref).norm() / (p_ref - p0).norm()) <= 8e-3
+    assert float(rel_fro(_np((p - (1 - wd * lr) * p0) / (-lr * scale)), _np(ns_fp32_torch(direction, SIMPLE5)))) <= TOL_FP32
+
+
+@pytest.mark.parametrize("method,wd", [("decoupled", 0.1), ("independent", 0.01), ("palm", 0.5), ("decoupled", 0.0)])
+def test_muon_step_takes_the_fused_update_and_agrees_with_the_statement_path(gpu, monkeypatch, method, wd):
+    shape, lr = (512, 1024), 0.02
+    w0 = torch.randn(shape, generator=torch.Generator().manual_seed(1)) * 0.02
+    p, q = nn.Parameter(w0.clone().to(gpu)), nn.Parameter(w0.clone().to(gpu))
+    kw = dict(lr=lr, momentum=0.95, nesterov=True, weight_decay=wd, weight_decay_method=method,
+              coefficient_type="simple", use_syrk=True)
+    fused, plain = muon.Muon([p], **kw), muon.Muon([q], **kw)
+    calls = []
+    real = hip_kernels.fused_muon_update
+    monkeypatch.setattr(hip_kernels, "fused_muon_update", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    for step in range(3):
+        g = llama_grad(shape, seed=200 + step).to(gpu)
+        p.grad, q.grad = g.clone(), g.clone()
+        fused.step()
+        n_calls = len(calls)
+        monkeypatch.setattr(muon, "FUSED_MUON_STEP", False)
+        plain.step()
+        monkeypatch.setattr(muon, "FUSED_MUON_STEP", True)
+        assert len(calls) == n_calls == step + 1  # the fused optimizer used the library call, the plain one did not
+    torch.testing.assert_close(fused.state[p]["momentum_buffer"], plain.state[q]["momentum_buffer"], rtol=2e-6, atol=5e-9)
+    assert float((p.detach() - q.detach()).norm() / (q.detach() - w0.to(gpu)).norm()) <= 8e-3
+
+
+def test_muon_step_keeps_the_statement_path_when_something_watches_the_update(gpu, monkeypatch):
+    calls = []
+    real = hip_kernels.fused_muon_update
+    monkeypatch.setattr(hip_kernels, "fused_muon_update", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+
+    class Watching(muon.Muon):
+        def pre_weight_update_fn_inplace(self, p, update):
+            self.seen = update.shape
+
+    for cls, kw in ((Watching, {}), (muon.Muon, {"weight_decay": 0.1, "weight_decay_method": "l2"}),
+                    (muon.Muon, {"fp32_matmul_prec": "highest"})):
+        p = nn.Parameter(torch.randn(64, 128, device=gpu))
+        p.grad = torch.randn_like(p)
+        cls([p], use_syrk=True, **kw).step()
+    assert calls == []
