@@ -35,6 +35,7 @@ M, N, NS_STEPS = 4096, 14336, 5
 WORKLOADS = {
     "mlp": (4096, 14336),          # Llama-3-8B MLP gradient (headline)
     "attn": (4096, 4096),          # Llama-3-8B attention projection
+    "attn_x8": (8, 4096, 4096),    # eight attention projections in one batched call (multi-tensor grouping)
     "mlp_tall": (14336, 4096),     # same MLP weight stored (out, in): exercises the K-strided kernels
     "per_head": (32, 128, 4096),   # 32 heads in one grouped launch
     "moe_shard": (8, 1792, 4096),  # 8 experts, single-GPU shard shape

@@ -30,6 +30,10 @@ struct GemmParams {
   const uint16_t* P;
   const uint16_t* Q;
   int64_t ldp, ldq, p_bs, q_bs;  // leading dims / batch strides in elements
+  // Two-level batch of the operands (fast kernel only): batch entry y reads P at (y / batch_inner) * p_bs +
+  // (y % batch_inner) * p_bs2, likewise Q.  batch_inner <= 1 means the plain one-level batch.
+  int batch_inner;
+  int64_t p_bs2, q_bs2;
   const uint16_t* Cin;           // bf16, indexed like OUT; may be null when beta == 0
   int64_t ldc, c_bs;
   void* Out;                     // bf16 or float32, row-major (M x N)

@@ -88,6 +88,11 @@ using CfgHalfN = FastCfg<256, 2, 4, 64, 2, 1, 128>;
 using CfgSyrk192 = FastCfg<192, 2, 2, 64, 3, MI_SYRK192_KSPLIT>;
 #else
 // 16 x 16 x 32 MFMA variants: one wavefront per SIMD (4 per workgroup), accumulators in 256 / 128 / 144 registers.
+#define MI_HAS_SMALL_CFGS 1
+// Batched small matrices (per-head shapes, 128 rows): GEMM+AXPY tile 128 x 256 (wavefronts of 128 x 64) and a
+// 128 x 128 tile (wavefronts of 64 x 64) for the split-K Gram partials.
+using CfgM128 = FastCfg<128, 1, 4, 64, 2, 1, 256, 16>;
+using CfgT128 = FastCfg<128, 2, 2, 64, 3, 1, 128, 16>;
 using CfgBig = FastCfg<256, 2, 2, 64, 2, 1, 256, 16>;     // wavefronts of 128 x 128
 #ifndef MI_HALFN_NS
 #define MI_HALFN_NS 3
@@ -612,8 +617,14 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
 
   FastLoader<C, P_KS, C::TILE_M, EDGE> lp;
   FastLoader<C, Q_KS, C::TILE_N, EDGE> lq;
-  lp.init(p.P + batch * p.p_bs, p.ldp, m0, p.M, wave, lane);
-  lq.init(p.Q + batch * p.q_bs, p.ldq, n0, p.N, wave, lane);
+  int64_t p_off = batch * p.p_bs, q_off = batch * p.q_bs;
+  if (p.batch_inner > 1) {  // K slices of one matrix as separate batch entries (split-K products)
+    const int64_t outer = batch / p.batch_inner, inner = batch % p.batch_inner;
+    p_off = outer * p.p_bs + inner * p.p_bs2;
+    q_off = outer * p.q_bs + inner * p.q_bs2;
+  }
+  lp.init(p.P + p_off, p.ldp, m0, p.M, wave, lane);
+  lq.init(p.Q + q_off, p.ldq, n0, p.N, wave, lane);
 
   constexpr int MI = C::MI, ACC_N = MI == 32 ? 16 : 4;
   typename AccVec<MI>::type acc[FM][FN];

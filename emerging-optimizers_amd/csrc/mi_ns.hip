@@ -161,6 +161,13 @@ static int launch_class(TileClass tc, const GemmParams& p, int64_t batch, hipStr
     }
     if (p.M % 256 == 0 && p.N % 256 == 0) return launch_fast<CfgBig, P_KS, Q_KS, MODE, OUT_F32>(p, batch, stream);
   }
+#ifdef MI_HAS_SMALL_CFGS
+  if constexpr (MODE == MODE_GEMM && !P_KS && Q_KS) {
+    // short, wide products (per-head shapes): 128 x 256 tiles keep the direct-to-LDS loads and the coalesced epilogue
+    if (k_ok && p.M % 128 == 0 && p.M < 1024 && p.N % 256 == 0 && p.N >= 256)
+      return launch_fast<CfgM128, false, true, MODE, OUT_F32>(p, batch, stream);
+  }
+#endif
   switch (tc) {
     case TILE_BIG:
       return launch_one<256, 256, 64, 2, 2, P_KS, Q_KS, MODE, OUT_F32>(p, batch, stream);
@@ -626,10 +633,82 @@ static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, in
   return MI_OK;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Gram matrices of batched short, wide matrices (per-head shapes: 32 x 128 x 4096).  One 128 x 128 output tile
+// per matrix cannot fill the chip, so the K range is cut into S slices that run as separate batch entries of a
+// plain product (float32 partials), and a second kernel adds the slices in a fixed order, subtracts the
+// diagonal shift and mirrors the lower triangle (bitwise symmetric bf16 result).
+// ---------------------------------------------------------------------------------------------
+// The slice length is fixed (512 columns), so the number of slices -- and with it the order of the float32
+// additions -- depends on the shape of one matrix only: a batched call and per-matrix calls agree bit for bit.
+static int small_gram_splits(int64_t batch, int64_t m, int64_t n) {
+#ifdef MI_HAS_SMALL_CFGS
+  if (m % 128 != 0 || m > 256 || n % 512 != 0 || n < 1024) return 0;
+  const int64_t splits = n / 512;
+  if (batch * splits > 65535) return 0;
+  return (int)splits;
+#else
+  (void)batch; (void)m; (void)n;
+  return 0;
+#endif
+}
+
+__global__ void __launch_bounds__(256) gram_reduce_kernel(const float* __restrict__ partials, int splits, int m,
+                                                          const float* __restrict__ slots_in, int nslots_in,
+                                                          float* __restrict__ shift_io, uint16_t* __restrict__ out) {
+  const int64_t b = blockIdx.y;
+  __shared__ float red[4];
+  // diagonal shift of this matrix: ||X||_F^2 / m from the partial sums the previous kernel left
+  float part = 0.0f;
+  for (int i = threadIdx.x; i < nslots_in; i += 256) part += slots_in[b * nslots_in + i];
+  const float shift = block_sum_f32<256>(part, red) / (float)m;
+  if (blockIdx.x == 0 && threadIdx.x == 0) shift_io[b] = shift;
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= m * m) return;
+  const int i = idx / m, j = idx % m;
+  if (j > i) return;  // the lower triangle is summed, the upper one is its mirror image
+  const float* __restrict__ src = partials + (b * splits) * (int64_t)m * m + idx;
+  float acc = 0.0f;
+  for (int s = 0; s < splits; ++s) acc += src[(int64_t)s * m * m];
+  if (i == j) acc -= shift;
+  const uint16_t h = __builtin_bit_cast(uint16_t, (__bf16)acc);
+  uint16_t* __restrict__ ob = out + b * (int64_t)m * m;
+  ob[(int64_t)i * m + j] = h;
+  ob[(int64_t)j * m + i] = h;
+}
+
+#ifdef MI_HAS_SMALL_CFGS
+static int small_gram(const uint16_t* X, int64_t batch, int64_t m, int64_t n, int splits, float* partials,
+                      const float* slots_in, int nslots_in, float* shift_io, uint16_t* gram, hipStream_t stream) {
+  GemmParams p{};
+  p.P = p.Q = X;
+  p.ldp = p.ldq = n;
+  p.p_bs = p.q_bs = m * n;
+  p.batch_inner = splits;
+  p.p_bs2 = p.q_bs2 = n / splits;
+  p.Out = partials;
+  p.ldo = m;
+  p.o_bs = m * m;
+  p.M = p.N = (int)m;
+  p.K = (int)(n / splits);
+  p.alpha = 1.0f;
+  p.beta = 0.0f;
+  p.out_scale = 1.0f;
+  int rc = launch_fast<CfgT128, false, false, MODE_GEMM, true>(p, batch * splits, stream);
+  if (rc != MI_OK) return rc;
+  dim3 grid((unsigned)((m * m + 255) / 256), (unsigned)batch), block(256);
+  hipLaunchKernelGGL(gram_reduce_kernel, grid, block, 0, stream, partials, splits, (int)m, slots_in, nslots_in, shift_io, gram);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "gram_reduce launch failed: %s", hipGetErrorString(e));
+  return MI_OK;
+}
+#endif
+
 static size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct NsWorkspace {
-  size_t x0, x1, a, b, partials, norm, slots, shift, result, total;
+  size_t x0, x1, a, b, partials, norm, slots, shift, result, gpart, total;
+  int gram_splits;  // > 0: split-K Gram path of short, wide batches
   int64_t max_slots;
 };
 
@@ -653,6 +732,10 @@ static NsWorkspace ns_layout(int64_t batch, int64_t rows, int64_t cols) {
   // final transpose into `out`
   w.result = off;
   if (rows > cols) off += align_up((size_t)batch * rows * cols * sizeof(float), 256);
+  // float32 partial Gram matrices of the split-K path
+  w.gram_splits = small_gram_splits(batch, m, rows < cols ? cols : rows);
+  w.gpart = off;
+  off += align_up((size_t)batch * w.gram_splits * m * m * sizeof(float), 256);
   w.total = off;
   return w;
 }
@@ -718,7 +801,13 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
     ShiftArgs sh_gram{SHIFT_GRAM, b, c, slots, nslots, shift, nullptr};
     {
       ProfScope prof(PROF_GRAM, stream);
-      rc = syrk_impl(xbuf[cur], batch, m, n, x_bs, ld, trans, nullptr, 0, m, 1.0f, 0.0f, gram, g_bs, m, 0, stream, &sh_gram);
+#ifdef MI_HAS_SMALL_CFGS
+      if (w.gram_splits > 0)
+        rc = small_gram(xbuf[cur], batch, m, n, w.gram_splits, reinterpret_cast<float*>(ws + w.gpart), slots, nslots, shift,
+                        gram, stream);
+      else
+#endif
+        rc = syrk_impl(xbuf[cur], batch, m, n, x_bs, ld, trans, nullptr, 0, m, 1.0f, 0.0f, gram, g_bs, m, 0, stream, &sh_gram);
     }
     if (rc != MI_OK) return rc;
     const uint16_t* mult = gram;
