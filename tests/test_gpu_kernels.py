@@ -139,7 +139,8 @@ def test_syrk_config2_shape_properties(gpu):
 
 
 # ---------------------------------------------------------------- GEMM + AXPY
-@pytest.mark.parametrize("b,m,n", [(1, 32, 64), (2, 128, 256), (1, 256, 1024), (1, 1024, 2304), (1, 1024, 16640), (3, 64, 8), (1, 8, 64), (2, 264, 520)])
+@pytest.mark.parametrize("b,m,n", [(1, 32, 64), (2, 128, 256), (1, 256, 1024), (1, 1024, 2304), (1, 1024, 16640), (3, 64, 8), (1, 8, 64), (2, 264, 520),
+                                   (2, 128, 512), (3, 384, 768), (1, 512, 256), (5, 896, 256)])
 @pytest.mark.parametrize("trans", [False, True])
 def test_gemm_axpy_integer_exact(gpu, b, m, n, trans):
     x = _int_bf16((b, n, m) if trans else (b, m, n), -2, 3, gpu)

@@ -45,7 +45,9 @@ def test_tsyrk_step_bit_equal_to_gemm_step_and_oracle(gpu, shape):
 
 
 # ---------------------------------------------------------------- fused driver, small shapes vs the numpy oracle
-@pytest.mark.parametrize("shape", [(256, 512), (512, 256), (64, 64), (8, 16), (3, 128, 384), (2, 384, 128), (1024, 1280)])
+# (4, 128, 1024), (2, 256, 1536) and (1536, 256) take the split-K Gram path of short, wide matrices
+@pytest.mark.parametrize("shape", [(256, 512), (512, 256), (64, 64), (8, 16), (3, 128, 384), (2, 384, 128), (1024, 1280),
+                                   (4, 128, 1024), (2, 256, 1536), (1536, 256)])
 @pytest.mark.parametrize("kind,steps", [("simple", 5), ("quintic", 5), ("cubic5", 5), ("polar_express", 8)])
 def test_fused_matches_oracle(gpu, shape, kind, steps):
     x = torch.randn(*shape)
