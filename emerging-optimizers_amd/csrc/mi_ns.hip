@@ -426,7 +426,20 @@ __global__ void __launch_bounds__(NORM_THREADS) sumsq_kernel(const float* __rest
     total = block_sum<double>((s0 + s1) + (s2 + s3), scratch_d);
   } else {
     float s0 = 0, s1 = 0, s2 = 0, s3 = 0;
-    for (int64_t i = (int64_t)blockIdx.x * NORM_THREADS + threadIdx.x; i < nvec; i += stride) {
+    int64_t i = (int64_t)blockIdx.x * NORM_THREADS + threadIdx.x;
+    // four independent 16-byte loads in flight per lane: a single one leaves HBM latency exposed
+    for (; i + 3 * stride < nvec; i += 4 * stride) {
+      const float4 v0 = fetch(i), v1 = fetch(i + stride), v2 = fetch(i + 2 * stride), v3 = fetch(i + 3 * stride);
+      s0 = __builtin_fmaf(v0.x, v0.x, s0); s1 = __builtin_fmaf(v0.y, v0.y, s1);
+      s2 = __builtin_fmaf(v0.z, v0.z, s2); s3 = __builtin_fmaf(v0.w, v0.w, s3);
+      s0 = __builtin_fmaf(v1.x, v1.x, s0); s1 = __builtin_fmaf(v1.y, v1.y, s1);
+      s2 = __builtin_fmaf(v1.z, v1.z, s2); s3 = __builtin_fmaf(v1.w, v1.w, s3);
+      s0 = __builtin_fmaf(v2.x, v2.x, s0); s1 = __builtin_fmaf(v2.y, v2.y, s1);
+      s2 = __builtin_fmaf(v2.z, v2.z, s2); s3 = __builtin_fmaf(v2.w, v2.w, s3);
+      s0 = __builtin_fmaf(v3.x, v3.x, s0); s1 = __builtin_fmaf(v3.y, v3.y, s1);
+      s2 = __builtin_fmaf(v3.z, v3.z, s2); s3 = __builtin_fmaf(v3.w, v3.w, s3);
+    }
+    for (; i < nvec; i += stride) {
       float4 v = fetch(i);
       s0 = __builtin_fmaf(v.x, v.x, s0);
       s1 = __builtin_fmaf(v.y, v.y, s1);
