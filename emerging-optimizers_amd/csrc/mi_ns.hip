@@ -139,17 +139,39 @@ static int num_cus() {
   return cached;
 }
 
-// SYRK tile of the fast path.  192 x 192 tiles (253 lower-triangle workgroups at 4096 rows: one round on 256 CUs,
-// where 256 x 256 tiles give 136 and leave 47 % of the CUs idle) were at least as fast as 256 x 256 tiles on every
-// shape measured, batched or not, multiples of 256 included (1024 .. 14336 rows, K 1792 .. 14336): the finer
-// granularity wins back more in partial rounds and diagonal tiles than the smaller tile loses in operand reuse.
-static bool syrk_prefers_192(int64_t n, int64_t batch) {
-#ifdef MI_FORCE_SYRK192
-  return MI_FORCE_SYRK192 != 0;  // tuning builds only
+// Tile choice of the fast path by modelled time: rounds of workgroups over the CUs times the cost of one tile.
+// Measured on this part (SYRK n = 1024 .. 4096, batch 1 .. 16, K 1024 .. 14336; GEMM m = 1024 .. 4096):
+//  * SYRK: 192 x 192 tiles (253 lower-triangle workgroups at 4096 rows = one round on 256 CUs) were never slower than
+//    256 x 256 tiles, batched or not; 128 x 128 tiles cost about 1.4x per FLOP but win whenever 192-tiles cannot fill the
+//    chip or waste most of a round (2048 rows: 66 vs 136 workgroups; 2 x 3072 rows: 272 vs 600).
+//  * GEMM: 256 x 128 tiles cost about 1.27x per FLOP of 256 x 256 tiles and win when the latter leave CUs idle
+//    (1024 x 4096: 64 tiles).
+enum SyrkTile { SYRK_TILE_128, SYRK_TILE_192 };
+static SyrkTile pick_syrk_tile(int64_t n, int64_t batch) {
+#if defined(MI_HAS_SMALL_CFGS) && defined(MI_FORCE_SYRK128)
+  if (MI_FORCE_SYRK128) return SYRK_TILE_128;  // tuning builds only
 #endif
-  (void)n;
-  (void)batch;
-  return true;
+#ifdef MI_HAS_SMALL_CFGS
+  const int64_t cus = num_cus();
+  auto rounds = [&](int64_t tile) {
+    const int64_t t = ceil_div(n, tile);
+    return ceil_div(t * (t + 1) / 2 * batch, cus);
+  };
+  const double cost192 = (double)rounds(192) * 192.0 * 192.0;
+  const double cost128 = (double)rounds(128) * 128.0 * 128.0 * 1.4;
+  if (n % 128 == 0 && cost128 < cost192) return SYRK_TILE_128;
+#else
+  (void)n; (void)batch;
+#endif
+  return SYRK_TILE_192;
+}
+// 256 x 128 instead of 256 x 256 GEMM tiles for the whole product?
+static bool gemm_prefers_half_tiles(int64_t m, int64_t n, int64_t batch) {
+#if defined(MI_FORCE_GEMM_HALF)
+  if (MI_FORCE_GEMM_HALF) return true;  // tuning builds only
+#endif
+  const int64_t cus = num_cus(), tiles = (m / 256) * (n / 256) * batch;
+  return (double)ceil_div(2 * tiles, cus) * 0.5 * 1.27 < (double)ceil_div(tiles, cus);
 }
 
 template <bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
@@ -157,7 +179,14 @@ static int launch_class(TileClass tc, const GemmParams& p, int64_t batch, hipStr
   const bool k_ok = p.K % 64 == 0 && p.K >= 64;
   if (k_ok && p.M >= 1024 && p.N >= 1024) {
     if constexpr (MODE == MODE_SYRK && !P_KS && !Q_KS) {
-      if (syrk_prefers_192(p.M, batch)) return launch_fast<CfgSyrk192, false, false, MODE, OUT_F32>(p, batch, stream);
+#ifdef MI_HAS_SMALL_CFGS
+      if (pick_syrk_tile(p.M, batch) == SYRK_TILE_128) return launch_fast<CfgT128, false, false, MODE, OUT_F32>(p, batch, stream);
+#endif
+      return launch_fast<CfgSyrk192, false, false, MODE, OUT_F32>(p, batch, stream);
+    }
+    if constexpr (MODE == MODE_GEMM && !P_KS && Q_KS) {
+      if (p.M % 256 == 0 && p.N % 256 == 0 && gemm_prefers_half_tiles(p.M, p.N, batch))
+        return launch_fast<CfgHalfN, false, true, MODE, OUT_F32>(p, batch, stream);
     }
     if (p.M % 256 == 0 && p.N % 256 == 0) return launch_fast<CfgBig, P_KS, Q_KS, MODE, OUT_F32>(p, batch, stream);
   }
