@@ -31,7 +31,7 @@ PEAK_BF16_TFLOPS = 2516.6  # MI355X dense bf16 MFMA: 256 CU x 2.4 GHz x 4096 FLO
 # of the same run, whose traffic is known (229 376 KiB read, 114 688 KiB written): factors 1.995 and 1.000.
 GEMM_AXPY_TRAFFIC_BYTES = int(((405954.4 + 146826.3) * 1.995 + (98328.0 + 16392.0) * 1.000) * 1024)
 M, N, NS_STEPS = 4096, 14336, 5
-# Other BASELINE configurations, timed with --workload (the default and the graded line is "mlp").
+# Other benchmark configurations, timed with --workload (the default, "mlp", is the headline).
 WORKLOADS = {
     "mlp": (4096, 14336),          # Llama-3-8B MLP gradient (headline)
     "attn": (4096, 4096),          # Llama-3-8B attention projection
@@ -101,7 +101,7 @@ def cpu_baseline(x_cpu):
 
 
 def batched_syrk_workload(args):
-    """BASELINE configuration 2: batched_tsyrk_ex alone on 16 x (2048 x 8192) bf16, TFLOP/s on B n^2 k."""
+    """Batched SYRK configuration: batched_tsyrk_ex alone on 16 x (2048 x 8192) bf16, TFLOP/s on B n^2 k."""
     import torch
 
     from emerging_optimizers import _hip
@@ -171,7 +171,7 @@ def muon_step_workload(args):
 
 
 def side_workload(args):
-    """Times another BASELINE configuration through the same entry point; one JSON line, no roofline legs."""
+    """Times another benchmark configuration through the same entry point; one JSON line, no roofline legs."""
     import torch
 
     if args.workload == "batched_syrk":
@@ -233,7 +233,7 @@ def main():
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-core baseline leg")
-    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="mlp", help="BASELINE configuration to time")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="mlp", help="benchmark configuration to time")
     args = ap.parse_args()
     if args.workload != "mlp":
         return side_workload(args)

@@ -1,16 +1,17 @@
 // Fast path of the bf16 tile engine for the MFMA-bound shapes (K % 64 == 0, no K tail; row edges are
 // allowed and handled by clamped loads plus a guarded epilogue).
 //
-// A variant is described by FastCfg: square workgroup tile, wavefront grid, ring-slot depth BK and number
-// of ring slots.  Global -> LDS goes through the direct-to-LDS load (16 bytes per lane, a wavefront fills
-// 1 KB of LDS at base + 16 * lane); the slots form a ring with one barrier per K tile (see the kernel).
-// Because LDS placement is fixed by the lane id, swizzling is done by choosing which global chunk a
-// lane fetches:
+// A variant is described by FastCfg: workgroup tile (TILE_M x TILE_N), wavefront grid, ring-slot depth BK, number
+// of ring slots and the MFMA shape.  Global -> LDS goes through the direct-to-LDS load (16 bytes per lane, a
+// wavefront fills 1 KB of LDS at base + 16 * lane); the slots form a ring with one barrier per K tile (see the
+// kernel).  Because LDS placement is fixed by the lane id, swizzling is done by choosing which global chunk a lane
+// fetches:
 //   K-contiguous operand: LDS row = 128 B (8 chunks); chunk c of row r sits at slot c ^ ((r >> 1) & 7),
-//     so the 16 rows one quarter-wave reads with ds_read_b128 cover all 64 banks.
-//   K-strided operand: LDS row = one k (256 values = 32 chunks); chunk c of row k sits at slot
-//     (c + 4 k) mod 32; fragments are fetched with the LDS transpose read ds_read_b64_tr_b16, which
-//     returns to lane i of a 16-lane group the four k-values of column i from four consecutive k-rows.
+//     so the 16 rows one pass of a ds_read_b128 reads cover all 64 banks.
+//   K-strided operand: LDS row = one k (ROWS values); chunk c of row k sits at slot (c + ks_rot(k)) mod chunks;
+//     fragments are fetched with the LDS transpose read ds_read_b64_tr_b16, which returns to lane i of a 16-lane
+//     group the four k-values of row i from four consecutive k-rows.
+// tests/test_lds_layout_model.py restates loader and fragment reads on the host and checks them against each other.
 #pragma once
 #include <type_traits>
 #include <utility>

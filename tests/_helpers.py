@@ -1,4 +1,4 @@
-"""Shared test helpers (input generators for the BASELINE configurations, comparison metrics)."""
+"""Shared test helpers (input generators for the benchmark configurations, comparison metrics)."""
 
 import json
 import os

@@ -167,7 +167,7 @@ def test_gpu_torch_reference_is_trustworthy(gpu):
     assert rel_fro(got.cpu(), want) < 1e-5
 
 
-# ---------------------------------------------------------------- BASELINE configurations at full size
+# ---------------------------------------------------------------- benchmark configurations at full size
 def _sv_band(out, lo=0.55, hi=1.25):
     """Singular values of the result via the eigenvalues of the small Gram matrix in float64."""
     y = out.double()
