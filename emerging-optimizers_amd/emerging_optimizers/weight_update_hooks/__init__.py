@@ -1,3 +1,4 @@
 from .base import HookStateT, NoOpWeightUpdateHook, WeightUpdateHook
+from .hyperball import HyperballHook
 
-__all__ = ["HookStateT", "NoOpWeightUpdateHook", "WeightUpdateHook"]
+__all__ = ["HookStateT", "HyperballHook", "NoOpWeightUpdateHook", "WeightUpdateHook"]
