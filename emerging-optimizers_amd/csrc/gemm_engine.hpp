@@ -36,10 +36,12 @@ struct GemmParams {
   int64_t p_bs2, q_bs2;
   const uint16_t* Cin;           // bf16, indexed like OUT; may be null when beta == 0
   int64_t ldc, c_bs;
+  const uint16_t* Cin2;          // SYRK mode, bf16 output: optional second addend, same layout as Cin
   void* Out;                     // bf16 or float32, row-major (M x N)
   int64_t ldo, o_bs;
   int M, N, K;
   float alpha, beta, out_scale;
+  float beta2;                   // coefficient of Cin2
   float out_accum;               // float32 output only: Out = out_accum * Out + out_scale * value (0: plain store)
   int tiles_m, tiles_n;
   int skip_upper;
@@ -48,7 +50,8 @@ struct GemmParams {
   // deviations of the diagonal instead of on its O(1) magnitude; the identity part is folded back into
   // the epilogue scalars of the two kernels that consume A', which keeps the algebra exact for any s.
   int shift_mode;            // SHIFT_*
-  float cb, cc;              // step coefficients b, c (host values)
+  float ca, cb, cc;          // step coefficients a, b, c (host values)
+  float ca2, cb2, cc2;       // SHIFT_PAIR_*: coefficients of the second step of a pair
   const float* slots_in;     // SHIFT_GRAM: per-tile partial sums of squares of X, [batch][nslots_in]
   int nslots_in;
   float* shift_io;           // [batch]: written by SHIFT_GRAM, read by SHIFT_POLY / SHIFT_APPLY
@@ -56,7 +59,19 @@ struct GemmParams {
   int slot_stride, slot_base;  //   at slots_out[batch * slot_stride + slot_base + blockIdx.x]
 };
 
-enum { SHIFT_NONE = 0, SHIFT_GRAM = 1, SHIFT_POLY = 2, SHIFT_APPLY = 3 };
+// Two consecutive steps can share one Gram matrix, because every factor involved is a polynomial of it and
+// they all commute.  With A = s I + D (D stored), step 1 = (a1, b1, c1), step 2 = (a2, b2, c2):
+//   R1 = c1 D^2 + (b1 + 2 c1 s) D                 q1 = e1 I + R1,  e1 = a1 + b1 s + c1 s^2      [SHIFT_POLY]
+//   T  = q1 A   = e1 s I + T',   T'  = R1 D  + e1 D  + s R1                                      [SHIFT_PAIR_T]
+//   A2 = q1 T   = s2 I + D2,     D2  = R1 T' + e1 T' + e1 s R1,    s2 = e1^2 s                   [SHIFT_PAIR_A2]
+//   R2 = c2 D2^2 + (b2 + 2 c2 s2) D2              q2 = e2 I + R2,  e2 = a2 + b2 s2 + c2 s2^2    [SHIFT_PAIR_POLY2]
+//   q2 q1 = e1 e2 I + S,         S   = R2 R1 + e2 R1 + e1 R2                                     [SHIFT_PAIR_Q]
+//   X'' = e1 e2 X + S X                                                                          [SHIFT_PAIR_APPLY]
+// which replaces the second step's X X^T and one of the two B X products by four m x m products.
+enum {
+  SHIFT_NONE = 0, SHIFT_GRAM = 1, SHIFT_POLY = 2, SHIFT_APPLY = 3,
+  SHIFT_PAIR_T = 4, SHIFT_PAIR_A2 = 5, SHIFT_PAIR_POLY2 = 6, SHIFT_PAIR_Q = 7, SHIFT_PAIR_APPLY = 8
+};
 
 // Byte offset of 16-byte chunk `chunk` of row `row` in an LDS tile whose rows hold BK bf16 values.
 // The XOR swizzle spreads the 16 rows that one quarter-wave reads (same chunk, consecutive rows)
@@ -236,9 +251,9 @@ __device__ __forceinline__ float block_sum_f32(float v, float* red) {
   return t;
 }
 
-// Resolves the diagonal shift s for this workgroup and returns the effective (alpha, beta).
+// Resolves the diagonal shift s for this workgroup and the effective coefficients of the addends.
 template <int NT>
-__device__ __forceinline__ float resolve_shift(const GemmParams& p, int64_t batch, float* red, float& beta) {
+__device__ __forceinline__ float resolve_shift(const GemmParams& p, int64_t batch, float* red, float& beta, float& beta2) {
   float s = 0.0f;
   if (p.shift_mode == SHIFT_GRAM) {
     float part = 0.0f;
@@ -252,6 +267,18 @@ __device__ __forceinline__ float resolve_shift(const GemmParams& p, int64_t batc
   } else if (p.shift_mode == SHIFT_APPLY) {
     s = p.shift_io[batch];
     beta = beta + p.cb * s + p.cc * s * s;  // X' = (a + b s + c s^2) X + B' X
+  } else if (p.shift_mode >= SHIFT_PAIR_T) {
+    s = p.shift_io[batch];
+    const float e1 = p.ca + p.cb * s + p.cc * s * s;
+    const float s2 = e1 * e1 * s;
+    const float e2 = p.ca2 + p.cb2 * s2 + p.cc2 * s2 * s2;
+    switch (p.shift_mode) {
+      case SHIFT_PAIR_T: beta = e1; beta2 = s; break;
+      case SHIFT_PAIR_A2: beta = e1; beta2 = e1 * s; break;
+      case SHIFT_PAIR_POLY2: beta = p.cb2 + 2.0f * p.cc2 * s2; break;
+      case SHIFT_PAIR_Q: beta = e2; beta2 = e1; break;
+      default: beta = e1 * e2; break;  // SHIFT_PAIR_APPLY
+    }
   }
   return s;
 }
@@ -263,11 +290,13 @@ __device__ __forceinline__ float resolve_shift(const GemmParams& p, int64_t batc
 template <int MODE, bool OUT_F32, bool GUARD, int FM, int FN, int NT, int MI = 32, class ACC = f32x16_t>
 __device__ __forceinline__ void tile_epilogue(const GemmParams& p, ACC (&acc)[FM][FN], int m_base, int n_base,
                                               int lane, int64_t batch, bool diag, float alpha, float beta, float shift,
-                                              float* red) {
+                                              float* red, float beta2 = 0.0f) {
   constexpr int G = MI == 32 ? 4 : 1;
   const int frow = lane & (MI - 1), fk = lane / MI;
   const uint16_t* __restrict__ Cb = p.Cin ? p.Cin + batch * p.c_bs : nullptr;
   const bool use_c = beta != 0.0f && Cb != nullptr;
+  const uint16_t* __restrict__ Cb2 = (MODE == MODE_SYRK && p.Cin2) ? p.Cin2 + batch * p.c_bs : nullptr;
+  const bool use_c2 = beta2 != 0.0f && Cb2 != nullptr;
   // All Cin pieces are requested before the first store (stores may alias Cin as far as the compiler knows, so
   // loads left between them would each wait out a full memory latency).
   constexpr bool HOIST_C = FM * FN * G * 2 <= 96;  // register budget
@@ -310,6 +339,11 @@ __device__ __forceinline__ void tile_epilogue(const GemmParams& p, ACC (&acc)[FM
           }
 #pragma unroll
           for (int r = 0; r < 4; ++r) v[r] = __builtin_fmaf(beta, c[r], v[r]);
+        }
+        if (use_c2) {
+          const f32x4_t c = load_bf16x4_as_f32(Cb2 + (int64_t)m * p.ldc + n);
+#pragma unroll
+          for (int r = 0; r < 4; ++r) v[r] = __builtin_fmaf(beta2, c[r], v[r]);
         }
         if (MODE == MODE_SYRK && p.shift_mode == SHIFT_GRAM && diag) {
 #pragma unroll
@@ -447,11 +481,11 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_bf16_kernel(GemmParams p) 
     __syncthreads();
   }
 
-  float beta = p.beta;
-  const float shift = resolve_shift<NT>(p, batch, red, beta);
+  float beta = p.beta, beta2 = p.beta2;
+  const float shift = resolve_shift<NT>(p, batch, red, beta, beta2);
   const bool diag = (MODE == MODE_SYRK) && (tm == tn);
   tile_epilogue<MODE, OUT_F32, true, FM, FN, NT>(p, acc, m0 + wm * TM, n0 + wn * TN, lane, batch, diag, p.alpha, beta,
-                                                 shift, red);
+                                                 shift, red, beta2);
 }
 
 }  // namespace mi

@@ -460,7 +460,7 @@ __device__ __forceinline__ void syrk_cin_prefetch(const GemmParams& p, int m0, i
 template <class C, bool GUARD>
 __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename AccVec<C::MI>::type (&acc)[C::FM][C::FN],
                                                   char* lds, int lane, int wm, int wn, int m0, int n0, int64_t batch,
-                                                  bool diag, float alpha, float beta, float shift,
+                                                  bool diag, float alpha, float beta, float beta2, float shift,
                                                   const uint4 (&cin_pre)[SyrkStage<C>::CIN_EARLY ? SyrkStage<C>::NCH : 1]) {
   using S = SyrkStage<C>;
   constexpr int TILE = S::TILE, LDT = S::LDT, MI = C::MI, G = MI == 32 ? 4 : 1, FM = C::FM, FN = C::FN;
@@ -476,16 +476,52 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
   const uint16_t* __restrict__ Cb = p.Cin ? p.Cin + batch * p.c_bs : nullptr;
   const bool use_c = beta != 0.0f && Cb != nullptr;
 
+  const uint16_t* __restrict__ Cb2 = p.Cin2 ? p.Cin2 + batch * p.c_bs : nullptr;
+  const bool use_c2 = beta2 != 0.0f && Cb2 != nullptr;
+
   uint2 val[FM][FN][G];  // finished bf16 quads of this lane
-  // ---- values: alpha * acc (+ beta * Cin) (- shift on the diagonal), rounded to bf16 ----
-#pragma unroll
-  for (int h = 0; h < NPASS; ++h) {
-    if (use_c) {
-      __syncthreads();  // the ring (or the previous pass) is no longer read
+  // ---- values: alpha * acc (+ beta * Cin) (+ beta2 * Cin2) (- shift on the diagonal), rounded to bf16 ----
+  if constexpr (NPASS == 1) {
+    constexpr int h = 0;
+    // the second addend is requested first, so that its latency hides behind the staging of the first
+    uint4 c2[NCH];
+    if (use_c2) {
 #pragma unroll
       for (int it = 0; it < NCH; ++it) {
         const int c = tid + it * C::NT, row = c / CPRW, c8 = c % CPRW;
-        const int m = m0 + h * RP + row, n = n0 + c8 * 8;
+        const int m = m0 + row, n = n0 + c8 * 8;
+        c2[it] = make_uint4(0u, 0u, 0u, 0u);
+        if (!GUARD || (m < p.M && n < p.N)) c2[it] = *reinterpret_cast<const uint4*>(Cb2 + (int64_t)m * p.ldc + n);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+#pragma unroll
+        for (int e = 0; e < 4 * G; ++e) acc[i][j][e] = alpha * acc[i][j][e];
+    // adds coef * (the tile staged in LDS) to this wavefront's accumulators
+    auto add_staged = [&](float coef) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int g = 0; g < G; ++g) {
+            const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
+            const uint2 raw = *reinterpret_cast<const uint2*>(lds + (ml * LDT + nl) * 2);
+            acc[i][j][4 * g + 0] = __builtin_fmaf(coef, __uint_as_float(raw.x << 16), acc[i][j][4 * g + 0]);
+            acc[i][j][4 * g + 1] = __builtin_fmaf(coef, __uint_as_float(raw.x & 0xffff0000u), acc[i][j][4 * g + 1]);
+            acc[i][j][4 * g + 2] = __builtin_fmaf(coef, __uint_as_float(raw.y << 16), acc[i][j][4 * g + 2]);
+            acc[i][j][4 * g + 3] = __builtin_fmaf(coef, __uint_as_float(raw.y & 0xffff0000u), acc[i][j][4 * g + 3]);
+          }
+    };
+    if (use_c) {
+      __syncthreads();  // the ring is no longer read
+#pragma unroll
+      for (int it = 0; it < NCH; ++it) {
+        const int c = tid + it * C::NT, row = c / CPRW, c8 = c % CPRW;
+        const int m = m0 + row, n = n0 + c8 * 8;
         uint4 v = make_uint4(0u, 0u, 0u, 0u);
         if constexpr (S::CIN_EARLY)
           v = cin_pre[it];  // fetched before the K loop
@@ -494,32 +530,83 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
         *reinterpret_cast<uint4*>(lds + (row * LDT + c8 * 8) * 2) = v;
       }
       __syncthreads();
+      add_staged(beta);
     }
-    if (mw / RP == h) {
+    if (use_c2) {
+      __syncthreads();
 #pragma unroll
-      for (int i = 0; i < FM; ++i)
+      for (int it = 0; it < NCH; ++it) {
+        const int c = tid + it * C::NT, row = c / CPRW, c8 = c % CPRW;
+        *reinterpret_cast<uint4*>(lds + (row * LDT + c8 * 8) * 2) = c2[it];
+      }
+      __syncthreads();
+      add_staged(beta2);
+    }
 #pragma unroll
-        for (int j = 0; j < FN; ++j)
+    for (int i = 0; i < FM; ++i)
 #pragma unroll
-          for (int g = 0; g < G; ++g) {
-            const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
-            f32x4_t v;
+      for (int j = 0; j < FN; ++j)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][4 * g + r];
-            if (use_c) {
-              const uint2 raw = *reinterpret_cast<const uint2*>(lds + ((ml - h * RP) * LDT + nl) * 2);
-              v[0] = __builtin_fmaf(beta, __uint_as_float(raw.x << 16), v[0]);
-              v[1] = __builtin_fmaf(beta, __uint_as_float(raw.x & 0xffff0000u), v[1]);
-              v[2] = __builtin_fmaf(beta, __uint_as_float(raw.y << 16), v[2]);
-              v[3] = __builtin_fmaf(beta, __uint_as_float(raw.y & 0xffff0000u), v[3]);
-            }
-            if (p.shift_mode == SHIFT_GRAM && diag) {
+        for (int g = 0; g < G; ++g) {
+          const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
+          f32x4_t v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+          if (p.shift_mode == SHIFT_GRAM && diag) {
 #pragma unroll
-              for (int r = 0; r < 4; ++r)
-                if (nl + r == ml) v[r] -= shift;
-            }
-            val[i][j][g] = __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));
+            for (int r = 0; r < 4; ++r)
+              if (nl + r == ml) v[r] -= shift;
           }
+          val[i][j][g] = __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));
+        }
+    (void)h;
+  } else {
+    // a tile staged in passes: Cin goes through LDS pass by pass, Cin2 (rare here) is read in accumulator layout
+#pragma unroll
+    for (int h = 0; h < NPASS; ++h) {
+      if (use_c) {
+        __syncthreads();  // the ring (or the previous pass) is no longer read
+#pragma unroll
+        for (int it = 0; it < NCH; ++it) {
+          const int c = tid + it * C::NT, row = c / CPRW, c8 = c % CPRW;
+          const int m = m0 + h * RP + row, n = n0 + c8 * 8;
+          uint4 v = make_uint4(0u, 0u, 0u, 0u);
+          if (!GUARD || (m < p.M && n < p.N)) v = *reinterpret_cast<const uint4*>(Cb + (int64_t)m * p.ldc + n);
+          *reinterpret_cast<uint4*>(lds + (row * LDT + c8 * 8) * 2) = v;
+        }
+        __syncthreads();
+      }
+      if (mw / RP == h) {
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+          for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+              const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
+              f32x4_t v;
+#pragma unroll
+              for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][4 * g + r];
+              if (use_c) {
+                const uint2 raw = *reinterpret_cast<const uint2*>(lds + ((ml - h * RP) * LDT + nl) * 2);
+                v[0] = __builtin_fmaf(beta, __uint_as_float(raw.x << 16), v[0]);
+                v[1] = __builtin_fmaf(beta, __uint_as_float(raw.x & 0xffff0000u), v[1]);
+                v[2] = __builtin_fmaf(beta, __uint_as_float(raw.y << 16), v[2]);
+                v[3] = __builtin_fmaf(beta, __uint_as_float(raw.y & 0xffff0000u), v[3]);
+              }
+              if (use_c2 && (!GUARD || (m0 + ml < p.M && n0 + nl < p.N))) {
+                const uint2 raw = *reinterpret_cast<const uint2*>(Cb2 + (int64_t)(m0 + ml) * p.ldc + n0 + nl);
+                v[0] = __builtin_fmaf(beta2, __uint_as_float(raw.x << 16), v[0]);
+                v[1] = __builtin_fmaf(beta2, __uint_as_float(raw.x & 0xffff0000u), v[1]);
+                v[2] = __builtin_fmaf(beta2, __uint_as_float(raw.y << 16), v[2]);
+                v[3] = __builtin_fmaf(beta2, __uint_as_float(raw.y & 0xffff0000u), v[3]);
+              }
+              if (p.shift_mode == SHIFT_GRAM && diag) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                  if (nl + r == ml) v[r] -= shift;
+              }
+              val[i][j][g] = __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));
+            }
+      }
     }
   }
   auto elem = [&](const uint2& q, int r) -> uint16_t {
@@ -887,21 +974,21 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
 #ifdef MI_TIMING
   const long long t_loop = __builtin_readcyclecounter();
 #endif
-  float beta = p.beta;
-  const float shift = resolve_shift<NT>(p, batch, red, beta);
+  float beta = p.beta, beta2 = p.beta2;
+  const float shift = resolve_shift<NT>(p, batch, red, beta, beta2);
   const bool diag = (MODE == MODE_SYRK) && (tm == tn);
   if constexpr (MODE == MODE_GEMM && (C::TN == 32 || C::TN == 64 || C::TN == 128)) {
     __syncthreads();  // every wavefront has finished reading the ring: it can be reused as staging space
     gemm_epilogue_lds<C, OUT_F32, EDGE>(p, acc, &ring[0][0], wave, lane, m0 + wm * C::TM, n0 + wn * C::TN, batch, p.alpha,
                                         beta, red);
   } else if constexpr (SYRK_STAGED) {
-    syrk_epilogue_lds<C, EDGE>(p, acc, &ring[0][0], lane, wm, wn, m0, n0, batch, diag, p.alpha, beta, shift, cin_pre);
+    syrk_epilogue_lds<C, EDGE>(p, acc, &ring[0][0], lane, wm, wn, m0, n0, batch, diag, p.alpha, beta, beta2, shift, cin_pre);
   } else {
     static_assert(C::KSPLIT == 1 || MODE == MODE_SYRK, "the K-group variant is wired for SYRK only");
     // (SYRK never takes the per-workgroup sum at the end of tile_epilogue, so group 1 may simply skip it)
     if (C::KSPLIT == 1 || kgroup == 0)
       tile_epilogue<MODE, OUT_F32, EDGE, FM, FN, NT, MI>(p, acc, m0 + wm * C::TM, n0 + wn * C::TN, lane, batch, diag, p.alpha,
-                                                     beta, shift, red);
+                                                     beta, shift, red, beta2);
   }
 #ifdef MI_TIMING
   if (p.slots_in && lane == 0) {  // debug build only: slots_in doubles as the timing dump

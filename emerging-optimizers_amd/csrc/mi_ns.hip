@@ -215,10 +215,15 @@ struct ShiftArgs {
   int nslots_in;
   float* shift_io;
   float* slots_out;
+  float ca = 0.0f, ca2 = 0.0f, cb2 = 0.0f, cc2 = 0.0f;  // SHIFT_PAIR_*: a of the first step and (a, b, c) of the second
   void apply(GemmParams& p) const {
     p.shift_mode = mode;
+    p.ca = ca;
     p.cb = cb;
     p.cc = cc;
+    p.ca2 = ca2;
+    p.cb2 = cb2;
+    p.cc2 = cc2;
     p.slots_in = slots_in;
     p.nslots_in = nslots_in;
     p.shift_io = shift_io;
@@ -229,9 +234,13 @@ struct ShiftArgs {
 };
 
 // D = alpha * A A^T + beta * C, bf16 out.
+// Inside the fused driver the same lower-triangle kernel also forms products of two commuting symmetric matrices:
+// `other` != null computes alpha * A other^T (symmetric in exact arithmetic; the lower triangle is computed and
+// mirrored), and `C2` is a second addend laid out like C whose coefficient a SHIFT_PAIR_* mode supplies.
 static int syrk_impl(const void* A, int64_t batch, int64_t n, int64_t k, int64_t a_bs, int64_t a_ld, int a_trans,
                      const void* C, int64_t c_bs, int64_t c_ld, float alpha, float beta, void* D, int64_t d_bs,
-                     int64_t d_ld, int skip_upper, hipStream_t stream, const ShiftArgs* sh = nullptr) {
+                     int64_t d_ld, int skip_upper, hipStream_t stream, const ShiftArgs* sh = nullptr,
+                     const void* other = nullptr, const void* C2 = nullptr) {
   if (!A || !D) return fail(MI_ERR_BAD_ARG, "mi_syrk_bf16: A and D must not be null");
   if (batch < 0 || n < 0 || k < 0) return fail(MI_ERR_BAD_ARG, "mi_syrk_bf16: negative extent");
   if (beta != 0.0f && !C) return fail(MI_ERR_BAD_ARG, "mi_syrk_bf16: C is null but beta != 0");
@@ -245,7 +254,10 @@ static int syrk_impl(const void* A, int64_t batch, int64_t n, int64_t k, int64_t
   if (batch == 0 || n == 0) return MI_OK;
 
   GemmParams p{};
-  p.P = p.Q = static_cast<const uint16_t*>(A);
+  p.P = static_cast<const uint16_t*>(A);
+  p.Q = other ? static_cast<const uint16_t*>(other) : p.P;
+  p.Cin2 = static_cast<const uint16_t*>(C2);
+  p.beta2 = C2 ? 1.0f : 0.0f;  // replaced by the shift mode
   p.ldp = p.ldq = a_ld;
   p.p_bs = p.q_bs = a_bs;
   p.Cin = (beta != 0.0f) ? static_cast<const uint16_t*>(C) : nullptr;
@@ -749,10 +761,23 @@ static int small_gram(const uint16_t* X, int64_t batch, int64_t m, int64_t n, in
 static size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct NsWorkspace {
-  size_t x0, x1, a, b, partials, norm, slots, shift, result, gpart, total;
+  size_t x0, x1, a, b, t, d2, partials, norm, slots, shift, result, gpart, total;
   int gram_splits;  // > 0: split-K Gram path of short, wide batches
+  int pairs;        // steps may be taken two at a time on one Gram matrix (two more m x m buffers)
   int64_t max_slots;
 };
+
+// Whether two consecutive steps share one Gram matrix (see SHIFT_PAIR_* in gemm_engine.hpp).  A pair trades one
+// X X^T and one B X (3 m^2 n multiply-adds) for four m x m products, which pays for wide matrices only; a pair on a
+// square matrix would also sit close to the 1e-2 tolerance.  MI_NS_PAIRS=0 switches pairing off, MI_NS_PAIRS=force
+// pairs wherever the kernels allow it (used by the tests to reach the pair kernels with small matrices).
+static int ns_pairs_enabled(int64_t m, int64_t n, int gram_splits) {
+  if (gram_splits > 0) return 0;
+  const char* env = getenv("MI_NS_PAIRS");
+  if (env && env[0] == '0') return 0;
+  if (env && env[0] == 'f') return 1;
+  return m >= 1024 && n >= 2 * m;
+}
 
 static NsWorkspace ns_layout(int64_t batch, int64_t rows, int64_t cols) {
   const int64_t m = rows < cols ? rows : cols;
@@ -764,6 +789,10 @@ static NsWorkspace ns_layout(int64_t batch, int64_t rows, int64_t cols) {
   w.x1 = off; off += xbytes;
   w.a = off; off += gbytes;
   w.b = off; off += gbytes;
+  w.gram_splits = small_gram_splits(batch, m, rows < cols ? cols : rows);
+  w.pairs = ns_pairs_enabled(m, rows < cols ? cols : rows, w.gram_splits);
+  w.t = off; off += w.pairs ? gbytes : 0;
+  w.d2 = off; off += w.pairs ? gbytes : 0;
   w.partials = off; off += align_up((size_t)batch * NORM_MAX_BLOCKS * sizeof(double), 256);
   w.norm = off; off += align_up((size_t)batch * sizeof(float), 256);
   // one float per GEMM workgroup; the smallest tile class (64 x 64) bounds the count
@@ -775,7 +804,6 @@ static NsWorkspace ns_layout(int64_t batch, int64_t rows, int64_t cols) {
   w.result = off;
   if (rows > cols) off += align_up((size_t)batch * rows * cols * sizeof(float), 256);
   // float32 partial Gram matrices of the split-K path
-  w.gram_splits = small_gram_splits(batch, m, rows < cols ? cols : rows);
   w.gpart = off;
   off += align_up((size_t)batch * w.gram_splits * m * m * sizeof(float), 256);
   w.total = off;
@@ -836,9 +864,13 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
 
   int cur = 0;
   int nslots = 1;  // the normalisation kernel left one value per matrix
-  for (int s = 0; s < steps; ++s) {
+  bool want_pair = true;  // pairs alternate with single steps: two pairs in a row lose accuracy on flat spectra
+  for (int s = 0; s < steps;) {
     const float a = abc[3 * s], b = abc[3 * s + 1], c = abc[3 * s + 2];
-    const bool last = (s + 1 == steps);
+    const bool pair = w.pairs && want_pair && s + 1 < steps && c != 0.0f && abc[3 * s + 5] != 0.0f;
+    const int taken = pair ? 2 : 1;
+    const bool last = (s + taken == steps);
+    want_pair = !pair;
     // A' = X X^T - s I  (s = ||X||_F^2 / m from the partial sums the previous kernel left)
     ShiftArgs sh_gram{SHIFT_GRAM, b, c, slots, nslots, shift, nullptr};
     {
@@ -865,18 +897,45 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
       mult = poly;
       alpha = 1.0f;
     }
-    // X' = (a + b s + c s^2) X + B' X      (cubic: (a + b s) X + b A' X)
+    int apply_mode = SHIFT_APPLY;
+    float a2 = 0.0f, b2 = 0.0f, c2 = 0.0f;
+    if (pair) {
+      // The second step on the same Gram matrix: four products of commuting symmetric m x m matrices (the host
+      // coefficient 1 of each addend is replaced on the device, where the shift is known).
+      a2 = abc[3 * s + 3], b2 = abc[3 * s + 4], c2 = abc[3 * s + 5];
+      uint16_t* tbuf = reinterpret_cast<uint16_t*>(ws + w.t);
+      uint16_t* d2 = reinterpret_cast<uint16_t*>(ws + w.d2);
+      auto product = [&](int mode, const uint16_t* left, const uint16_t* right, const uint16_t* add2, float al, float be,
+                         uint16_t* dst) {
+        ShiftArgs sh{mode, b, c, nullptr, 0, shift, nullptr, a, a2, b2, c2};
+        ProfScope prof(PROF_POLY, stream);
+        return syrk_impl(left, batch, m, m, g_bs, m, 0, right, g_bs, m, al, be, dst, g_bs, m, 0, stream, &sh,
+                         right == left ? nullptr : right, add2);
+      };
+      // T' = R1 D + e1 D + s R1
+      if ((rc = product(SHIFT_PAIR_T, poly, gram, poly, 1.0f, 1.0f, tbuf)) != MI_OK) return rc;
+      // D2 = R1 T' + e1 T' + e1 s R1
+      if ((rc = product(SHIFT_PAIR_A2, poly, tbuf, poly, 1.0f, 1.0f, d2)) != MI_OK) return rc;
+      // R2 = c2 D2^2 + (b2 + 2 c2 s2) D2     (D is no longer needed: its buffer takes R2)
+      if ((rc = product(SHIFT_PAIR_POLY2, d2, d2, nullptr, c2, b2, gram)) != MI_OK) return rc;
+      // S = R2 R1 + e2 R1 + e1 R2            (T' is no longer needed)
+      if ((rc = product(SHIFT_PAIR_Q, gram, poly, gram, 1.0f, 1.0f, tbuf)) != MI_OK) return rc;
+      mult = tbuf;
+      apply_mode = SHIFT_PAIR_APPLY;
+    }
+    // X' = (a + b s + c s^2) X + B' X      (cubic: (a + b s) X + b A' X;  pair: e1 e2 X + S X)
     void* dst = last ? static_cast<void*>(result) : static_cast<void*>(xbuf[cur ^ 1]);
-    ShiftArgs sh_apply{SHIFT_APPLY, b, c, nullptr, 0, shift, last ? nullptr : slots};
+    ShiftArgs sh_apply{apply_mode, b, c, nullptr, 0, shift, last ? nullptr : slots, a, a2, b2, c2};
     {
       ProfScope prof(PROF_APPLY, stream);
-      rc = gemm_axpy_impl(mult, g_bs, m, xbuf[cur], x_bs, ld, trans, dst, x_bs, ld, batch, m, n, alpha, a,
+      rc = gemm_axpy_impl(mult, g_bs, m, xbuf[cur], x_bs, ld, trans, dst, x_bs, ld, batch, m, n, alpha, pair ? 1.0f : a,
                           last ? 1 : 0, last ? out_scale : 1.0f, stream, &sh_apply, (last && !tall) ? out_accum : 0.0f);
     }
     if (rc != MI_OK) return rc;
     nslots = g_last_tiles;
     if (nslots > w.max_slots) return fail(MI_ERR_WORKSPACE, "internal: %d partial-sum slots exceed the %lld reserved", nslots, (long long)w.max_slots);
     cur ^= 1;
+    s += taken;
   }
   if (tall) {
     ProfScope prof(PROF_NORMALIZE, stream);

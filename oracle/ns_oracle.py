@@ -221,6 +221,26 @@ def newton_schulz(
     return _mT(X) if transpose else X
 
 
+def pair_schedule(coeffs: Sequence[tuple[float, float, float]], pairs: bool) -> list[int]:
+    """Group sizes of the single-call GPU driver: 2 = two steps on one Gram matrix, 1 = an ordinary step.
+
+    Pairs alternate with single steps, starting with a pair; a pair needs quintic coefficients (c != 0) in both
+    of its steps.  ``pairs=False`` gives all ones.
+    """
+    groups, s, want_pair = [], 0, True
+    while s < len(coeffs):
+        pair = pairs and want_pair and s + 1 < len(coeffs) and coeffs[s][2] != 0.0 and coeffs[s + 1][2] != 0.0
+        groups.append(2 if pair else 1)
+        s += groups[-1]
+        want_pair = not pair
+    return groups
+
+
+def _mirror_lower(mat: np.ndarray) -> np.ndarray:
+    """What the lower-triangle kernels store: the computed lower triangle and its mirror image."""
+    return np.tril(mat) + _mT(np.tril(mat, -1))
+
+
 def newton_schulz_shifted_bf16(
     x: np.ndarray,
     steps: int,
@@ -228,6 +248,7 @@ def newton_schulz_shifted_bf16(
     custom_coefficient_sets=None,
     eps: float = 1e-15,
     normalize_in_double: bool = False,
+    pairs: bool | None = None,
 ) -> np.ndarray:
     """CPU model of the rounding schedule of the single-call GPU driver (``mi_newton_schulz_bf16``).
 
@@ -237,6 +258,14 @@ def newton_schulz_shifted_bf16(
     with s = ||X||_F^2 / m instead and folds the identity part into the epilogue scalars
         B' = c A'^2 + (b + 2 c s) A',      X' = (a + b s + c s^2) X + B' X,
     which is algebraically the same iteration for any s.  The last step is written to float32 unrounded.
+
+    For wide matrices (m >= 1024, n >= 2 m; ``pairs`` overrides the rule) the driver takes steps two at a time
+    on one Gram matrix (see :func:`pair_schedule`).  All factors are polynomials of A and commute, so with
+    q1 = e1 I + R1 (R1 = B' of the first step, e1 = a1 + b1 s + c1 s^2):
+        A2 = q1^2 A = s2 I + D2,  T' = R1 A' + e1 A' + s R1,  D2 = R1 T' + e1 T' + e1 s R1,  s2 = e1^2 s,
+        R2 = c2 D2^2 + (b2 + 2 c2 s2) D2,  e2 = a2 + b2 s2 + c2 s2^2,
+        X'' = e1 e2 X + S X,  S = R2 R1 + e2 R1 + e1 R2,
+    each m x m product computed on its lower triangle, mirrored and rounded to bf16.
     This function reproduces those rounding points so that GPU results can be compared tightly.
     """
     x = np.asarray(x)
@@ -246,21 +275,37 @@ def newton_schulz_shifted_bf16(
     if transpose:
         x = _mT(x)
     X = round_to_bf16(frobenius_normalize(x, eps, normalize_in_double))
-    m = X.shape[-2]
+    m, n = X.shape[-2:]
     f = np.float32
     sumsq = np.ones(X.shape[:-2] + (1, 1), dtype=np.float32)
     coeffs = expand_coefficients(steps, coefficient_type, custom_coefficient_sets)
+    if pairs is None:
+        pairs = m >= 1024 and n >= 2 * m
     eye = np.eye(m, dtype=np.float32)
-    for i, (a, b, c) in enumerate(coeffs):
+    done = 0
+    for group in pair_schedule(coeffs, pairs):
+        a, b, c = (f(v) for v in coeffs[done])
         s = sumsq / f(m)
         gram = round_to_bf16(np.matmul(X, _mT(X)) - s * eye)
-        if c != 0.0:
-            poly = round_to_bf16(f(c) * np.matmul(gram, gram) + (f(b) + f(2.0) * f(c) * s) * gram)
-            Xn = (f(a) + f(b) * s + f(c) * s * s) * X + np.matmul(poly, X)
+        if group == 2:
+            a2, b2, c2 = (f(v) for v in coeffs[done + 1])
+            r1 = round_to_bf16(c * np.matmul(gram, gram) + (b + f(2.0) * c * s) * gram)
+            e1 = a + b * s + c * s * s
+            t = round_to_bf16(_mirror_lower(np.matmul(r1, gram) + e1 * gram + s * r1))
+            d2 = round_to_bf16(_mirror_lower(np.matmul(r1, t) + e1 * t + (e1 * s) * r1))
+            s2 = e1 * e1 * s
+            r2 = round_to_bf16(c2 * np.matmul(d2, d2) + (b2 + f(2.0) * c2 * s2) * d2)
+            e2 = a2 + b2 * s2 + c2 * s2 * s2
+            q = round_to_bf16(_mirror_lower(np.matmul(r2, r1) + e2 * r1 + e1 * r2))
+            Xn = (e1 * e2) * X + np.matmul(q, X)
+        elif c != 0.0:
+            poly = round_to_bf16(c * np.matmul(gram, gram) + (b + f(2.0) * c * s) * gram)
+            Xn = (a + b * s + c * s * s) * X + np.matmul(poly, X)
         else:
-            Xn = (f(a) + f(b) * s) * X + f(b) * np.matmul(gram, X)
+            Xn = (a + b * s) * X + b * np.matmul(gram, X)
+        done += group
         sumsq = np.sum(Xn * Xn, axis=(-2, -1), keepdims=True, dtype=np.float32)
-        X = Xn if i + 1 == len(coeffs) else round_to_bf16(Xn)
+        X = Xn if done == len(coeffs) else round_to_bf16(Xn)
     X = X.astype(np.float32)
     return _mT(X) if transpose else X
 

@@ -68,6 +68,53 @@ def test_fused_matches_oracle(gpu, shape, kind, steps):
     assert rel_fro(got.cpu(), want32) <= rel_fro(ref_sched, want32) + 1e-3
 
 
+@pytest.fixture
+def forced_pairs(monkeypatch):
+    """Makes the driver take steps two at a time on one Gram matrix wherever its kernels allow it (by itself it
+    does so only for matrices with at least 1024 rows and twice as many columns)."""
+    monkeypatch.setenv("MI_NS_PAIRS", "force")
+
+
+# (1024, 2048) and (2, 1024, 2304) pair up by the driver's own rule (no override needed)
+@pytest.mark.parametrize("shape", [(256, 512), (512, 256), (64, 64), (8, 16), (3, 128, 384), (200, 456), (1024, 1280),
+                                   (1024, 2048), (2, 1024, 2304)])
+@pytest.mark.parametrize("kind,steps", [("simple", 5), ("quintic", 5), ("quintic", 4), ("cubic5", 5), ("polar_express", 8)])
+def test_paired_steps_match_oracle(gpu, forced_pairs, shape, kind, steps):
+    x = torch.randn(*shape)
+    with utils.fp32_matmul_precision("medium"):
+        got = muon_utils.newton_schulz(x.to(gpu), steps=steps, coefficient_type=kind, use_syrk=True)
+    want32 = O.newton_schulz(x.numpy(), steps, kind)
+    tol = TOL_FP32 if min(shape[-2:]) >= 64 else 3e-2
+    near_square = max(shape[-2:]) < 2 * min(shape[-2:])
+    if near_square:
+        tol = max(tol, 1.3e-2)  # outside the driver's own rule: pairs cost accuracy there
+    assert rel_fro(got.cpu(), want32) <= tol
+    model = O.newton_schulz_shifted_bf16(x.numpy(), steps, kind, pairs=True)
+    # (a nearly square random matrix has singular values close to zero, which amplify every flipped rounding)
+    assert rel_fro(got.cpu(), model) <= (2.5e-3 if near_square else 1e-3) * steps + 1e-3
+    if kind != "cubic5":  # cubic steps never pair: the override must then change nothing, else it must
+        single = O.newton_schulz_shifted_bf16(x.numpy(), steps, kind, pairs=False)
+        assert rel_fro(model, single) > 1e-5
+
+
+def test_pair_rule_by_shape(gpu, monkeypatch):
+    """Wide matrices pair up by default, MI_NS_PAIRS=0 switches that off; both stay within tolerance."""
+    x = torch.randn(1024, 2560)
+    want32 = O.newton_schulz(x.numpy(), 5, "quintic")
+    outs = {}
+    for env in (None, "0"):
+        if env is None:
+            monkeypatch.delenv("MI_NS_PAIRS", raising=False)
+        else:
+            monkeypatch.setenv("MI_NS_PAIRS", env)
+        with utils.fp32_matmul_precision("medium"):
+            outs[env] = muon_utils.newton_schulz(x.to(gpu), steps=5, coefficient_type="quintic", use_syrk=True).cpu()
+        assert rel_fro(outs[env], want32) <= TOL_FP32
+    assert rel_fro(outs[None], O.newton_schulz_shifted_bf16(x.numpy(), 5, "quintic", pairs=True)) <= 6e-3
+    assert rel_fro(outs["0"], O.newton_schulz_shifted_bf16(x.numpy(), 5, "quintic", pairs=False)) <= 6e-3
+    assert not torch.equal(outs[None], outs["0"])
+
+
 def test_fused_known_answers(gpu):
     for case, x, want in known_answer_cases():
         with utils.fp32_matmul_precision("medium"):

@@ -217,6 +217,22 @@ def test_shifted_schedule_model_is_the_same_iteration():
     finally:
         O.round_to_bf16 = saved
     np.testing.assert_allclose(exact, O.newton_schulz(x, 5, "simple"), atol=3e-6)
+    # the same for steps taken two at a time on one Gram matrix (pairs of commuting polynomials)
+    assert O.pair_schedule([(1, 1, 1)] * 5, True) == [2, 1, 2] and O.pair_schedule([(1, 1, 1)] * 8, True) == [2, 1, 2, 1, 2]
+    assert O.pair_schedule([(1, 1, 1)] * 4, True) == [2, 1, 1] and O.pair_schedule([(1, 1, 0)] * 3, True) == [1, 1, 1]
+    assert O.pair_schedule([(1, 1, 1)] * 5, False) == [1] * 5
+    wide = rng.standard_normal((64, 256)).astype(np.float32)
+    for kind, steps in (("simple", 5), ("quintic", 5), ("polar_express", 8), ("cubic5", 5)):
+        try:
+            O.round_to_bf16 = lambda v: np.asarray(v, dtype=np.float32)
+            exact = O.newton_schulz_shifted_bf16(wide, steps, kind, pairs=True)
+        finally:
+            O.round_to_bf16 = saved
+        np.testing.assert_allclose(exact, O.newton_schulz(wide, steps, kind), atol=2e-5)
+        hi = O.newton_schulz(wide, steps, kind, compute_dtype=np.float64)
+        e_pair = np.linalg.norm(O.newton_schulz_shifted_bf16(wide, steps, kind, pairs=True) - hi) / np.linalg.norm(hi)
+        e_single = np.linalg.norm(O.newton_schulz_shifted_bf16(wide, steps, kind, pairs=False) - hi) / np.linalg.norm(hi)
+        assert e_pair < 8e-3 and e_pair < e_single + 1e-3, (kind, e_pair, e_single)
     # scalar known answers: no worse than the reference's bf16 schedule (tiny matrices with singular values
     # spread over 2^-6 .. 1 are hard for any bf16 schedule, hence the comparison instead of a fixed bound)
     fro = lambda g, w: np.linalg.norm(g - w) / np.linalg.norm(w)
