@@ -55,6 +55,9 @@ struct GemmParams {
   const float* slots_in;     // SHIFT_GRAM: per-tile partial sums of squares of X, [batch][nslots_in]
   int nslots_in;
   float* shift_io;           // [batch]: written by SHIFT_GRAM, read by SHIFT_POLY / SHIFT_APPLY
+  // Fused driver, first group of steps only: X is held unnormalised (bf16 of the input) and xscale[batch] =
+  // 1 / ||x||_F is applied where X enters a product: squared in SHIFT_GRAM, once in the apply modes.  Null: 1.
+  const float* xscale;
   float* slots_out;          // GEMM mode: per-workgroup sum of squares of the output,
   int slot_stride, slot_base;  //   at slots_out[batch * slot_stride + slot_base + blockIdx.x]
 };
@@ -253,7 +256,8 @@ __device__ __forceinline__ float block_sum_f32(float v, float* red) {
 
 // Resolves the diagonal shift s for this workgroup and the effective coefficients of the addends.
 template <int NT>
-__device__ __forceinline__ float resolve_shift(const GemmParams& p, int64_t batch, float* red, float& beta, float& beta2) {
+__device__ __forceinline__ float resolve_shift(const GemmParams& p, int64_t batch, float* red, float& alpha, float& beta,
+                                               float& beta2) {
   float s = 0.0f;
   if (p.shift_mode == SHIFT_GRAM) {
     float part = 0.0f;
@@ -278,6 +282,15 @@ __device__ __forceinline__ float resolve_shift(const GemmParams& p, int64_t batc
       case SHIFT_PAIR_POLY2: beta = p.cb2 + 2.0f * p.cc2 * s2; break;
       case SHIFT_PAIR_Q: beta = e2; beta2 = e1; break;
       default: beta = e1 * e2; break;  // SHIFT_PAIR_APPLY
+    }
+  }
+  if (p.xscale != nullptr) {
+    const float r = p.xscale[batch];
+    if (p.shift_mode == SHIFT_GRAM) {
+      alpha *= r * r;
+    } else {
+      alpha *= r;
+      beta *= r;
     }
   }
   return s;
@@ -481,10 +494,10 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_bf16_kernel(GemmParams p) 
     __syncthreads();
   }
 
-  float beta = p.beta, beta2 = p.beta2;
-  const float shift = resolve_shift<NT>(p, batch, red, beta, beta2);
+  float alpha = p.alpha, beta = p.beta, beta2 = p.beta2;
+  const float shift = resolve_shift<NT>(p, batch, red, alpha, beta, beta2);
   const bool diag = (MODE == MODE_SYRK) && (tm == tn);
-  tile_epilogue<MODE, OUT_F32, true, FM, FN, NT>(p, acc, m0 + wm * TM, n0 + wn * TN, lane, batch, diag, p.alpha, beta,
+  tile_epilogue<MODE, OUT_F32, true, FM, FN, NT>(p, acc, m0 + wm * TM, n0 + wn * TN, lane, batch, diag, alpha, beta,
                                                  shift, red, beta2);
 }
 

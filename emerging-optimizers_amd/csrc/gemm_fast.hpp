@@ -974,20 +974,20 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
 #ifdef MI_TIMING
   const long long t_loop = __builtin_readcyclecounter();
 #endif
-  float beta = p.beta, beta2 = p.beta2;
-  const float shift = resolve_shift<NT>(p, batch, red, beta, beta2);
+  float alpha = p.alpha, beta = p.beta, beta2 = p.beta2;
+  const float shift = resolve_shift<NT>(p, batch, red, alpha, beta, beta2);
   const bool diag = (MODE == MODE_SYRK) && (tm == tn);
   if constexpr (MODE == MODE_GEMM && (C::TN == 32 || C::TN == 64 || C::TN == 128)) {
     __syncthreads();  // every wavefront has finished reading the ring: it can be reused as staging space
-    gemm_epilogue_lds<C, OUT_F32, EDGE>(p, acc, &ring[0][0], wave, lane, m0 + wm * C::TM, n0 + wn * C::TN, batch, p.alpha,
+    gemm_epilogue_lds<C, OUT_F32, EDGE>(p, acc, &ring[0][0], wave, lane, m0 + wm * C::TM, n0 + wn * C::TN, batch, alpha,
                                         beta, red);
   } else if constexpr (SYRK_STAGED) {
-    syrk_epilogue_lds<C, EDGE>(p, acc, &ring[0][0], lane, wm, wn, m0, n0, batch, diag, p.alpha, beta, beta2, shift, cin_pre);
+    syrk_epilogue_lds<C, EDGE>(p, acc, &ring[0][0], lane, wm, wn, m0, n0, batch, diag, alpha, beta, beta2, shift, cin_pre);
   } else {
     static_assert(C::KSPLIT == 1 || MODE == MODE_SYRK, "the K-group variant is wired for SYRK only");
     // (SYRK never takes the per-workgroup sum at the end of tile_epilogue, so group 1 may simply skip it)
     if (C::KSPLIT == 1 || kgroup == 0)
-      tile_epilogue<MODE, OUT_F32, EDGE, FM, FN, NT, MI>(p, acc, m0 + wm * C::TM, n0 + wn * C::TN, lane, batch, diag, p.alpha,
+      tile_epilogue<MODE, OUT_F32, EDGE, FM, FN, NT, MI>(p, acc, m0 + wm * C::TM, n0 + wn * C::TN, lane, batch, diag, alpha,
                                                      beta, shift, red, beta2);
   }
 #ifdef MI_TIMING

@@ -216,8 +216,10 @@ struct ShiftArgs {
   float* shift_io;
   float* slots_out;
   float ca = 0.0f, ca2 = 0.0f, cb2 = 0.0f, cc2 = 0.0f;  // SHIFT_PAIR_*: a of the first step and (a, b, c) of the second
+  const float* xscale = nullptr;  // first group of steps on an unnormalised X
   void apply(GemmParams& p) const {
     p.shift_mode = mode;
+    p.xscale = xscale;
     p.ca = ca;
     p.cb = cb;
     p.cc = cc;
@@ -378,6 +380,8 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
 // ---------------------------------------------------------------------------------------------
 static constexpr int NORM_THREADS = 256;
 static constexpr int NORM_MAX_BLOCKS = 1024;  // partials per matrix
+// Frobenius norms in this range let the divide be deferred to the consumers of X (see scale_cast_kernel).
+static constexpr float NORM_DEFER_MIN = 1e-10f, NORM_DEFER_MAX = 1e10f;
 
 static int norm_blocks(int64_t numel) {
   int64_t vec = numel / 4;  // float4 units
@@ -428,10 +432,14 @@ __device__ __forceinline__ float momentum_direction(float g, float buf_new, floa
   return nesterov ? torch_lerp(g, buf_new, beta) : buf_new;
 }
 
+// `raw_out` != null: the values that are summed are also written out as bf16, unnormalised (bf16 has the exponent
+// range of float32, so this loses nothing that the later divide would keep).
 template <bool F64>
 __global__ void __launch_bounds__(NORM_THREADS) sumsq_kernel(const float* __restrict__ x, int64_t numel,
-                                                             double* __restrict__ partials, MomentumSrc mom) {
+                                                             double* __restrict__ partials, MomentumSrc mom,
+                                                             uint16_t* __restrict__ raw_out) {
   const int64_t b = blockIdx.y;
+  uint2* __restrict__ rv = raw_out ? reinterpret_cast<uint2*>(raw_out + b * numel) : nullptr;
   const float4* __restrict__ xv = reinterpret_cast<const float4*>(x + b * numel);
   float4* __restrict__ bv = mom.buf ? reinterpret_cast<float4*>(mom.buf + b * numel) : nullptr;
   const int64_t nvec = numel / 4;
@@ -449,6 +457,10 @@ __global__ void __launch_bounds__(NORM_THREADS) sumsq_kernel(const float* __rest
       v.y = momentum_direction(v.y, m.y, mom.beta, mom.nesterov);
       v.z = momentum_direction(v.z, m.z, mom.beta, mom.nesterov);
       v.w = momentum_direction(v.w, m.w, mom.beta, mom.nesterov);
+    }
+    if (rv) {
+      const f32x4_t f = {v.x, v.y, v.z, v.w};
+      rv[i] = __builtin_bit_cast(uint2, __builtin_convertvector(f, bf16x4_t));
     }
     return v;
   };
@@ -499,7 +511,8 @@ __global__ void __launch_bounds__(NORM_THREADS) scale_cast_kernel(const float* _
                                                                   const double* __restrict__ partials, int nparts,
                                                                   float eps, float post_scale, void* __restrict__ out,
                                                                   float* __restrict__ dev_norm,
-                                                                  float* __restrict__ sumsq_out, MomentumSrc mom) {
+                                                                  float* __restrict__ sumsq_out, MomentumSrc mom,
+                                                                  float* __restrict__ xscale) {
   const int64_t b = blockIdx.y;
   __shared__ double scratch_d[NORM_THREADS / 64];
   double s = 0;
@@ -512,11 +525,20 @@ __global__ void __launch_bounds__(NORM_THREADS) scale_cast_kernel(const float* _
     divisor = fmaxf(sqrtf((float)s), eps);
   }
   if (dev_norm && blockIdx.x == 0 && threadIdx.x == 0) dev_norm[b] = divisor;
+  // `xscale` != null: `out` already holds the unnormalised bf16 values (sumsq_kernel wrote them).  For a norm in
+  // the range where squares of the entries neither overflow nor vanish in float32 the divide is left to the
+  // kernels that consume X (they multiply by xscale) and this pass ends here; otherwise it normalises as usual.
+  bool deferred = false;
+  if (xscale) {
+    deferred = divisor >= NORM_DEFER_MIN && divisor <= NORM_DEFER_MAX;  // false for NaN
+    if (blockIdx.x == 0 && threadIdx.x == 0) xscale[b] = deferred ? 1.0f / divisor : 1.0f;
+  }
   if (sumsq_out && blockIdx.x == 0 && threadIdx.x == 0) {
     // squared Frobenius norm of the normalised matrix: 1 unless the divisor was clamped
     const float ratio = sqrtf((float)s) / divisor;
     sumsq_out[b] = (divisor > 0.0f && ratio == ratio) ? ratio * ratio : 0.0f;
   }
+  if (deferred) return;
 
   const int64_t nvec8 = numel / 8;
   const float4* __restrict__ xv = reinterpret_cast<const float4*>(x + b * numel);
@@ -649,7 +671,7 @@ __global__ void __launch_bounds__(256) transpose_f32_kernel(const float* __restr
 static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, int f64, void* out, int out_bf16,
                      float post_scale, double* partials, float* dev_norm, hipStream_t stream,
                      float* sumsq_out = nullptr, int64_t t_rows = 0, int64_t t_cols = 0,
-                     MomentumSrc mom = MomentumSrc{nullptr, 0.0f, 0}) {
+                     MomentumSrc mom = MomentumSrc{nullptr, 0.0f, 0}, float* xscale = nullptr) {
   if (!x || !out || !partials) return fail(MI_ERR_BAD_ARG, "mi_frob_normalize: null pointer");
   if (batch < 0 || numel < 0) return fail(MI_ERR_BAD_ARG, "mi_frob_normalize: negative extent");
   if (numel % 8) return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_frob_normalize: numel must be a multiple of 8, got %lld", (long long)numel);
@@ -658,10 +680,12 @@ static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, in
   if (batch == 0 || numel == 0) return MI_OK;
   const int nb = norm_blocks(numel);
   dim3 grid1(nb, (unsigned)batch), block(NORM_THREADS);
+  if (xscale && (t_rows > 0 || !out_bf16)) return fail(MI_ERR_BAD_ARG, "internal: deferred normalisation needs a plain bf16 output");
+  uint16_t* raw_out = xscale ? static_cast<uint16_t*>(out) : nullptr;
   if (f64)
-    hipLaunchKernelGGL(sumsq_kernel<true>, grid1, block, 0, stream, x, numel, partials, mom);
+    hipLaunchKernelGGL(sumsq_kernel<true>, grid1, block, 0, stream, x, numel, partials, mom, raw_out);
   else
-    hipLaunchKernelGGL(sumsq_kernel<false>, grid1, block, 0, stream, x, numel, partials, mom);
+    hipLaunchKernelGGL(sumsq_kernel<false>, grid1, block, 0, stream, x, numel, partials, mom, raw_out);
   if (t_rows > 0) {
     // bf16 output transposed to (t_cols x t_rows)
     dim3 gridt((unsigned)((t_cols + 63) / 64), (unsigned)((t_rows + 63) / 64), (unsigned)batch);
@@ -675,7 +699,7 @@ static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, in
   if (want < 1) want = 1;
   if (want > 4096) want = 4096;
   dim3 grid2((unsigned)want, (unsigned)batch);
-#define MI_SC(F, B) hipLaunchKernelGGL((scale_cast_kernel<F, B>), grid2, block, 0, stream, x, numel, partials, nb, eps, post_scale, out, dev_norm, sumsq_out, mom)
+#define MI_SC(F, B) hipLaunchKernelGGL((scale_cast_kernel<F, B>), grid2, block, 0, stream, x, numel, partials, nb, eps, post_scale, out, dev_norm, sumsq_out, mom, xscale)
   if (f64) {
     if (out_bf16) MI_SC(true, true); else MI_SC(true, false);
   } else {
@@ -709,9 +733,11 @@ static int small_gram_splits(int64_t batch, int64_t m, int64_t n) {
 
 __global__ void __launch_bounds__(256) gram_reduce_kernel(const float* __restrict__ partials, int splits, int m,
                                                           const float* __restrict__ slots_in, int nslots_in,
-                                                          float* __restrict__ shift_io, uint16_t* __restrict__ out) {
+                                                          float* __restrict__ shift_io, uint16_t* __restrict__ out,
+                                                          const float* __restrict__ xscale) {
   const int64_t b = blockIdx.y;
   __shared__ float red[4];
+  const float r = xscale ? xscale[b] : 1.0f;
   // diagonal shift of this matrix: ||X||_F^2 / m from the partial sums the previous kernel left
   float part = 0.0f;
   for (int i = threadIdx.x; i < nslots_in; i += 256) part += slots_in[b * nslots_in + i];
@@ -724,6 +750,7 @@ __global__ void __launch_bounds__(256) gram_reduce_kernel(const float* __restric
   const float* __restrict__ src = partials + (b * splits) * (int64_t)m * m + idx;
   float acc = 0.0f;
   for (int s = 0; s < splits; ++s) acc += src[(int64_t)s * m * m];
+  acc *= r * r;
   if (i == j) acc -= shift;
   const uint16_t h = __builtin_bit_cast(uint16_t, (__bf16)acc);
   uint16_t* __restrict__ ob = out + b * (int64_t)m * m;
@@ -733,7 +760,8 @@ __global__ void __launch_bounds__(256) gram_reduce_kernel(const float* __restric
 
 #ifdef MI_HAS_SMALL_CFGS
 static int small_gram(const uint16_t* X, int64_t batch, int64_t m, int64_t n, int splits, float* partials,
-                      const float* slots_in, int nslots_in, float* shift_io, uint16_t* gram, hipStream_t stream) {
+                      const float* slots_in, int nslots_in, float* shift_io, uint16_t* gram, hipStream_t stream,
+                      const float* xscale) {
   GemmParams p{};
   p.P = p.Q = X;
   p.ldp = p.ldq = n;
@@ -751,7 +779,7 @@ static int small_gram(const uint16_t* X, int64_t batch, int64_t m, int64_t n, in
   int rc = launch_fast<CfgT128, false, false, MODE_GEMM, true>(p, batch * splits, stream);
   if (rc != MI_OK) return rc;
   dim3 grid((unsigned)((m * m + 255) / 256), (unsigned)batch), block(256);
-  hipLaunchKernelGGL(gram_reduce_kernel, grid, block, 0, stream, partials, splits, (int)m, slots_in, nslots_in, shift_io, gram);
+  hipLaunchKernelGGL(gram_reduce_kernel, grid, block, 0, stream, partials, splits, (int)m, slots_in, nslots_in, shift_io, gram, xscale);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "gram_reduce launch failed: %s", hipGetErrorString(e));
   return MI_OK;
@@ -761,7 +789,7 @@ static int small_gram(const uint16_t* X, int64_t batch, int64_t m, int64_t n, in
 static size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct NsWorkspace {
-  size_t x0, x1, a, b, t, d2, partials, norm, slots, shift, result, gpart, total;
+  size_t x0, x1, a, b, t, d2, partials, norm, slots, shift, xscale, result, gpart, total;
   int gram_splits;  // > 0: split-K Gram path of short, wide batches
   int pairs;        // steps may be taken two at a time on one Gram matrix (two more m x m buffers)
   int64_t max_slots;
@@ -799,6 +827,7 @@ static NsWorkspace ns_layout(int64_t batch, int64_t rows, int64_t cols) {
   w.max_slots = ((rows + 63) / 64) * ((cols + 63) / 64);
   w.slots = off; off += align_up((size_t)batch * w.max_slots * sizeof(float), 256);
   w.shift = off; off += align_up((size_t)batch * sizeof(float), 256);
+  w.xscale = off; off += align_up((size_t)batch * sizeof(float), 256);
   // tall inputs iterate on the transposed orientation; their float32 result is staged here before the
   // final transpose into `out`
   w.result = off;
@@ -854,11 +883,15 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
   const int64_t ld = n;
   const int64_t x_bs = numel, g_bs = m * m;
   float* result = tall ? reinterpret_cast<float*>(ws + w.result) : out;
+  // A wide (or square) input is cast to bf16 by the pass that sums its squares, and the divide by the norm is
+  // folded into the first Gram product and the first B X product (one pass over the float32 input instead of two).
+  // A tall input needs the transposing second pass anyway.
+  float* xscale = tall ? nullptr : reinterpret_cast<float*>(ws + w.xscale);
   int rc;
   {
     ProfScope prof(PROF_NORMALIZE, stream);
     rc = frob_impl(x, batch, numel, eps, accumulate_fp64, xbuf[0], /*out_bf16=*/1, 1.0f, partials, norm, stream, slots,
-                   tall ? rows : 0, tall ? cols : 0, mom);
+                   tall ? rows : 0, tall ? cols : 0, mom, xscale);
   }
   if (rc != MI_OK) return rc;
 
@@ -873,12 +906,14 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
     want_pair = !pair;
     // A' = X X^T - s I  (s = ||X||_F^2 / m from the partial sums the previous kernel left)
     ShiftArgs sh_gram{SHIFT_GRAM, b, c, slots, nslots, shift, nullptr};
+    const float* xs = (s == 0) ? xscale : nullptr;  // only the input of the first group is unnormalised
+    sh_gram.xscale = xs;
     {
       ProfScope prof(PROF_GRAM, stream);
 #ifdef MI_HAS_SMALL_CFGS
       if (w.gram_splits > 0)
         rc = small_gram(xbuf[cur], batch, m, n, w.gram_splits, reinterpret_cast<float*>(ws + w.gpart), slots, nslots, shift,
-                        gram, stream);
+                        gram, stream, xs);
       else
 #endif
         rc = syrk_impl(xbuf[cur], batch, m, n, x_bs, ld, trans, nullptr, 0, m, 1.0f, 0.0f, gram, g_bs, m, 0, stream, &sh_gram);
@@ -926,6 +961,7 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
     // X' = (a + b s + c s^2) X + B' X      (cubic: (a + b s) X + b A' X;  pair: e1 e2 X + S X)
     void* dst = last ? static_cast<void*>(result) : static_cast<void*>(xbuf[cur ^ 1]);
     ShiftArgs sh_apply{apply_mode, b, c, nullptr, 0, shift, last ? nullptr : slots, a, a2, b2, c2};
+    sh_apply.xscale = xs;
     {
       ProfScope prof(PROF_APPLY, stream);
       rc = gemm_axpy_impl(mult, g_bs, m, xbuf[cur], x_bs, ld, trans, dst, x_bs, ld, batch, m, n, alpha, pair ? 1.0f : a,

@@ -258,6 +258,8 @@ def newton_schulz_shifted_bf16(
     with s = ||X||_F^2 / m instead and folds the identity part into the epilogue scalars
         B' = c A'^2 + (b + 2 c s) A',      X' = (a + b s + c s^2) X + B' X,
     which is algebraically the same iteration for any s.  The last step is written to float32 unrounded.
+    Inputs that are not tall are rounded to bf16 before the division by the norm, which then enters the first
+    products as a scalar (one pass over the float32 input instead of two).
 
     For wide matrices (m >= 1024, n >= 2 m; ``pairs`` overrides the rule) the driver takes steps two at a time
     on one Gram matrix (see :func:`pair_schedule`).  All factors are polynomials of A and commute, so with
@@ -274,11 +276,25 @@ def newton_schulz_shifted_bf16(
     transpose = x.shape[-2] > x.shape[-1]
     if transpose:
         x = _mT(x)
-    X = round_to_bf16(frobenius_normalize(x, eps, normalize_in_double))
-    m, n = X.shape[-2:]
     f = np.float32
-    sumsq = np.ones(X.shape[:-2] + (1, 1), dtype=np.float32)
+    m, n = x.shape[-2:]
     coeffs = expand_coefficients(steps, coefficient_type, custom_coefficient_sets)
+    # A wide or square input is cast to bf16 unnormalised and 1 / ||x||_F enters the first group's products
+    # (r^2 in the Gram matrix, r in X' = ... ); a tall one is normalised before the cast.  The deferral is limited
+    # to norms whose squares are safe in float32.
+    if normalize_in_double:
+        norm = np.sqrt(np.sum(x.astype(np.float64) ** 2, axis=(-2, -1), keepdims=True)).astype(np.float32)
+    else:
+        norm = np.maximum(np.sqrt(np.sum(x * x, axis=(-2, -1), keepdims=True, dtype=np.float32)), f(eps))
+    deferred = (not transpose) and len(coeffs) > 0 and bool(np.all((norm >= f(1e-10)) & (norm <= f(1e10))))
+    if deferred:
+        X = round_to_bf16(x)
+        r = f(1.0) / norm
+        sumsq = (np.sqrt(np.sum(x * x, axis=(-2, -1), keepdims=True, dtype=np.float32)) / norm) ** 2
+    else:
+        X = round_to_bf16(frobenius_normalize(x, eps, normalize_in_double))
+        r = np.ones_like(norm)
+        sumsq = np.ones(X.shape[:-2] + (1, 1), dtype=np.float32)
     if pairs is None:
         pairs = m >= 1024 and n >= 2 * m
     eye = np.eye(m, dtype=np.float32)
@@ -286,7 +302,7 @@ def newton_schulz_shifted_bf16(
     for group in pair_schedule(coeffs, pairs):
         a, b, c = (f(v) for v in coeffs[done])
         s = sumsq / f(m)
-        gram = round_to_bf16(np.matmul(X, _mT(X)) - s * eye)
+        gram = round_to_bf16((r * r) * np.matmul(X, _mT(X)) - s * eye)
         if group == 2:
             a2, b2, c2 = (f(v) for v in coeffs[done + 1])
             r1 = round_to_bf16(c * np.matmul(gram, gram) + (b + f(2.0) * c * s) * gram)
@@ -297,13 +313,14 @@ def newton_schulz_shifted_bf16(
             r2 = round_to_bf16(c2 * np.matmul(d2, d2) + (b2 + f(2.0) * c2 * s2) * d2)
             e2 = a2 + b2 * s2 + c2 * s2 * s2
             q = round_to_bf16(_mirror_lower(np.matmul(r2, r1) + e2 * r1 + e1 * r2))
-            Xn = (e1 * e2) * X + np.matmul(q, X)
+            Xn = (e1 * e2 * r) * X + r * np.matmul(q, X)
         elif c != 0.0:
             poly = round_to_bf16(c * np.matmul(gram, gram) + (b + f(2.0) * c * s) * gram)
-            Xn = (a + b * s + c * s * s) * X + np.matmul(poly, X)
+            Xn = ((a + b * s + c * s * s) * r) * X + r * np.matmul(poly, X)
         else:
-            Xn = (a + b * s) * X + b * np.matmul(gram, X)
+            Xn = ((a + b * s) * r) * X + (b * r) * np.matmul(gram, X)
         done += group
+        r = np.ones_like(norm)  # from here on X is normalised
         sumsq = np.sum(Xn * Xn, axis=(-2, -1), keepdims=True, dtype=np.float32)
         X = Xn if done == len(coeffs) else round_to_bf16(Xn)
     X = X.astype(np.float32)
