@@ -254,11 +254,14 @@ __device__ __forceinline__ float block_sum_f32(float v, float* red) {
   return t;
 }
 
-// Resolves the diagonal shift s for this workgroup and the effective coefficients of the addends.
+// The diagonal shift s of this workgroup's matrix and the effective coefficients of product and addends
+// (returned by value: scalars handed out by reference end up in scratch memory).
+struct Scalars {
+  float shift, alpha, beta, beta2;
+};
 template <int NT>
-__device__ __forceinline__ float resolve_shift(const GemmParams& p, int64_t batch, float* red, float& alpha, float& beta,
-                                               float& beta2) {
-  float s = 0.0f;
+__device__ __forceinline__ Scalars resolve_shift(const GemmParams& p, int64_t batch, float* red) {
+  float s = 0.0f, alpha = p.alpha, beta = p.beta, beta2 = p.beta2;
   if (p.shift_mode == SHIFT_GRAM) {
     float part = 0.0f;
     const float* sl = p.slots_in + batch * p.nslots_in;
@@ -276,13 +279,9 @@ __device__ __forceinline__ float resolve_shift(const GemmParams& p, int64_t batc
     const float e1 = p.ca + p.cb * s + p.cc * s * s;
     const float s2 = e1 * e1 * s;
     const float e2 = p.ca2 + p.cb2 * s2 + p.cc2 * s2 * s2;
-    switch (p.shift_mode) {
-      case SHIFT_PAIR_T: beta = e1; beta2 = s; break;
-      case SHIFT_PAIR_A2: beta = e1; beta2 = e1 * s; break;
-      case SHIFT_PAIR_POLY2: beta = p.cb2 + 2.0f * p.cc2 * s2; break;
-      case SHIFT_PAIR_Q: beta = e2; beta2 = e1; break;
-      default: beta = e1 * e2; break;  // SHIFT_PAIR_APPLY
-    }
+    const int mode = p.shift_mode;
+    beta = mode == SHIFT_PAIR_POLY2 ? p.cb2 + 2.0f * p.cc2 * s2 : mode == SHIFT_PAIR_Q ? e2 : mode == SHIFT_PAIR_APPLY ? e1 * e2 : e1;
+    beta2 = mode == SHIFT_PAIR_T ? s : mode == SHIFT_PAIR_A2 ? e1 * s : mode == SHIFT_PAIR_Q ? e1 : beta2;
   }
   if (p.xscale != nullptr) {
     const float r = p.xscale[batch];
@@ -293,7 +292,7 @@ __device__ __forceinline__ float resolve_shift(const GemmParams& p, int64_t batc
       beta *= r;
     }
   }
-  return s;
+  return Scalars{s, alpha, beta, beta2};
 }
 
 // Epilogue shared by both kernels.  MI names the MFMA tile the accumulators come from:
@@ -494,11 +493,10 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_bf16_kernel(GemmParams p) 
     __syncthreads();
   }
 
-  float alpha = p.alpha, beta = p.beta, beta2 = p.beta2;
-  const float shift = resolve_shift<NT>(p, batch, red, alpha, beta, beta2);
+  const Scalars sc = resolve_shift<NT>(p, batch, red);
   const bool diag = (MODE == MODE_SYRK) && (tm == tn);
-  tile_epilogue<MODE, OUT_F32, true, FM, FN, NT>(p, acc, m0 + wm * TM, n0 + wn * TN, lane, batch, diag, alpha, beta,
-                                                 shift, red, beta2);
+  tile_epilogue<MODE, OUT_F32, true, FM, FN, NT>(p, acc, m0 + wm * TM, n0 + wn * TN, lane, batch, diag, sc.alpha, sc.beta,
+                                                 sc.shift, red, sc.beta2);
 }
 
 }  // namespace mi

@@ -974,8 +974,8 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
 #ifdef MI_TIMING
   const long long t_loop = __builtin_readcyclecounter();
 #endif
-  float alpha = p.alpha, beta = p.beta, beta2 = p.beta2;
-  const float shift = resolve_shift<NT>(p, batch, red, alpha, beta, beta2);
+  const Scalars sc = resolve_shift<NT>(p, batch, red);
+  const float alpha = sc.alpha, beta = sc.beta, beta2 = sc.beta2, shift = sc.shift;
   const bool diag = (MODE == MODE_SYRK) && (tm == tn);
   if constexpr (MODE == MODE_GEMM && (C::TN == 32 || C::TN == 64 || C::TN == 128)) {
     __syncthreads();  // every wavefront has finished reading the ring: it can be reused as staging space

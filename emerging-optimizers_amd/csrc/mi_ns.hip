@@ -697,7 +697,9 @@ static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, in
   }
   int64_t want = (numel / 8 + (int64_t)NORM_THREADS * 4 - 1) / ((int64_t)NORM_THREADS * 4);
   if (want < 1) want = 1;
-  if (want > 4096) want = 4096;
+  // (with a deferred divide nearly every call ends after the norm check: fewer, longer-running workgroups then)
+  const int64_t cap = xscale ? 1024 : 4096;
+  if (want > cap) want = cap;
   dim3 grid2((unsigned)want, (unsigned)batch);
 #define MI_SC(F, B) hipLaunchKernelGGL((scale_cast_kernel<F, B>), grid2, block, 0, stream, x, numel, partials, nb, eps, post_scale, out, dev_norm, sumsq_out, mom, xscale)
   if (f64) {

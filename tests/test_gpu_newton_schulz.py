@@ -115,6 +115,23 @@ def test_pair_rule_by_shape(gpu, monkeypatch):
     assert not torch.equal(outs[None], outs["0"])
 
 
+@pytest.mark.parametrize("shape", [(256, 512), (2, 128, 1024), (1024, 2048)])
+def test_deferred_normalisation_is_scale_invariant(gpu, shape):
+    """A wide input is cast to bf16 unnormalised and 1/norm enters the first products; norms outside
+    [1e-10, 1e10] take the normalising pass instead.  Powers of two commute with every rounding, so inside
+    either regime the result does not depend on the scale at all, and across regimes only by rounding."""
+    x = torch.randn(*shape)
+    want32 = O.newton_schulz(x.numpy(), 5, "quintic")
+    outs = {}
+    for k in (0, -20, 20, -45, 50):
+        with utils.fp32_matmul_precision("medium"):
+            outs[k] = muon_utils.newton_schulz((x * 2.0**k).to(gpu), steps=5, coefficient_type="quintic", use_syrk=True).cpu()
+        assert rel_fro(outs[k], want32) <= TOL_FP32, k
+    assert torch.equal(outs[0], outs[-20]) and torch.equal(outs[0], outs[20])  # deferred regime
+    assert torch.equal(outs[-45], outs[50])                                     # normalising regime
+    assert not torch.equal(outs[0], outs[50])
+
+
 def test_fused_known_answers(gpu):
     for case, x, want in known_answer_cases():
         with utils.fp32_matmul_precision("medium"):
