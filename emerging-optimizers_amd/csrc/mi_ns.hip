@@ -572,63 +572,143 @@ __global__ void __launch_bounds__(NORM_THREADS) scale_cast_kernel(const float* _
   }
 }
 
-// Tall inputs (rows > cols): the divide + bf16 cast also transposes, so that the iteration can run on the
-// (cols x rows) orientation with K-contiguous operands (the fastest kernels), and the float32 result is
-// transposed back once at the end.  64 x 64 tiles through LDS, 16-byte global accesses on both sides.
+// Tall inputs (rows > cols): the bf16 cast also transposes, so that the iteration can run on the (cols x rows)
+// orientation with K-contiguous operands (the fastest kernels), and the float32 result is transposed back once at
+// the end.  64 x 64 tiles through LDS, 16-byte global accesses on both sides; every workgroup walks over tiles
+// blockIdx.x, blockIdx.x + gridDim.x, ...
+struct TileWalk {
+  int64_t rows, cols;
+  int tiles_c;
+  int64_t ntiles;
+  __device__ TileWalk(int64_t r, int64_t c) : rows(r), cols(c), tiles_c((int)((c + 63) / 64)), ntiles(((r + 63) / 64) * ((c + 63) / 64)) {}
+};
+// One 64 x 64 tile of `tile` (float32, [row][col]) -> bf16 at out[(c0 + c) * rows + r0 + r], values divided by `div`.
+__device__ __forceinline__ void store_tile_transposed(const float (&tile)[64][65], uint16_t* __restrict__ ob, int64_t rows,
+                                                      int64_t cols, int64_t r0, int64_t c0, float div) {
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int c = pass * 32 + (threadIdx.x >> 3), r = (threadIdx.x & 7) * 8;
+    if (c0 + c < cols && r0 + r < rows) {
+      f32x4_t lo = {tile[r][c] / div, tile[r + 1][c] / div, tile[r + 2][c] / div, tile[r + 3][c] / div};
+      f32x4_t hi = {tile[r + 4][c] / div, tile[r + 5][c] / div, tile[r + 6][c] / div, tile[r + 7][c] / div};
+      const uint2 a = __builtin_bit_cast(uint2, __builtin_convertvector(lo, bf16x4_t));
+      const uint2 d = __builtin_bit_cast(uint2, __builtin_convertvector(hi, bf16x4_t));
+      *reinterpret_cast<uint4*>(ob + (c0 + c) * rows + r0 + r) = make_uint4(a.x, a.y, d.x, d.y);
+    }
+  }
+}
+
+// First pass of a tall input when the divide is deferred: sum of squares (one partial per workgroup), momentum
+// update in place if asked for, and the unnormalised bf16 cast, transposed.
+template <bool F64>
+__global__ void __launch_bounds__(256) sumsq_transpose_kernel(const float* __restrict__ x, int64_t rows, int64_t cols,
+                                                              double* __restrict__ partials, MomentumSrc mom,
+                                                              uint16_t* __restrict__ raw_out) {
+  const int64_t b = blockIdx.y;
+  __shared__ double scratch_d[NORM_THREADS / 64];
+  __shared__ float tile[64][65];
+  const TileWalk w(rows, cols);
+  const float* __restrict__ xb = x + b * rows * cols;
+  float* __restrict__ mb = mom.buf ? mom.buf + b * rows * cols : nullptr;
+  uint16_t* __restrict__ ob = raw_out + b * rows * cols;
+  float sf = 0.0f;
+  double sd = 0.0;
+  for (int64_t t = blockIdx.x; t < w.ntiles; t += gridDim.x) {
+    const int64_t r0 = (t / w.tiles_c) * 64, c0 = (t % w.tiles_c) * 64;
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+      const int r = pass * 16 + (threadIdx.x >> 4), c = (threadIdx.x & 15) * 4;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (r0 + r < rows && c0 + c < cols) {
+        const int64_t at = (r0 + r) * cols + c0 + c;
+        v = *reinterpret_cast<const float4*>(xb + at);
+        if (mb) {
+          float4 m = *reinterpret_cast<const float4*>(mb + at);
+          m.x = torch_lerp(m.x, v.x, 1.0f - mom.beta);
+          m.y = torch_lerp(m.y, v.y, 1.0f - mom.beta);
+          m.z = torch_lerp(m.z, v.z, 1.0f - mom.beta);
+          m.w = torch_lerp(m.w, v.w, 1.0f - mom.beta);
+          *reinterpret_cast<float4*>(mb + at) = m;
+          v.x = momentum_direction(v.x, m.x, mom.beta, mom.nesterov);
+          v.y = momentum_direction(v.y, m.y, mom.beta, mom.nesterov);
+          v.z = momentum_direction(v.z, m.z, mom.beta, mom.nesterov);
+          v.w = momentum_direction(v.w, m.w, mom.beta, mom.nesterov);
+        }
+      }
+      if (F64) {
+        sd += (double)v.x * (double)v.x + (double)v.y * (double)v.y + (double)v.z * (double)v.z + (double)v.w * (double)v.w;
+      } else {
+        sf = __builtin_fmaf(v.x, v.x, sf);
+        sf = __builtin_fmaf(v.y, v.y, sf);
+        sf = __builtin_fmaf(v.z, v.z, sf);
+        sf = __builtin_fmaf(v.w, v.w, sf);
+      }
+      tile[r][c] = v.x;
+      tile[r][c + 1] = v.y;
+      tile[r][c + 2] = v.z;
+      tile[r][c + 3] = v.w;
+    }
+    __syncthreads();
+    store_tile_transposed(tile, ob, rows, cols, r0, c0, 1.0f);
+    __syncthreads();
+  }
+  const double total = block_sum<double>(F64 ? sd : (double)sf, scratch_d);
+  if (threadIdx.x == 0) partials[b * gridDim.x + blockIdx.x] = total;
+}
+
+// Divide + bf16 cast + transpose.  `xscale` != null: `out` already holds the unnormalised cast; this pass then only
+// has work to do for a norm outside the range where the divide may be deferred (see scale_cast_kernel).
 __global__ void __launch_bounds__(256) scale_cast_transpose_kernel(const float* __restrict__ x, int64_t rows, int64_t cols,
                                                                    const double* __restrict__ partials, int nparts,
                                                                    float eps, int f64, uint16_t* __restrict__ out,
                                                                    float* __restrict__ dev_norm,
-                                                                   float* __restrict__ sumsq_out, MomentumSrc mom) {
-  const int64_t b = blockIdx.z;
+                                                                   float* __restrict__ sumsq_out, MomentumSrc mom,
+                                                                   float* __restrict__ xscale) {
+  const int64_t b = blockIdx.y;
   __shared__ double scratch_d[NORM_THREADS / 64];
   __shared__ float tile[64][65];
   double s = 0;
   for (int i = threadIdx.x; i < nparts; i += NORM_THREADS) s += partials[b * nparts + i];
   s = block_sum<double>(s, scratch_d);
   const float divisor = f64 ? (float)sqrt(s) : fmaxf(sqrtf((float)s), eps);
-  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+  bool deferred = false;
+  if (xscale) deferred = divisor >= NORM_DEFER_MIN && divisor <= NORM_DEFER_MAX;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
     if (dev_norm) dev_norm[b] = divisor;
     if (sumsq_out) {
       const float ratio = sqrtf((float)s) / divisor;
       sumsq_out[b] = (divisor > 0.0f && ratio == ratio) ? ratio * ratio : 0.0f;
     }
+    if (xscale) xscale[b] = deferred ? 1.0f / divisor : 1.0f;
   }
-  const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+  if (deferred) return;
+  const TileWalk w(rows, cols);
   const float* __restrict__ xb = x + b * rows * cols;
-  // read 64 rows x 64 cols: thread t handles row t/4 (+ 16 per pass... 4 passes), 16 columns... use float4 x 4 passes
-#pragma unroll
-  for (int pass = 0; pass < 4; ++pass) {
-    const int r = pass * 16 + (threadIdx.x >> 4), c = (threadIdx.x & 15) * 4;
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (r0 + r < rows && c0 + c < cols) {
-      v = *reinterpret_cast<const float4*>(xb + (r0 + r) * cols + c0 + c);
-      if (mom.buf) {
-        const float4 mb = *reinterpret_cast<const float4*>(mom.buf + b * rows * cols + (r0 + r) * cols + c0 + c);
-        v.x = momentum_direction(v.x, mb.x, mom.beta, mom.nesterov);
-        v.y = momentum_direction(v.y, mb.y, mom.beta, mom.nesterov);
-        v.z = momentum_direction(v.z, mb.z, mom.beta, mom.nesterov);
-        v.w = momentum_direction(v.w, mb.w, mom.beta, mom.nesterov);
-      }
-    }
-    tile[r][c] = v.x / divisor;
-    tile[r][c + 1] = v.y / divisor;
-    tile[r][c + 2] = v.z / divisor;
-    tile[r][c + 3] = v.w / divisor;
-  }
-  __syncthreads();
-  // write transposed: out[(c0 + c)][r0 + r], 8 consecutive r per thread (16 bytes of bf16)
   uint16_t* __restrict__ ob = out + b * rows * cols;
+  for (int64_t t = blockIdx.x; t < w.ntiles; t += gridDim.x) {
+    const int64_t r0 = (t / w.tiles_c) * 64, c0 = (t % w.tiles_c) * 64;
 #pragma unroll
-  for (int pass = 0; pass < 2; ++pass) {
-    const int c = pass * 32 + (threadIdx.x >> 3), r = (threadIdx.x & 7) * 8;
-    if (c0 + c < cols && r0 + r < rows) {
-      f32x4_t lo = {tile[r][c], tile[r + 1][c], tile[r + 2][c], tile[r + 3][c]};
-      f32x4_t hi = {tile[r + 4][c], tile[r + 5][c], tile[r + 6][c], tile[r + 7][c]};
-      const uint2 a = __builtin_bit_cast(uint2, __builtin_convertvector(lo, bf16x4_t));
-      const uint2 d = __builtin_bit_cast(uint2, __builtin_convertvector(hi, bf16x4_t));
-      *reinterpret_cast<uint4*>(ob + (c0 + c) * rows + r0 + r) = make_uint4(a.x, a.y, d.x, d.y);
+    for (int pass = 0; pass < 4; ++pass) {
+      const int r = pass * 16 + (threadIdx.x >> 4), c = (threadIdx.x & 15) * 4;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (r0 + r < rows && c0 + c < cols) {
+        v = *reinterpret_cast<const float4*>(xb + (r0 + r) * cols + c0 + c);
+        if (mom.buf) {
+          const float4 mb = *reinterpret_cast<const float4*>(mom.buf + b * rows * cols + (r0 + r) * cols + c0 + c);
+          v.x = momentum_direction(v.x, mb.x, mom.beta, mom.nesterov);
+          v.y = momentum_direction(v.y, mb.y, mom.beta, mom.nesterov);
+          v.z = momentum_direction(v.z, mb.z, mom.beta, mom.nesterov);
+          v.w = momentum_direction(v.w, mb.w, mom.beta, mom.nesterov);
+        }
+      }
+      tile[r][c] = v.x;
+      tile[r][c + 1] = v.y;
+      tile[r][c + 2] = v.z;
+      tile[r][c + 3] = v.w;
     }
+    __syncthreads();
+    store_tile_transposed(tile, ob, rows, cols, r0, c0, divisor);
+    __syncthreads();
   }
 }
 
@@ -680,17 +760,29 @@ static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, in
   if (batch == 0 || numel == 0) return MI_OK;
   const int nb = norm_blocks(numel);
   dim3 grid1(nb, (unsigned)batch), block(NORM_THREADS);
-  if (xscale && (t_rows > 0 || !out_bf16)) return fail(MI_ERR_BAD_ARG, "internal: deferred normalisation needs a plain bf16 output");
+  if (xscale && !out_bf16) return fail(MI_ERR_BAD_ARG, "internal: deferred normalisation needs a bf16 output");
   uint16_t* raw_out = xscale ? static_cast<uint16_t*>(out) : nullptr;
-  if (f64)
+  int nparts = nb;
+  if (t_rows > 0 && xscale) {
+    // tall input, deferred divide: the first pass already transposes (one partial per workgroup of the tile walk)
+    const int64_t ntiles = ((t_rows + 63) / 64) * ((t_cols + 63) / 64);
+    nparts = (int)(ntiles < NORM_MAX_BLOCKS ? ntiles : NORM_MAX_BLOCKS);
+    dim3 gridw((unsigned)nparts, (unsigned)batch);
+    if (f64)
+      hipLaunchKernelGGL(sumsq_transpose_kernel<true>, gridw, block, 0, stream, x, t_rows, t_cols, partials, mom, raw_out);
+    else
+      hipLaunchKernelGGL(sumsq_transpose_kernel<false>, gridw, block, 0, stream, x, t_rows, t_cols, partials, mom, raw_out);
+  } else if (f64) {
     hipLaunchKernelGGL(sumsq_kernel<true>, grid1, block, 0, stream, x, numel, partials, mom, raw_out);
-  else
+  } else {
     hipLaunchKernelGGL(sumsq_kernel<false>, grid1, block, 0, stream, x, numel, partials, mom, raw_out);
+  }
   if (t_rows > 0) {
     // bf16 output transposed to (t_cols x t_rows)
-    dim3 gridt((unsigned)((t_cols + 63) / 64), (unsigned)((t_rows + 63) / 64), (unsigned)batch);
-    hipLaunchKernelGGL(scale_cast_transpose_kernel, gridt, block, 0, stream, x, t_rows, t_cols, partials, nb, eps, f64,
-                       static_cast<uint16_t*>(out), dev_norm, sumsq_out, mom);
+    const int64_t ntiles = ((t_rows + 63) / 64) * ((t_cols + 63) / 64);
+    dim3 gridt((unsigned)(ntiles < 2048 ? ntiles : 2048), (unsigned)batch);
+    hipLaunchKernelGGL(scale_cast_transpose_kernel, gridt, block, 0, stream, x, t_rows, t_cols, partials, nparts, eps, f64,
+                       static_cast<uint16_t*>(out), dev_norm, sumsq_out, mom, xscale);
     hipError_t et = hipGetLastError();
     if (et != hipSuccess) return fail(MI_ERR_LAUNCH, "mi_frob_normalize launch failed: %s", hipGetErrorString(et));
     return MI_OK;
@@ -885,10 +977,9 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
   const int64_t ld = n;
   const int64_t x_bs = numel, g_bs = m * m;
   float* result = tall ? reinterpret_cast<float*>(ws + w.result) : out;
-  // A wide (or square) input is cast to bf16 by the pass that sums its squares, and the divide by the norm is
-  // folded into the first Gram product and the first B X product (one pass over the float32 input instead of two).
-  // A tall input needs the transposing second pass anyway.
-  float* xscale = tall ? nullptr : reinterpret_cast<float*>(ws + w.xscale);
+  // The input is cast to bf16 by the pass that sums its squares (transposing, if it is tall), and the divide by the
+  // norm is folded into the first Gram product and the first B X product: one pass over the float32 input, not two.
+  float* xscale = reinterpret_cast<float*>(ws + w.xscale);
   int rc;
   {
     ProfScope prof(PROF_NORMALIZE, stream);

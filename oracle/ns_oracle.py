@@ -258,8 +258,8 @@ def newton_schulz_shifted_bf16(
     with s = ||X||_F^2 / m instead and folds the identity part into the epilogue scalars
         B' = c A'^2 + (b + 2 c s) A',      X' = (a + b s + c s^2) X + B' X,
     which is algebraically the same iteration for any s.  The last step is written to float32 unrounded.
-    Inputs that are not tall are rounded to bf16 before the division by the norm, which then enters the first
-    products as a scalar (one pass over the float32 input instead of two).
+    The input is rounded to bf16 before the division by the norm, which then enters the first products as a
+    scalar (one pass over the float32 input instead of two).
 
     For wide matrices (m >= 1024, n >= 2 m; ``pairs`` overrides the rule) the driver takes steps two at a time
     on one Gram matrix (see :func:`pair_schedule`).  All factors are polynomials of A and commute, so with
@@ -279,14 +279,13 @@ def newton_schulz_shifted_bf16(
     f = np.float32
     m, n = x.shape[-2:]
     coeffs = expand_coefficients(steps, coefficient_type, custom_coefficient_sets)
-    # A wide or square input is cast to bf16 unnormalised and 1 / ||x||_F enters the first group's products
-    # (r^2 in the Gram matrix, r in X' = ... ); a tall one is normalised before the cast.  The deferral is limited
-    # to norms whose squares are safe in float32.
+    # The input is cast to bf16 unnormalised and 1 / ||x||_F enters the first group's products (r^2 in the Gram
+    # matrix, r in X' = ...).  The deferral is limited to norms whose squares are safe in float32.
     if normalize_in_double:
         norm = np.sqrt(np.sum(x.astype(np.float64) ** 2, axis=(-2, -1), keepdims=True)).astype(np.float32)
     else:
         norm = np.maximum(np.sqrt(np.sum(x * x, axis=(-2, -1), keepdims=True, dtype=np.float32)), f(eps))
-    deferred = (not transpose) and len(coeffs) > 0 and bool(np.all((norm >= f(1e-10)) & (norm <= f(1e10))))
+    deferred = len(coeffs) > 0 and bool(np.all((norm >= f(1e-10)) & (norm <= f(1e10))))
     if deferred:
         X = round_to_bf16(x)
         r = f(1.0) / norm

@@ -115,9 +115,9 @@ def test_pair_rule_by_shape(gpu, monkeypatch):
     assert not torch.equal(outs[None], outs["0"])
 
 
-@pytest.mark.parametrize("shape", [(256, 512), (2, 128, 1024), (1024, 2048)])
+@pytest.mark.parametrize("shape", [(256, 512), (2, 128, 1024), (1024, 2048), (512, 256), (2, 1000, 504), (2048, 1024)])
 def test_deferred_normalisation_is_scale_invariant(gpu, shape):
-    """A wide input is cast to bf16 unnormalised and 1/norm enters the first products; norms outside
+    """The input is cast to bf16 unnormalised and 1/norm enters the first products; norms outside
     [1e-10, 1e10] take the normalising pass instead.  Powers of two commute with every rounding, so inside
     either regime the result does not depend on the scale at all, and across regimes only by rounding."""
     x = torch.randn(*shape)
