@@ -891,14 +891,16 @@ struct NsWorkspace {
 
 // Whether two consecutive steps share one Gram matrix (see SHIFT_PAIR_* in gemm_engine.hpp).  A pair trades one
 // X X^T and one B X (3 m^2 n multiply-adds) for four m x m products, which pays for wide matrices only; a pair on a
-// square matrix would also sit close to the 1e-2 tolerance.  MI_NS_PAIRS=0 switches pairing off, MI_NS_PAIRS=force
+// square matrix would also sit close to the 1e-2 tolerance; below 1024 rows the kernels are launch-bound and a pair
+// has more launches, except on the split-K Gram path.  MI_NS_PAIRS=0 switches pairing off, MI_NS_PAIRS=force
 // pairs wherever the kernels allow it (used by the tests to reach the pair kernels with small matrices).
 static int ns_pairs_enabled(int64_t m, int64_t n, int gram_splits) {
-  if (gram_splits > 0) return 0;
   const char* env = getenv("MI_NS_PAIRS");
   if (env && env[0] == '0') return 0;
   if (env && env[0] == 'f') return 1;
-  return m >= 1024 && n >= 2 * m;
+  // (the split-K Gram path serves short matrices at least four times as wide as tall: a pair there trades two
+  // passes over X for four tiny products at the same number of launches)
+  return gram_splits > 0 || (m >= 1024 && n >= 2 * m);
 }
 
 static NsWorkspace ns_layout(int64_t batch, int64_t rows, int64_t cols) {

@@ -261,7 +261,8 @@ def newton_schulz_shifted_bf16(
     The input is rounded to bf16 before the division by the norm, which then enters the first products as a
     scalar (one pass over the float32 input instead of two).
 
-    For wide matrices (m >= 1024, n >= 2 m; ``pairs`` overrides the rule) the driver takes steps two at a time
+    For wide matrices (m >= 1024 and n >= 2 m, or the short, very wide per-head shapes whose Gram matrix is summed
+    from K slices; ``pairs`` overrides the rule) the driver takes steps two at a time
     on one Gram matrix (see :func:`pair_schedule`).  All factors are polynomials of A and commute, so with
     q1 = e1 I + R1 (R1 = B' of the first step, e1 = a1 + b1 s + c1 s^2):
         A2 = q1^2 A = s2 I + D2,  T' = R1 A' + e1 A' + s R1,  D2 = R1 T' + e1 T' + e1 s R1,  s2 = e1^2 s,
@@ -295,7 +296,9 @@ def newton_schulz_shifted_bf16(
         r = np.ones_like(norm)
         sumsq = np.ones(X.shape[:-2] + (1, 1), dtype=np.float32)
     if pairs is None:
-        pairs = m >= 1024 and n >= 2 * m
+        batch = int(np.prod(x.shape[:-2])) if x.ndim == 3 else 1
+        split_k_gram = m % 128 == 0 and m <= 256 and n % 512 == 0 and n >= 1024 and batch * (n // 512) <= 65535
+        pairs = split_k_gram or (m >= 1024 and n >= 2 * m)
     eye = np.eye(m, dtype=np.float32)
     done = 0
     for group in pair_schedule(coeffs, pairs):
