@@ -42,6 +42,7 @@ WORKLOADS = {
     "moe": (8, 4096, 14336),       # 8 stacked experts at full shape (1.9 GB of float32 gradients)
     "batched_syrk": (16, 2048, 8192),  # batched SYRK alone (no Newton-Schulz), bf16 in / bf16 out
     "muon_step": (4096, 14336),    # whole Muon.step() (momentum 0.95, Nesterov, weight decay) on the headline gradient
+    "muon_heads": (32, 128, 4096),  # Muon.step() over 32 separate 128x4096 parameters: serial loop vs one batched call
 }
 COEFFS = [(3.4445, -4.7750, 2.0315)] * NS_STEPS  # "simple" table cycled
 
@@ -170,9 +171,54 @@ def muon_step_workload(args):
     }))
 
 
+def muon_heads_workload(args):
+    """Muon.step over many small parameters of one shape: the reference's serial loop against group_same_shape."""
+    import torch
+
+    from emerging_optimizers import _hip
+    from emerging_optimizers.orthogonalized_optimizers.muon import Muon
+
+    _hip.lib()
+    dev = torch.device("cuda:0")
+    heads, m, n = WORKLOADS["muon_heads"]
+    gen = torch.Generator().manual_seed(2)
+    grads = [(torch.randn(heads, m, n, generator=gen) * 1e-3).to(dev) for _ in range(2)]
+    ms = {}
+    for grouped in (False, True):
+        ps = [torch.nn.Parameter((torch.randn(m, n, generator=gen) * 0.02).to(dev)) for _ in range(heads)]
+        opt = Muon(ps, lr=3e-4, momentum=0.95, nesterov=True, weight_decay=0.01, num_ns_steps=NS_STEPS,
+                   coefficient_type="simple", use_syrk=True, fp32_matmul_prec="medium", group_same_shape=grouped)
+
+        def one(i):
+            for h, p in enumerate(ps):
+                p.grad = grads[i % 2][h]
+            opt.step()
+
+        for i in range(args.warmup):
+            one(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            one(i)
+        torch.cuda.synchronize()
+        ms[grouped] = (time.perf_counter() - t0) / args.steps * 1e3
+    print(json.dumps({
+        "metric": "Muon.step ms over 32 parameters of 128x4096 (one batched orthogonalisation per shape)",
+        "value": round(ms[True], 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms[True], 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"Muon.step on {heads} separate {m}x{n} float32 weights, momentum 0.95, Nesterov, decoupled "
+                               "weight decay, 5 'simple' NS steps; group_same_shape=True",
+                   "ms_serial_loop": round(ms[False], 4), "speedup": round(ms[False] / ms[True], 2)},
+    }))
+
+
 def side_workload(args):
     """Times another benchmark configuration through the same entry point; one JSON line, no roofline legs."""
     import torch
+
+    if args.workload == "muon_heads":
+        return muon_heads_workload(args)
 
     if args.workload == "batched_syrk":
         return batched_syrk_workload(args)

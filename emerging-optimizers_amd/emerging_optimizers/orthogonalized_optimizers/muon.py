@@ -83,6 +83,7 @@ class Muon(OrthogonalizedOptimizer[HookStateT]):
         scale_mode: see :func:`get_muon_scale_factor`.
         extra_scale_factor: further multiplier of the update (0.2 roughly matches AdamW's update RMS).
         use_syrk: run the iteration on the hand-written SYRK/GEMM kernels.
+        group_same_shape: one batched orthogonalisation per distinct parameter shape (see the base class).
     """
 
     def __init__(
@@ -101,6 +102,7 @@ class Muon(OrthogonalizedOptimizer[HookStateT]):
         extra_scale_factor: float = 1.0,
         use_syrk: bool = False,
         weight_update_hook: Optional[WeightUpdateHook[HookStateT]] = None,
+        group_same_shape: bool = False,
     ) -> None:
         if num_ns_steps < 1:
             raise ValueError(f"num_ns_steps must be at least 1, got {num_ns_steps}")
@@ -139,6 +141,7 @@ class Muon(OrthogonalizedOptimizer[HookStateT]):
             fp32_matmul_prec=fp32_matmul_prec,
             scaled_orthogonalize_fn=scaled_orthogonalize_fn,
             weight_update_hook=weight_update_hook,
+            group_same_shape=group_same_shape,
         )
         self._own_scaled_orthogonalize_fn = scaled_orthogonalize_fn
 

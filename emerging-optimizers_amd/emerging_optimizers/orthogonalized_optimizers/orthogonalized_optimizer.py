@@ -45,6 +45,10 @@ class OrthogonalizedOptimizer(WeightDecayMixin, Optimizer, Generic[HookStateT]):
     Args:
         {_args_doc}
         scaled_orthogonalize_fn: maps the momentum tensor to the update; identity when omitted.
+        group_same_shape: orthogonalise all 2-D parameters of one shape (within a parameter group) in one
+            batched call instead of one call each.  Not in the reference, whose loop
+            (orthogonalized_optimizer.py:175-210) is serial; pays for many small matrices (attention heads kept
+            as separate parameters), where single calls are bound by launch latency.
         **kwargs: extra per-group defaults, stored unchecked.
     """
 
@@ -60,8 +64,10 @@ class OrthogonalizedOptimizer(WeightDecayMixin, Optimizer, Generic[HookStateT]):
         fp32_matmul_prec: FP32MatmulPrecT,
         scaled_orthogonalize_fn: Optional[Callable] = None,
         weight_update_hook: Optional[WeightUpdateHook[HookStateT]] = None,
+        group_same_shape: bool = False,
         **kwargs: Any,
     ):
+        self._group_same_shape = bool(group_same_shape)
         if scaled_orthogonalize_fn is None:
             _log.warning("scaled_orthogonalize_fn not provided. Using noop")
             scaled_orthogonalize_fn = torch.nn.Identity()
@@ -91,24 +97,51 @@ class OrthogonalizedOptimizer(WeightDecayMixin, Optimizer, Generic[HookStateT]):
             self._init_group(group)
             lr, beta = group["lr"], group["momentum"]
             extras = {k: v for k, v in group.items() if k != "params"}
+            shared = self._shapes_to_batch(group)
+            batches: dict = {}
             for p in group["params"]:
                 grad = p.grad
                 if grad is None:
                     continue
                 buf = self.state[p]["momentum_buffer"]
-                if self._fused_update(p, grad, buf, lr, beta, group["weight_decay"]):
+                key = (tuple(p.shape), p.dtype, p.device)
+                if key not in shared and self._fused_update(p, grad, buf, lr, beta, group["weight_decay"]):
                     continue
                 self._apply_weight_decay_inplace(p, grad, lr, group["weight_decay"])
                 buf.lerp_(grad, 1 - beta)
                 direction = grad.lerp(buf, beta) if self.nesterov else buf
+                if key in shared:
+                    batches.setdefault(key, []).append((p, direction))
+                    continue
                 with utils.fp32_matmul_precision(self.fp32_matmul_prec):
                     update = self.orthogonalize(p, direction, **extras)
-                self.pre_weight_update_fn_inplace(p, update)
-                hook_state = self._weight_update_hook.pre_weight_update_inplace(p, update)
-                p.add_(update, alpha=-lr)
-                self.post_weight_update_fn_inplace(p)
-                self._weight_update_hook.post_weight_update_inplace(p, hook_state)
+                self._apply_update(p, update, lr)
+            for members in batches.values():
+                # one batched orthogonalisation; every matrix of the stack is treated exactly as it would be alone
+                with utils.fp32_matmul_precision(self.fp32_matmul_prec):
+                    updates = self.scaled_orthogonalize_fn(torch.stack([d for _, d in members]))
+                for (p, _), update in zip(members, updates):
+                    self._apply_update(p, update, lr)
         return None
+
+    def _apply_update(self, p: torch.Tensor, update: torch.Tensor, lr: float) -> None:
+        self.pre_weight_update_fn_inplace(p, update)
+        hook_state = self._weight_update_hook.pre_weight_update_inplace(p, update)
+        p.add_(update, alpha=-lr)
+        self.post_weight_update_fn_inplace(p)
+        self._weight_update_hook.post_weight_update_inplace(p, hook_state)
+
+    def _shapes_to_batch(self, group: dict) -> set:
+        """(shape, dtype, device) keys shared by two or more 2-D parameters with gradients, when batching is on
+        and ``orthogonalize`` is the base implementation (an override may treat a parameter piecewise)."""
+        if not self._group_same_shape or type(self).orthogonalize is not OrthogonalizedOptimizer.orthogonalize:
+            return set()
+        seen: dict = {}
+        for p in group["params"]:
+            if p.grad is not None and p.dim() == 2:
+                key = (tuple(p.shape), p.dtype, p.device)
+                seen[key] = seen.get(key, 0) + 1
+        return {k for k, n in seen.items() if n > 1}
 
     def _fused_update(
         self, p: torch.Tensor, grad: torch.Tensor, buf: torch.Tensor, lr: float, beta: float, weight_decay: float

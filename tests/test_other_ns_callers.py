@@ -320,3 +320,66 @@ def test_muon_hyperball_on_the_kernels(gpu):
         assert abs(float(p.detach().norm()) - radius) < 1e-4
         res.append(p.detach() - w)
     assert float((res[0] - res[1]).norm() / res[1].norm()) <= 2e-2
+
+
+# ---------------------------------------------------------------- same-shape parameters in one batched call
+def _heads_model(device, n_heads=6):
+    torch.manual_seed(13)
+    ps = [nn.Parameter(torch.randn(128, 1024, device=device) * 0.02) for _ in range(n_heads)]
+    ps += [nn.Parameter(torch.randn(256, 512, device=device) * 0.02), nn.Parameter(torch.randn(64, 64, device=device))]
+    return ps
+
+
+def _run_steps(ps, opt, n=2):
+    g = torch.Generator().manual_seed(14)
+    for _ in range(n):
+        for p in ps:
+            p.grad = (torch.randn(p.shape, generator=g) * 1e-3).to(p.device)
+        opt.step()
+
+
+@pytest.mark.parametrize("nesterov", [False, True])
+def test_group_same_shape_equals_the_serial_loop(nesterov):
+    a, b = _heads_model("cpu"), _heads_model("cpu")
+    calls = []
+    kw = dict(lr=0.05, nesterov=nesterov, weight_decay=0.01, fp32_matmul_prec="highest")
+    grouped = oo.Muon(a, group_same_shape=True, **kw)
+    real = grouped.scaled_orthogonalize_fn
+    grouped.scaled_orthogonalize_fn = lambda t: (calls.append(tuple(t.shape)), real(t))[1]
+    serial = oo.Muon(b, **kw)
+    _run_steps(a, grouped)
+    _run_steps(b, serial)
+    assert sorted(calls[:3]) == [(6, 128, 1024), (64, 64), (256, 512)]  # one batched call for the six heads
+    for p, q in zip(a, b):
+        # (torch's batched and plain CPU matmuls differ in the last bits)
+        torch.testing.assert_close(p.detach(), q.detach(), rtol=1e-5, atol=2e-6)
+        assert torch.equal(grouped.state[p]["momentum_buffer"], serial.state[q]["momentum_buffer"])
+
+
+def test_group_same_shape_leaves_overridden_orthogonalize_alone():
+    class Split(oo.Muon):
+        def orthogonalize(self, p, grad, **kwargs):
+            return torch.cat([self.scaled_orthogonalize_fn(h) for h in grad.chunk(2, dim=0)], dim=0)
+
+    ps = _heads_model("cpu", 2)
+    opt = Split(ps, group_same_shape=True, fp32_matmul_prec="highest")
+    assert opt._shapes_to_batch(opt.param_groups[0]) == set()
+    _run_steps(ps, opt, 1)  # runs through the override, one parameter at a time
+
+
+@pytest.mark.gpu
+def test_group_same_shape_on_the_kernels(gpu):
+    from emerging_optimizers.orthogonalized_optimizers import muon as muon_mod
+    a, b = _heads_model(gpu), _heads_model(gpu)
+    _run_steps(a, oo.Muon(a, lr=0.05, use_syrk=True, nesterov=True, group_same_shape=True))
+    saved = muon_mod.FUSED_MUON_STEP
+    muon_mod.FUSED_MUON_STEP = False  # the one-call update rounds the weight update differently
+    try:
+        _run_steps(b, oo.Muon(b, lr=0.05, use_syrk=True, nesterov=True))
+    finally:
+        muon_mod.FUSED_MUON_STEP = saved
+    for p, q in zip(a[:6], b[:6]):
+        assert torch.equal(p.detach(), q.detach())  # a batch entry is computed exactly as the matrix alone
+    start = _heads_model(gpu)
+    for p, q, p0 in zip(a[6:], b[6:], start[6:]):  # shapes that occur once keep the one-call update
+        assert float((p.detach() - q.detach()).norm() / (q.detach() - p0.detach()).norm()) <= 1e-2
