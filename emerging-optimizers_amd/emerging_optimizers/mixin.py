@@ -38,3 +38,22 @@ class WeightDecayMixin:
         if shrink is None:
             raise ValueError(f"Invalid weight decay method: {method}")
         p.add_(p, alpha=-shrink)
+
+    def _apply_weight_decay_foreach_inplace(
+        self, params: list[torch.Tensor], grads: list[torch.Tensor], lr: float, weight_decay: float
+    ) -> None:
+        """The same update for a list of parameters, in one multi-tensor launch (element for element identical)."""
+        if weight_decay == 0.0 or not params:
+            return
+        method = getattr(self, "weight_decay_method", "l2")
+        if method == "l2":
+            torch._foreach_add_(grads, params, alpha=weight_decay)
+            return
+        shrink = {
+            "decoupled": weight_decay * lr,
+            "independent": weight_decay,
+            "palm": weight_decay * lr * lr,
+        }.get(method)
+        if shrink is None:
+            raise ValueError(f"Invalid weight decay method: {method}")
+        torch._foreach_add_(params, params, alpha=-shrink)

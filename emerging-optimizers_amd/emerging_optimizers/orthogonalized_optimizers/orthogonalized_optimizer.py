@@ -107,21 +107,30 @@ class OrthogonalizedOptimizer(WeightDecayMixin, Optimizer, Generic[HookStateT]):
                 key = (tuple(p.shape), p.dtype, p.device)
                 if key not in shared and self._fused_update(p, grad, buf, lr, beta, group["weight_decay"]):
                     continue
+                if key in shared:
+                    batches.setdefault(key, []).append(p)
+                    continue
                 self._apply_weight_decay_inplace(p, grad, lr, group["weight_decay"])
                 buf.lerp_(grad, 1 - beta)
                 direction = grad.lerp(buf, beta) if self.nesterov else buf
-                if key in shared:
-                    batches.setdefault(key, []).append((p, direction))
-                    continue
                 with utils.fp32_matmul_precision(self.fp32_matmul_prec):
                     update = self.orthogonalize(p, direction, **extras)
                 self._apply_update(p, update, lr)
             for members in batches.values():
-                # one batched orthogonalisation; every matrix of the stack is treated exactly as it would be alone
+                # Same statements as above, as multi-tensor launches, around one batched orthogonalisation in
+                # which every matrix of the stack is treated exactly as it would be alone.
+                grads = [p.grad for p in members]
+                bufs = [self.state[p]["momentum_buffer"] for p in members]
+                self._apply_weight_decay_foreach_inplace(members, grads, lr, group["weight_decay"])
+                torch._foreach_lerp_(bufs, grads, 1 - beta)
+                directions = torch._foreach_lerp(grads, bufs, beta) if self.nesterov else bufs
                 with utils.fp32_matmul_precision(self.fp32_matmul_prec):
-                    updates = self.scaled_orthogonalize_fn(torch.stack([d for _, d in members]))
-                for (p, _), update in zip(members, updates):
-                    self._apply_update(p, update, lr)
+                    updates = self.scaled_orthogonalize_fn(torch.stack(list(directions)))
+                if self._update_is_plain():
+                    torch._foreach_add_(members, list(updates.unbind(0)), alpha=-lr)
+                else:
+                    for p, update in zip(members, updates):
+                        self._apply_update(p, update, lr)
         return None
 
     def _apply_update(self, p: torch.Tensor, update: torch.Tensor, lr: float) -> None:
