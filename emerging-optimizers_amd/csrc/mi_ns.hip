@@ -852,10 +852,165 @@ __global__ void __launch_bounds__(256) gram_reduce_kernel(const float* __restric
   ob[(int64_t)j * m + i] = h;
 }
 
+// ---------------------------------------------------------------------------------------------
+// 128 x 128 matrices (one attention head each): everything between the split-K Gram partials and the B X product
+// of a step -- or of a pair of steps -- in one launch.  One workgroup per matrix keeps up to four 128 x 128 bf16
+// matrices in LDS (32 KB each, 16-byte chunks XOR-swizzled by row so that the 32 rows one fragment read touches
+// fall into different banks) and forms
+//   D  = r^2 sum_s partial_s - s I                       (what gram_reduce_kernel stores)
+//   R1 = c1 D^2 + (b1 + 2 c1 s) D                        single step: the result
+//   T' = R1 D + e1 D + s R1,  D2 = R1 T' + e1 T' + e1 s R1,  R2 = c2 D2^2 + (b2 + 2 c2 s2) D2,
+//   S  = R2 R1 + e2 R1 + e1 R2                           pair: the result
+// with the rounding points of the separate kernels: float32 accumulation, one rounding to bf16 per matrix, the lower
+// triangle computed and mirrored.
+// ---------------------------------------------------------------------------------------------
+static constexpr int CH_M = 128;                       // matrix size served
+static constexpr int CH_BYTES = CH_M * CH_M * 2;       // one matrix in LDS
+__device__ __forceinline__ int ch_off(int row, int chunk) { return row * (CH_M * 2) + (((chunk ^ row) & 15) << 4); }
+__device__ __forceinline__ int ch_elem(int row, int col) { return ch_off(row, col >> 3) + (col & 7) * 2; }
+
+// dst = alpha * P Q^T + beta1 * C1 + beta2 * C2 on the lower triangle, mirrored; all operands are LDS matrices.
+// Wavefront w of the 16 owns the 32 x 32 block (w / 4, w % 4); the six blocks above the diagonal are only ever
+// written as mirror images, so their wavefronts sit the product out.
+__device__ __forceinline__ void chain_product(const char* P, const char* Q, const char* C1, const char* C2, char* dst,
+                                              float alpha, float beta1, float beta2, int wave, int lane) {
+  const int ti = wave >> 2, tj = wave & 3;
+  if (tj <= ti) {
+    f32x16_t acc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = 0.0f;
+    const int frow = lane & 31, fk = lane >> 5;
+#pragma unroll
+    for (int q = 0; q < CH_M / 16; ++q) {
+      const bf16x8_t fp = *reinterpret_cast<const bf16x8_t*>(P + ch_off(ti * 32 + frow, 2 * q + fk));
+      const bf16x8_t fq = *reinterpret_cast<const bf16x8_t*>(Q + ch_off(tj * 32 + frow, 2 * q + fk));
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fq, fp, acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int m = ti * 32 + frow, n = tj * 32 + 8 * g + 4 * fk;
+      if (n > m) continue;  // all four columns lie above the diagonal
+      f32x4_t v;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) v[r] = alpha * acc[4 * g + r];
+      const uint2 c1 = *reinterpret_cast<const uint2*>(C1 + ch_elem(m, n));
+      v[0] = __builtin_fmaf(beta1, __uint_as_float(c1.x << 16), v[0]);
+      v[1] = __builtin_fmaf(beta1, __uint_as_float(c1.x & 0xffff0000u), v[1]);
+      v[2] = __builtin_fmaf(beta1, __uint_as_float(c1.y << 16), v[2]);
+      v[3] = __builtin_fmaf(beta1, __uint_as_float(c1.y & 0xffff0000u), v[3]);
+      if (C2 != nullptr) {
+        const uint2 c2 = *reinterpret_cast<const uint2*>(C2 + ch_elem(m, n));
+        v[0] = __builtin_fmaf(beta2, __uint_as_float(c2.x << 16), v[0]);
+        v[1] = __builtin_fmaf(beta2, __uint_as_float(c2.x & 0xffff0000u), v[1]);
+        v[2] = __builtin_fmaf(beta2, __uint_as_float(c2.y << 16), v[2]);
+        v[3] = __builtin_fmaf(beta2, __uint_as_float(c2.y & 0xffff0000u), v[3]);
+      }
+      const uint2 h = __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));
+      const uint16_t e[4] = {(uint16_t)(h.x & 0xffffu), (uint16_t)(h.x >> 16), (uint16_t)(h.y & 0xffffu), (uint16_t)(h.y >> 16)};
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (n + r <= m) *reinterpret_cast<uint16_t*>(dst + ch_elem(m, n + r)) = e[r];
+        if (n + r < m) *reinterpret_cast<uint16_t*>(dst + ch_elem(n + r, m)) = e[r];
+      }
+    }
+  }
+  __syncthreads();  // dst is complete, and nobody still reads what the next product overwrites
+}
+
+struct ChainArgs {
+  const float* partials;  // [batch][splits][128][128] float32
+  int splits;
+  const float* slots_in;  // partial sums of squares of X, [batch][nslots_in]
+  int nslots_in;
+  float* shift_io;        // [batch], written
+  const float* xscale;    // [batch] or null
+  float a1, b1, c1, a2, b2, c2;
+  int pair;
+  uint16_t* out;          // [batch][128][128] bf16: R1 (single step) or S (pair)
+};
+
+// 16 wavefronts per workgroup, one per 32 x 32 block of the products; together they stream the float32 partials in
+// (the only part that touches HBM; one workgroup per matrix leaves most of the chip idle, so each one needs many
+// loads in flight) and the result out.
+static constexpr int CH_THREADS = 1024;
+__global__ void __launch_bounds__(CH_THREADS) small_chain_kernel(ChainArgs a) {
+  __shared__ __align__(16) char chain_lds[4 * CH_BYTES];
+  __shared__ float red[CH_THREADS / 64];
+  const int64_t b = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  char* B0 = chain_lds;
+  char* B1 = chain_lds + CH_BYTES;
+  char* B2 = chain_lds + 2 * CH_BYTES;
+  char* B3 = chain_lds + 3 * CH_BYTES;
+  // shift and input scale of this matrix, as gram_reduce_kernel resolves them
+  float part = 0.0f;
+  for (int i = tid; i < a.nslots_in; i += CH_THREADS) part += a.slots_in[b * a.nslots_in + i];
+  const float s = block_sum_f32<CH_THREADS>(part, red) / (float)CH_M;
+  if (tid == 0) a.shift_io[b] = s;
+  const float r = a.xscale ? a.xscale[b] : 1.0f;
+  // D -> B0: four consecutive columns per thread and step, the slices added in their fixed order
+  const float* __restrict__ src = a.partials + b * a.splits * (int64_t)(CH_M * CH_M);
+  constexpr int GROUPS = CH_M * CH_M / 4, PER_THREAD = GROUPS / CH_THREADS, DEPTH = 4;
+  f32x4_t sum[PER_THREAD];
+#pragma unroll
+  for (int t = 0; t < PER_THREAD; ++t) sum[t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int sp0 = 0; sp0 < a.splits; sp0 += DEPTH) {
+    f32x4_t v[PER_THREAD][DEPTH];
+#pragma unroll
+    for (int t = 0; t < PER_THREAD; ++t) {
+      const int g = tid + t * CH_THREADS, i = g / (CH_M / 4), j = (g % (CH_M / 4)) * 4;
+#pragma unroll
+      for (int u = 0; u < DEPTH; ++u) {
+        v[t][u] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        if (j <= i && sp0 + u < a.splits)
+          v[t][u] = *reinterpret_cast<const f32x4_t*>(src + (int64_t)(sp0 + u) * (CH_M * CH_M) + (int64_t)g * 4);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < PER_THREAD; ++t)
+#pragma unroll
+      for (int u = 0; u < DEPTH; ++u)
+        if (sp0 + u < a.splits) sum[t] += v[t][u];
+  }
+#pragma unroll
+  for (int t = 0; t < PER_THREAD; ++t) {
+    const int g = tid + t * CH_THREADS, i = g / (CH_M / 4), j = (g % (CH_M / 4)) * 4;
+    if (j > i) continue;  // the whole group lies above the diagonal
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (j + e > i) continue;
+      float acc = sum[t][e] * (r * r);
+      if (i == j + e) acc -= s;
+      const uint16_t h = __builtin_bit_cast(uint16_t, (__bf16)acc);
+      *reinterpret_cast<uint16_t*>(B0 + ch_elem(i, j + e)) = h;
+      *reinterpret_cast<uint16_t*>(B0 + ch_elem(j + e, i)) = h;
+    }
+  }
+  __syncthreads();
+  const float e1 = a.a1 + a.b1 * s + a.c1 * s * s;
+  // R1 = c1 D^2 + (b1 + 2 c1 s) D -> B1
+  chain_product(B0, B0, B0, nullptr, B1, a.c1, a.b1 + 2.0f * a.c1 * s, 0.0f, wave, lane);
+  const char* result = B1;
+  if (a.pair) {
+    const float s2 = e1 * e1 * s;
+    const float e2 = a.a2 + a.b2 * s2 + a.c2 * s2 * s2;
+    chain_product(B1, B0, B0, B1, B2, 1.0f, e1, s, wave, lane);                               // T' -> B2
+    chain_product(B1, B2, B2, B1, B3, 1.0f, e1, e1 * s, wave, lane);                          // D2 -> B3
+    chain_product(B3, B3, B3, nullptr, B0, a.c2, a.b2 + 2.0f * a.c2 * s2, 0.0f, wave, lane);  // R2 -> B0
+    chain_product(B0, B1, B1, B0, B2, 1.0f, e2, e1, wave, lane);                              // S  -> B2
+    result = B2;
+  }
+  uint16_t* __restrict__ ob = a.out + b * (int64_t)(CH_M * CH_M);
+  for (int c = tid; c < CH_M * (CH_M / 8); c += CH_THREADS) {
+    const int row = c / (CH_M / 8), ch = c % (CH_M / 8);
+    *reinterpret_cast<uint4*>(ob + row * CH_M + ch * 8) = *reinterpret_cast<const uint4*>(result + ch_off(row, ch));
+  }
+}
+
 #ifdef MI_HAS_SMALL_CFGS
-static int small_gram(const uint16_t* X, int64_t batch, int64_t m, int64_t n, int splits, float* partials,
-                      const float* slots_in, int nslots_in, float* shift_io, uint16_t* gram, hipStream_t stream,
-                      const float* xscale) {
+// Split-K partial Gram matrices: the K range is cut into `splits` slices that run as extra batch entries.
+static int small_gram_partials(const uint16_t* X, int64_t batch, int64_t m, int64_t n, int splits, float* partials,
+                               hipStream_t stream) {
   GemmParams p{};
   p.P = p.Q = X;
   p.ldp = p.ldq = n;
@@ -870,12 +1025,41 @@ static int small_gram(const uint16_t* X, int64_t batch, int64_t m, int64_t n, in
   p.alpha = 1.0f;
   p.beta = 0.0f;
   p.out_scale = 1.0f;
-  int rc = launch_fast<CfgT128, false, false, MODE_GEMM, true>(p, batch * splits, stream);
+  return launch_fast<CfgT128, false, false, MODE_GEMM, true>(p, batch * splits, stream);
+}
+
+static int small_gram(const uint16_t* X, int64_t batch, int64_t m, int64_t n, int splits, float* partials,
+                      const float* slots_in, int nslots_in, float* shift_io, uint16_t* gram, hipStream_t stream,
+                      const float* xscale) {
+  int rc = small_gram_partials(X, batch, m, n, splits, partials, stream);
   if (rc != MI_OK) return rc;
   dim3 grid((unsigned)((m * m + 255) / 256), (unsigned)batch), block(256);
   hipLaunchKernelGGL(gram_reduce_kernel, grid, block, 0, stream, partials, splits, (int)m, slots_in, nslots_in, shift_io, gram, xscale);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "gram_reduce launch failed: %s", hipGetErrorString(e));
+  return MI_OK;
+}
+
+// Partials, then everything up to the multiplier of the B X product in one launch (128-row matrices only).
+static int small_chain(const uint16_t* X, int64_t batch, int64_t n, int splits, float* partials, const float* slots_in,
+                       int nslots_in, float* shift_io, const float* xscale, const float* abc1, const float* abc2,
+                       uint16_t* out, hipStream_t stream) {
+  int rc = small_gram_partials(X, batch, CH_M, n, splits, partials, stream);
+  if (rc != MI_OK) return rc;
+  ChainArgs a{};
+  a.partials = partials;
+  a.splits = splits;
+  a.slots_in = slots_in;
+  a.nslots_in = nslots_in;
+  a.shift_io = shift_io;
+  a.xscale = xscale;
+  a.a1 = abc1[0], a.b1 = abc1[1], a.c1 = abc1[2];
+  a.pair = abc2 != nullptr;
+  if (abc2) a.a2 = abc2[0], a.b2 = abc2[1], a.c2 = abc2[2];
+  a.out = out;
+  hipLaunchKernelGGL(small_chain_kernel, dim3((unsigned)batch), dim3(CH_THREADS), 0, stream, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "small_chain launch failed: %s", hipGetErrorString(e));
   return MI_OK;
 }
 #endif
@@ -999,59 +1183,80 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
     const int taken = pair ? 2 : 1;
     const bool last = (s + taken == steps);
     want_pair = !pair;
-    // A' = X X^T - s I  (s = ||X||_F^2 / m from the partial sums the previous kernel left)
-    ShiftArgs sh_gram{SHIFT_GRAM, b, c, slots, nslots, shift, nullptr};
     const float* xs = (s == 0) ? xscale : nullptr;  // only the input of the first group is unnormalised
-    sh_gram.xscale = xs;
-    {
-      ProfScope prof(PROF_GRAM, stream);
-#ifdef MI_HAS_SMALL_CFGS
-      if (w.gram_splits > 0)
-        rc = small_gram(xbuf[cur], batch, m, n, w.gram_splits, reinterpret_cast<float*>(ws + w.gpart), slots, nslots, shift,
-                        gram, stream, xs);
-      else
-#endif
-        rc = syrk_impl(xbuf[cur], batch, m, n, x_bs, ld, trans, nullptr, 0, m, 1.0f, 0.0f, gram, g_bs, m, 0, stream, &sh_gram);
-    }
-    if (rc != MI_OK) return rc;
     const uint16_t* mult = gram;
     float alpha = b;
-    if (c != 0.0f) {
-      // B' = c A'^2 + (b + 2 c s) A'
-      ShiftArgs sh_poly{SHIFT_POLY, b, c, nullptr, 0, shift, nullptr};
-      {
-        ProfScope prof(PROF_POLY, stream);
-        rc = syrk_impl(gram, batch, m, m, g_bs, m, 0, gram, g_bs, m, c, b, poly, g_bs, m, 0, stream, &sh_poly);
-      }
-      if (rc != MI_OK) return rc;
-      mult = poly;
-      alpha = 1.0f;
-    }
     int apply_mode = SHIFT_APPLY;
     float a2 = 0.0f, b2 = 0.0f, c2 = 0.0f;
-    if (pair) {
-      // The second step on the same Gram matrix: four products of commuting symmetric m x m matrices (the host
-      // coefficient 1 of each addend is replaced on the device, where the shift is known).
-      a2 = abc[3 * s + 3], b2 = abc[3 * s + 4], c2 = abc[3 * s + 5];
-      uint16_t* tbuf = reinterpret_cast<uint16_t*>(ws + w.t);
-      uint16_t* d2 = reinterpret_cast<uint16_t*>(ws + w.d2);
-      auto product = [&](int mode, const uint16_t* left, const uint16_t* right, const uint16_t* add2, float al, float be,
-                         uint16_t* dst) {
-        ShiftArgs sh{mode, b, c, nullptr, 0, shift, nullptr, a, a2, b2, c2};
-        ProfScope prof(PROF_POLY, stream);
-        return syrk_impl(left, batch, m, m, g_bs, m, 0, right, g_bs, m, al, be, dst, g_bs, m, 0, stream, &sh,
-                         right == left ? nullptr : right, add2);
-      };
-      // T' = R1 D + e1 D + s R1
-      if ((rc = product(SHIFT_PAIR_T, poly, gram, poly, 1.0f, 1.0f, tbuf)) != MI_OK) return rc;
-      // D2 = R1 T' + e1 T' + e1 s R1
-      if ((rc = product(SHIFT_PAIR_A2, poly, tbuf, poly, 1.0f, 1.0f, d2)) != MI_OK) return rc;
-      // R2 = c2 D2^2 + (b2 + 2 c2 s2) D2     (D is no longer needed: its buffer takes R2)
-      if ((rc = product(SHIFT_PAIR_POLY2, d2, d2, nullptr, c2, b2, gram)) != MI_OK) return rc;
-      // S = R2 R1 + e2 R1 + e1 R2            (T' is no longer needed)
-      if ((rc = product(SHIFT_PAIR_Q, gram, poly, gram, 1.0f, 1.0f, tbuf)) != MI_OK) return rc;
-      mult = tbuf;
-      apply_mode = SHIFT_PAIR_APPLY;
+    if (pair) a2 = abc[3 * s + 3], b2 = abc[3 * s + 4], c2 = abc[3 * s + 5];
+#ifdef MI_HAS_SMALL_CFGS
+    const bool chain = w.gram_splits > 0 && m == CH_M && c != 0.0f;
+#else
+    const bool chain = false;
+#endif
+    if (chain) {
+#ifdef MI_HAS_SMALL_CFGS
+      // 128-row matrices: Gram partials, then one launch per matrix for everything up to the multiplier of X
+      uint16_t* dst_mult = pair ? reinterpret_cast<uint16_t*>(ws + w.t) : poly;
+      {
+        ProfScope prof(PROF_GRAM, stream);
+        rc = small_chain(xbuf[cur], batch, n, w.gram_splits, reinterpret_cast<float*>(ws + w.gpart), slots, nslots, shift, xs,
+                         abc + 3 * s, pair ? abc + 3 * s + 3 : nullptr, dst_mult, stream);
+      }
+      if (rc != MI_OK) return rc;
+      mult = dst_mult;
+      alpha = 1.0f;
+      if (pair) apply_mode = SHIFT_PAIR_APPLY;
+#endif
+    } else {
+      // A' = X X^T - s I  (s = ||X||_F^2 / m from the partial sums the previous kernel left)
+      ShiftArgs sh_gram{SHIFT_GRAM, b, c, slots, nslots, shift, nullptr};
+      sh_gram.xscale = xs;
+      {
+        ProfScope prof(PROF_GRAM, stream);
+#ifdef MI_HAS_SMALL_CFGS
+        if (w.gram_splits > 0)
+          rc = small_gram(xbuf[cur], batch, m, n, w.gram_splits, reinterpret_cast<float*>(ws + w.gpart), slots, nslots, shift,
+                          gram, stream, xs);
+        else
+#endif
+          rc = syrk_impl(xbuf[cur], batch, m, n, x_bs, ld, trans, nullptr, 0, m, 1.0f, 0.0f, gram, g_bs, m, 0, stream, &sh_gram);
+      }
+      if (rc != MI_OK) return rc;
+      if (c != 0.0f) {
+        // B' = c A'^2 + (b + 2 c s) A'
+        ShiftArgs sh_poly{SHIFT_POLY, b, c, nullptr, 0, shift, nullptr};
+        {
+          ProfScope prof(PROF_POLY, stream);
+          rc = syrk_impl(gram, batch, m, m, g_bs, m, 0, gram, g_bs, m, c, b, poly, g_bs, m, 0, stream, &sh_poly);
+        }
+        if (rc != MI_OK) return rc;
+        mult = poly;
+        alpha = 1.0f;
+      }
+      if (pair) {
+        // The second step on the same Gram matrix: four products of commuting symmetric m x m matrices (the host
+        // coefficient 1 of each addend is replaced on the device, where the shift is known).
+        uint16_t* tbuf = reinterpret_cast<uint16_t*>(ws + w.t);
+        uint16_t* d2 = reinterpret_cast<uint16_t*>(ws + w.d2);
+        auto product = [&](int mode, const uint16_t* left, const uint16_t* right, const uint16_t* add2, float al, float be,
+                           uint16_t* dst) {
+          ShiftArgs sh{mode, b, c, nullptr, 0, shift, nullptr, a, a2, b2, c2};
+          ProfScope prof(PROF_POLY, stream);
+          return syrk_impl(left, batch, m, m, g_bs, m, 0, right, g_bs, m, al, be, dst, g_bs, m, 0, stream, &sh,
+                           right == left ? nullptr : right, add2);
+        };
+        // T' = R1 D + e1 D + s R1
+        if ((rc = product(SHIFT_PAIR_T, poly, gram, poly, 1.0f, 1.0f, tbuf)) != MI_OK) return rc;
+        // D2 = R1 T' + e1 T' + e1 s R1
+        if ((rc = product(SHIFT_PAIR_A2, poly, tbuf, poly, 1.0f, 1.0f, d2)) != MI_OK) return rc;
+        // R2 = c2 D2^2 + (b2 + 2 c2 s2) D2     (D is no longer needed: its buffer takes R2)
+        if ((rc = product(SHIFT_PAIR_POLY2, d2, d2, nullptr, c2, b2, gram)) != MI_OK) return rc;
+        // S = R2 R1 + e2 R1 + e1 R2            (T' is no longer needed)
+        if ((rc = product(SHIFT_PAIR_Q, gram, poly, gram, 1.0f, 1.0f, tbuf)) != MI_OK) return rc;
+        mult = tbuf;
+        apply_mode = SHIFT_PAIR_APPLY;
+      }
     }
     // X' = (a + b s + c s^2) X + B' X      (cubic: (a + b s) X + b A' X;  pair: e1 e2 X + S X)
     void* dst = last ? static_cast<void*>(result) : static_cast<void*>(xbuf[cur ^ 1]);
