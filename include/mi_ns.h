@@ -117,6 +117,15 @@ size_t mi_frob_partials_len(int64_t batch, int64_t numel);
  * steps == 0 returns the normalised input.  rows and cols must be multiples of 8.
  * workspace: device scratch of at least mi_newton_schulz_workspace_bytes(batch, rows, cols) bytes,
  * 256-byte aligned.
+ *
+ * Two things differ from a literal step-by-step execution, neither of which changes the function computed:
+ *  - the input is cast to bf16 by the pass that sums its squares, and 1 / norm enters the first two products
+ *    as a device scalar (norms outside [1e-10, 1e10] are divided out before the cast instead);
+ *  - for matrices with at least 1024 rows and twice as many columns, and for 128/256-row matrices at least four
+ *    times as wide, consecutive quintic steps are taken two at a time on one Gram matrix (all factors are
+ *    polynomials of X X^T and commute): 5 steps run as 2 + 1 + 2.  The environment variable MI_NS_PAIRS, read at
+ *    every call (and by mi_newton_schulz_workspace_bytes), overrides this: "0" = one step at a time, "force" = pairs
+ *    at every size.
  */
 int mi_newton_schulz_bf16(const float* x, float* out, int64_t batch, int64_t rows, int64_t cols,
                           const float* abc, int steps, float eps, int accumulate_fp64,
@@ -135,9 +144,8 @@ size_t mi_newton_schulz_workspace_bytes(int64_t batch, int64_t rows, int64_t col
  *   emerging_optimizers/orthogonalized_optimizers/orthogonalized_optimizer.py:185-210
  * together with Muon's closure (muon.py:117-132): param_decay = 1 - wd*lr (decoupled), 1 - wd (independent),
  * 1 - wd*lr^2 (palm), 1 (no decay); update_scale = -lr * get_muon_scale_factor(...) * extra_scale_factor.
- * The momentum update and the sum of squares share one pass over grad and momentum, the divide + bf16 cast
- * recomputes d in a second pass, and the last GEMM epilogue (or the final transpose of a tall parameter)
- * updates param in place.  param, grad, momentum: float32 (batch, rows, cols) row-major contiguous, distinct
+ * The momentum update, the sum of squares and the bf16 cast of d share one pass over grad and momentum, and the
+ * last GEMM epilogue (or the final transpose of a tall parameter) updates param in place.  param, grad, momentum: float32 (batch, rows, cols) row-major contiguous, distinct
  * buffers.  Other arguments and the workspace as for mi_newton_schulz_bf16; steps >= 1; param_decay != 0.
  */
 int mi_muon_update_bf16(float* param, const float* grad, float* momentum, int64_t batch, int64_t rows, int64_t cols,
