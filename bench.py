@@ -325,13 +325,13 @@ def main():
     f_sym = NS_STEPS * (3 * M * M * N + M**3)
     f_full = NS_STEPS * (4 * M * M * N + 2 * M**3)
     tflops = f_sym / (ms_per_step * 1e-3) / 1e12
-    # What the driver executes: wide matrices take the steps as 2 + 1 + 2, where a pair of steps shares one
-    # X X^T and one B X and pays six m x m symmetric products instead of two (same result within the tolerance,
-    # checked below against float32).  MI_NS_PAIRS=0 restores one X X^T and one B X per step.
-    paired = os.environ.get("MI_NS_PAIRS", "")[:1] != "0" and M >= 1024 and N >= 2 * M
-    n_pairs = 2 if (paired and NS_STEPS == 5) else 0
-    f_exec = (NS_STEPS - n_pairs) * 3 * M * M * N + (NS_STEPS - 2 * n_pairs) * M**3 + n_pairs * 6 * M**3
-
+    # What the driver executes: wide matrices take the five steps as 3 + 2 (2 + 1 + 2 under MI_NS_PAIRS=pairs), where a
+    # group of g steps shares one X X^T and one B X and pays 4 g - 3 symmetric m x m products (same result within the
+    # tolerance, checked below against float32).  MI_NS_PAIRS=0 restores one X X^T and one B X per step.
+    env = os.environ.get("MI_NS_PAIRS", "")[:1]
+    wide = M >= 1024 and N >= 2 * M and NS_STEPS == 5
+    schedule = [1] * NS_STEPS if (env == "0" or not wide) else [2, 1, 2] if env in ("p", "f") else [3, 2]
+    f_exec = sum(3 * M * M * N + (4 * g - 3) * M**3 for g in schedule)
     # parity gate in the same job: float32 Newton-Schulz with torch on the GPU
     torch.set_float32_matmul_precision("highest")
     X = x / x.norm()
@@ -365,7 +365,7 @@ def main():
             "(N(0,1e-3^2) with 1% entries at 50 sigma), bf16 MFMA kernels with fp32 accumulation, float32 result",
             "flops_counted": "symmetric-halved 5*(3 m^2 n + m^3): the count of five ordinary steps, whatever the schedule",
             "tflops_full_count": round(f_full / (ms_per_step * 1e-3) / 1e12, 2),
-            "schedule": "2+1+2: steps 1-2 and 4-5 each share one Gram matrix" if n_pairs else "1+1+1+1+1",
+            "schedule": "+".join(map(str, schedule)) + " (steps of one group share one Gram matrix)",
             "tflops_executed": round(f_exec / (ms_per_step * 1e-3) / 1e12, 2),
             "launches_per_call": {n: n_kind[i] // args.steps for i, n in enumerate(["normalize_cast", "syrk_gram", "syrk_poly", "gemm_axpy"])},
             "pct_of_bf16_mfma_peak": round(100.0 * tflops / PEAK_BF16_TFLOPS, 2),

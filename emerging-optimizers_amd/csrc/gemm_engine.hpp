@@ -51,7 +51,8 @@ struct GemmParams {
   // the epilogue scalars of the two kernels that consume A', which keeps the algebra exact for any s.
   int shift_mode;            // SHIFT_*
   float ca, cb, cc;          // step coefficients a, b, c (host values)
-  float ca2, cb2, cc2;       // SHIFT_PAIR_*: coefficients of the second step of a pair
+  float co[3][3];            // SHIFT_GROUP_*: (a, b, c) of up to three steps that share one Gram matrix
+  int stage;                 // SHIFT_GROUP_*: which of them this launch belongs to (0-based)
   const float* slots_in;     // SHIFT_GRAM: per-tile partial sums of squares of X, [batch][nslots_in]
   int nslots_in;
   float* shift_io;           // [batch]: written by SHIFT_GRAM, read by SHIFT_POLY / SHIFT_APPLY
@@ -62,18 +63,18 @@ struct GemmParams {
   int slot_stride, slot_base;  //   at slots_out[batch * slot_stride + slot_base + blockIdx.x]
 };
 
-// Two consecutive steps can share one Gram matrix, because every factor involved is a polynomial of it and
-// they all commute.  With A = s I + D (D stored), step 1 = (a1, b1, c1), step 2 = (a2, b2, c2):
-//   R1 = c1 D^2 + (b1 + 2 c1 s) D                 q1 = e1 I + R1,  e1 = a1 + b1 s + c1 s^2      [SHIFT_POLY]
-//   T  = q1 A   = e1 s I + T',   T'  = R1 D  + e1 D  + s R1                                      [SHIFT_PAIR_T]
-//   A2 = q1 T   = s2 I + D2,     D2  = R1 T' + e1 T' + e1 s R1,    s2 = e1^2 s                   [SHIFT_PAIR_A2]
-//   R2 = c2 D2^2 + (b2 + 2 c2 s2) D2              q2 = e2 I + R2,  e2 = a2 + b2 s2 + c2 s2^2    [SHIFT_PAIR_POLY2]
-//   q2 q1 = e1 e2 I + S,         S   = R2 R1 + e2 R1 + e1 R2                                     [SHIFT_PAIR_Q]
-//   X'' = e1 e2 X + S X                                                                          [SHIFT_PAIR_APPLY]
-// which replaces the second step's X X^T and one of the two B X products by four m x m products.
+// Consecutive steps can share one Gram matrix, because every factor involved is a polynomial of it and they all
+// commute.  With A_k = s_k I + D_k (D_k stored), step k = (a_k, b_k, c_k), q_k = e_k I + R_k its multiplier and
+// Q_k = q_k ... q_1 = alpha_k I + S_k the accumulated one (alpha_k = e_1 ... e_k, S_1 = R_1):
+//   R_k  = c_k D_k^2 + (b_k + 2 c_k s_k) D_k,   e_k = a_k + b_k s_k + c_k s_k^2                [SHIFT_GROUP_POLY]
+//   S_k  = R_k S_{k-1} + e_k S_{k-1} + alpha_{k-1} R_k                          (k > 1)        [SHIFT_GROUP_Q]
+//   T'_k = R_k D_k + e_k D_k + s_k R_k                           (q_k A_k minus its identity)  [SHIFT_GROUP_T]
+//   D_{k+1} = R_k T'_k + e_k T'_k + e_k s_k R_k,  s_{k+1} = e_k^2 s_k     (A_{k+1} = q_k^2 A_k) [SHIFT_GROUP_A]
+//   X' = alpha_g X + S_g X  after the last step g of the group                                 [SHIFT_GROUP_APPLY]
+// A group of g steps costs one X X^T, one B X and 4 g - 3 products of m x m matrices instead of g of each.
 enum {
   SHIFT_NONE = 0, SHIFT_GRAM = 1, SHIFT_POLY = 2, SHIFT_APPLY = 3,
-  SHIFT_PAIR_T = 4, SHIFT_PAIR_A2 = 5, SHIFT_PAIR_POLY2 = 6, SHIFT_PAIR_Q = 7, SHIFT_PAIR_APPLY = 8
+  SHIFT_GROUP_POLY = 4, SHIFT_GROUP_T = 5, SHIFT_GROUP_A = 6, SHIFT_GROUP_Q = 7, SHIFT_GROUP_APPLY = 8
 };
 
 // Byte offset of 16-byte chunk `chunk` of row `row` in an LDS tile whose rows hold BK bf16 values.
@@ -274,14 +275,25 @@ __device__ __forceinline__ Scalars resolve_shift(const GemmParams& p, int64_t ba
   } else if (p.shift_mode == SHIFT_APPLY) {
     s = p.shift_io[batch];
     beta = beta + p.cb * s + p.cc * s * s;  // X' = (a + b s + c s^2) X + B' X
-  } else if (p.shift_mode >= SHIFT_PAIR_T) {
+  } else if (p.shift_mode >= SHIFT_GROUP_POLY) {
     s = p.shift_io[batch];
-    const float e1 = p.ca + p.cb * s + p.cc * s * s;
-    const float s2 = e1 * e1 * s;
-    const float e2 = p.ca2 + p.cb2 * s2 + p.cc2 * s2 * s2;
+    // walk the recursion up to this launch's step: sk = s_k, e = e_k, before = alpha_{k-1}
+    float sk = s, before = 1.0f, e = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+      if (j > p.stage) break;
+      e = p.co[j][0] + p.co[j][1] * sk + p.co[j][2] * sk * sk;
+      if (j < p.stage) {
+        before *= e;
+        sk = e * e * sk;
+      }
+    }
     const int mode = p.shift_mode;
-    beta = mode == SHIFT_PAIR_POLY2 ? p.cb2 + 2.0f * p.cc2 * s2 : mode == SHIFT_PAIR_Q ? e2 : mode == SHIFT_PAIR_APPLY ? e1 * e2 : e1;
-    beta2 = mode == SHIFT_PAIR_T ? s : mode == SHIFT_PAIR_A2 ? e1 * s : mode == SHIFT_PAIR_Q ? e1 : beta2;
+    // (selects instead of p.co[p.stage]: a dynamically indexed kernel argument would be copied to scratch)
+    const float bk = p.stage == 0 ? p.co[0][1] : p.stage == 1 ? p.co[1][1] : p.co[2][1];
+    const float ck = p.stage == 0 ? p.co[0][2] : p.stage == 1 ? p.co[1][2] : p.co[2][2];
+    beta = mode == SHIFT_GROUP_POLY ? bk + 2.0f * ck * sk : mode == SHIFT_GROUP_APPLY ? before * e : e;
+    beta2 = mode == SHIFT_GROUP_T ? sk : mode == SHIFT_GROUP_A ? e * sk : mode == SHIFT_GROUP_Q ? before : beta2;
   }
   if (p.xscale != nullptr) {
     const float r = p.xscale[batch];

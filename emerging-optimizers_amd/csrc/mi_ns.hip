@@ -215,17 +215,18 @@ struct ShiftArgs {
   int nslots_in;
   float* shift_io;
   float* slots_out;
-  float ca = 0.0f, ca2 = 0.0f, cb2 = 0.0f, cc2 = 0.0f;  // SHIFT_PAIR_*: a of the first step and (a, b, c) of the second
+  const float* group_abc = nullptr;  // SHIFT_GROUP_*: (a, b, c) of the steps of the group, 3 floats each
+  int group_size = 0, stage = 0;
   const float* xscale = nullptr;  // first group of steps on an unnormalised X
   void apply(GemmParams& p) const {
     p.shift_mode = mode;
     p.xscale = xscale;
-    p.ca = ca;
+    p.ca = 0.0f;
     p.cb = cb;
     p.cc = cc;
-    p.ca2 = ca2;
-    p.cb2 = cb2;
-    p.cc2 = cc2;
+    for (int j = 0; j < 3; ++j)
+      for (int e = 0; e < 3; ++e) p.co[j][e] = (group_abc && j < group_size) ? group_abc[3 * j + e] : 0.0f;
+    p.stage = stage;
     p.slots_in = slots_in;
     p.nslots_in = nslots_in;
     p.shift_io = shift_io;
@@ -238,7 +239,7 @@ struct ShiftArgs {
 // D = alpha * A A^T + beta * C, bf16 out.
 // Inside the fused driver the same lower-triangle kernel also forms products of two commuting symmetric matrices:
 // `other` != null computes alpha * A other^T (symmetric in exact arithmetic; the lower triangle is computed and
-// mirrored), and `C2` is a second addend laid out like C whose coefficient a SHIFT_PAIR_* mode supplies.
+// mirrored), and `C2` is a second addend laid out like C whose coefficient a SHIFT_GROUP_* mode supplies.
 static int syrk_impl(const void* A, int64_t batch, int64_t n, int64_t k, int64_t a_bs, int64_t a_ld, int a_trans,
                      const void* C, int64_t c_bs, int64_t c_ld, float alpha, float beta, void* D, int64_t d_bs,
                      int64_t d_ld, int skip_upper, hipStream_t stream, const ShiftArgs* sh = nullptr,
@@ -1073,18 +1074,38 @@ struct NsWorkspace {
   int64_t max_slots;
 };
 
-// Whether two consecutive steps share one Gram matrix (see SHIFT_PAIR_* in gemm_engine.hpp).  A pair trades one
-// X X^T and one B X (3 m^2 n multiply-adds) for four m x m products, which pays for wide matrices only; a pair on a
-// square matrix would also sit close to the 1e-2 tolerance; below 1024 rows the kernels are launch-bound and a pair
-// has more launches, except on the split-K Gram path.  MI_NS_PAIRS=0 switches pairing off, MI_NS_PAIRS=force
-// pairs wherever the kernels allow it (used by the tests to reach the pair kernels with small matrices).
+// Whether consecutive steps share one Gram matrix (see SHIFT_GROUP_* in gemm_engine.hpp): 0 = never, 1 = pairs,
+// 2 = pairs, and the first three steps as one group.  A group of g steps trades g - 1 X X^T and g - 1 B X products
+// (3 m^2 n multiply-adds each time) for 4 (g - 1) products of m x m matrices, which pays for wide matrices only; on
+// a square matrix it would also sit close to the 1e-2 tolerance; below 1024 rows the kernels are launch-bound and a
+// group has more launches, except on the split-K Gram path.  MI_NS_PAIRS=0 switches grouping off, MI_NS_PAIRS=pairs
+// keeps the rule but never takes three steps at once, MI_NS_PAIRS=force pairs wherever the kernels allow it (used
+// by the tests to reach the pair kernels with small matrices).
 static int ns_pairs_enabled(int64_t m, int64_t n, int gram_splits) {
   const char* env = getenv("MI_NS_PAIRS");
   if (env && env[0] == '0') return 0;
   if (env && env[0] == 'f') return 1;
   // (the split-K Gram path serves short matrices at least four times as wide as tall: a pair there trades two
   // passes over X for four tiny products at the same number of launches)
-  return gram_splits > 0 || (m >= 1024 && n >= 2 * m);
+  if (gram_splits > 0) return 1;
+  if (m >= 1024 && n >= 2 * m) return (env && env[0] == 'p') ? 1 : 2;
+  return 0;
+}
+
+// Size of the group of steps that starts at step s.  Pairs alternate with single steps (two pairs in a row from
+// the start lose accuracy on flat spectra).  Three steps go together only at the very start, where the steps that
+// follow damp what the longer chain of m x m products adds, and only if the rounding noise of the first Gram matrix
+// is not amplified too much on the way to the third (by (a_1 a_2)^2 in the directions of small singular values:
+// 141 for the "simple" coefficients, 260 for "quintic", above 1000 for "polar_express" and "cans").
+static int ns_group_size(int mode, const float* abc, int steps, int s, bool want_group) {
+  if (!mode || !want_group || s + 1 >= steps) return 1;
+  auto quintic = [&](int k) { return abc[3 * k + 2] != 0.0f; };
+  if (!quintic(s) || !quintic(s + 1)) return 1;
+  if (mode == 2 && s == 0 && steps >= 5 && quintic(2)) {
+    const double amp = (double)abc[0] * abc[3];
+    if (amp * amp <= 400.0) return 3;
+  }
+  return 2;
 }
 
 static NsWorkspace ns_layout(int64_t batch, int64_t rows, int64_t cols) {
@@ -1176,37 +1197,34 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
 
   int cur = 0;
   int nslots = 1;  // the normalisation kernel left one value per matrix
-  bool want_pair = true;  // pairs alternate with single steps: two pairs in a row lose accuracy on flat spectra
+  bool want_group = true;
   for (int s = 0; s < steps;) {
     const float a = abc[3 * s], b = abc[3 * s + 1], c = abc[3 * s + 2];
-    const bool pair = w.pairs && want_pair && s + 1 < steps && c != 0.0f && abc[3 * s + 5] != 0.0f;
-    const int taken = pair ? 2 : 1;
+    const int taken = ns_group_size(w.pairs, abc, steps, s, want_group);
     const bool last = (s + taken == steps);
-    want_pair = !pair;
+    want_group = taken != 2;  // a pair is followed by a single step; the opening triple may be followed by a pair
     const float* xs = (s == 0) ? xscale : nullptr;  // only the input of the first group is unnormalised
     const uint16_t* mult = gram;
     float alpha = b;
     int apply_mode = SHIFT_APPLY;
-    float a2 = 0.0f, b2 = 0.0f, c2 = 0.0f;
-    if (pair) a2 = abc[3 * s + 3], b2 = abc[3 * s + 4], c2 = abc[3 * s + 5];
 #ifdef MI_HAS_SMALL_CFGS
-    const bool chain = w.gram_splits > 0 && m == CH_M && c != 0.0f;
+    const bool chain = w.gram_splits > 0 && m == CH_M && c != 0.0f && taken <= 2;
 #else
     const bool chain = false;
 #endif
     if (chain) {
 #ifdef MI_HAS_SMALL_CFGS
       // 128-row matrices: Gram partials, then one launch per matrix for everything up to the multiplier of X
-      uint16_t* dst_mult = pair ? reinterpret_cast<uint16_t*>(ws + w.t) : poly;
+      uint16_t* dst_mult = taken == 2 ? reinterpret_cast<uint16_t*>(ws + w.t) : poly;
       {
         ProfScope prof(PROF_GRAM, stream);
         rc = small_chain(xbuf[cur], batch, n, w.gram_splits, reinterpret_cast<float*>(ws + w.gpart), slots, nslots, shift, xs,
-                         abc + 3 * s, pair ? abc + 3 * s + 3 : nullptr, dst_mult, stream);
+                         abc + 3 * s, taken == 2 ? abc + 3 * s + 3 : nullptr, dst_mult, stream);
       }
       if (rc != MI_OK) return rc;
       mult = dst_mult;
       alpha = 1.0f;
-      if (pair) apply_mode = SHIFT_PAIR_APPLY;
+      if (taken == 2) apply_mode = SHIFT_GROUP_APPLY;
 #endif
     } else {
       // A' = X X^T - s I  (s = ||X||_F^2 / m from the partial sums the previous kernel left)
@@ -1223,48 +1241,76 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
           rc = syrk_impl(xbuf[cur], batch, m, n, x_bs, ld, trans, nullptr, 0, m, 1.0f, 0.0f, gram, g_bs, m, 0, stream, &sh_gram);
       }
       if (rc != MI_OK) return rc;
-      if (c != 0.0f) {
-        // B' = c A'^2 + (b + 2 c s) A'
-        ShiftArgs sh_poly{SHIFT_POLY, b, c, nullptr, 0, shift, nullptr};
-        {
-          ProfScope prof(PROF_POLY, stream);
-          rc = syrk_impl(gram, batch, m, m, g_bs, m, 0, gram, g_bs, m, c, b, poly, g_bs, m, 0, stream, &sh_poly);
+      if (taken == 1) {
+        if (c != 0.0f) {
+          // B' = c A'^2 + (b + 2 c s) A'
+          ShiftArgs sh_poly{SHIFT_POLY, b, c, nullptr, 0, shift, nullptr};
+          {
+            ProfScope prof(PROF_POLY, stream);
+            rc = syrk_impl(gram, batch, m, m, g_bs, m, 0, gram, g_bs, m, c, b, poly, g_bs, m, 0, stream, &sh_poly);
+          }
+          if (rc != MI_OK) return rc;
+          mult = poly;
+          alpha = 1.0f;
         }
-        if (rc != MI_OK) return rc;
-        mult = poly;
-        alpha = 1.0f;
-      }
-      if (pair) {
-        // The second step on the same Gram matrix: four products of commuting symmetric m x m matrices (the host
-        // coefficient 1 of each addend is replaced on the device, where the shift is known).
-        uint16_t* tbuf = reinterpret_cast<uint16_t*>(ws + w.t);
-        uint16_t* d2 = reinterpret_cast<uint16_t*>(ws + w.d2);
-        auto product = [&](int mode, const uint16_t* left, const uint16_t* right, const uint16_t* add2, float al, float be,
+      } else {
+        // Several steps on this Gram matrix: products of commuting symmetric m x m matrices (SHIFT_GROUP_* in
+        // gemm_engine.hpp; the host coefficient 1 of each addend is replaced on the device, where the shift is
+        // known).  Four buffers go round: D_k stays in `gram`, the others are handed out and returned as the
+        // matrices they hold die.
+        uint16_t* pool[3] = {poly, reinterpret_cast<uint16_t*>(ws + w.t), reinterpret_cast<uint16_t*>(ws + w.d2)};
+        int free_n = 3;
+        auto take = [&]() { return pool[--free_n]; };
+        auto give = [&](uint16_t* buf) { pool[free_n++] = buf; };
+        auto product = [&](int mode, int stage, const uint16_t* left, const uint16_t* right, const uint16_t* add2, float al,
                            uint16_t* dst) {
-          ShiftArgs sh{mode, b, c, nullptr, 0, shift, nullptr, a, a2, b2, c2};
+          ShiftArgs sh{mode, b, c, nullptr, 0, shift, nullptr};
+          sh.group_abc = abc + 3 * s;
+          sh.group_size = taken;
+          sh.stage = stage;
           ProfScope prof(PROF_POLY, stream);
-          return syrk_impl(left, batch, m, m, g_bs, m, 0, right, g_bs, m, al, be, dst, g_bs, m, 0, stream, &sh,
+          return syrk_impl(left, batch, m, m, g_bs, m, 0, right, g_bs, m, al, 1.0f, dst, g_bs, m, 0, stream, &sh,
                            right == left ? nullptr : right, add2);
         };
-        // T' = R1 D + e1 D + s R1
-        if ((rc = product(SHIFT_PAIR_T, poly, gram, poly, 1.0f, 1.0f, tbuf)) != MI_OK) return rc;
-        // D2 = R1 T' + e1 T' + e1 s R1
-        if ((rc = product(SHIFT_PAIR_A2, poly, tbuf, poly, 1.0f, 1.0f, d2)) != MI_OK) return rc;
-        // R2 = c2 D2^2 + (b2 + 2 c2 s2) D2     (D is no longer needed: its buffer takes R2)
-        if ((rc = product(SHIFT_PAIR_POLY2, d2, d2, nullptr, c2, b2, gram)) != MI_OK) return rc;
-        // S = R2 R1 + e2 R1 + e1 R2            (T' is no longer needed)
-        if ((rc = product(SHIFT_PAIR_Q, gram, poly, gram, 1.0f, 1.0f, tbuf)) != MI_OK) return rc;
-        mult = tbuf;
-        apply_mode = SHIFT_PAIR_APPLY;
+        uint16_t* D = gram;
+        uint16_t* S = nullptr;  // S_{k-1}
+        for (int k = 0; k < taken; ++k) {
+          // R_k = c_k D_k^2 + (b_k + 2 c_k s_k) D_k
+          uint16_t* R = take();
+          if ((rc = product(SHIFT_GROUP_POLY, k, D, D, nullptr, abc[3 * (s + k) + 2], R)) != MI_OK) return rc;
+          if (k == 0) {
+            S = R;  // S_1 = R_1
+          } else {
+            // S_k = R_k S_{k-1} + e_k S_{k-1} + alpha_{k-1} R_k
+            uint16_t* Sk = take();
+            if ((rc = product(SHIFT_GROUP_Q, k, R, S, R, 1.0f, Sk)) != MI_OK) return rc;
+            give(S);
+            S = Sk;
+          }
+          if (k + 1 < taken) {
+            // T'_k = R_k D_k + e_k D_k + s_k R_k, then D_{k+1} = R_k T'_k + e_k T'_k + e_k s_k R_k over D_k
+            uint16_t* T = take();
+            if ((rc = product(SHIFT_GROUP_T, k, R, D, R, 1.0f, T)) != MI_OK) return rc;
+            if ((rc = product(SHIFT_GROUP_A, k, R, T, R, 1.0f, D)) != MI_OK) return rc;
+            give(T);
+          }
+          if (k > 0) give(R);  // (R_1 lives on as S_1)
+        }
+        mult = S;
+        alpha = 1.0f;
+        apply_mode = SHIFT_GROUP_APPLY;
       }
     }
     // X' = (a + b s + c s^2) X + B' X      (cubic: (a + b s) X + b A' X;  pair: e1 e2 X + S X)
     void* dst = last ? static_cast<void*>(result) : static_cast<void*>(xbuf[cur ^ 1]);
-    ShiftArgs sh_apply{apply_mode, b, c, nullptr, 0, shift, last ? nullptr : slots, a, a2, b2, c2};
+    ShiftArgs sh_apply{apply_mode, b, c, nullptr, 0, shift, last ? nullptr : slots};
+    sh_apply.group_abc = abc + 3 * s;
+    sh_apply.group_size = taken;
+    sh_apply.stage = taken - 1;
     sh_apply.xscale = xs;
     {
       ProfScope prof(PROF_APPLY, stream);
-      rc = gemm_axpy_impl(mult, g_bs, m, xbuf[cur], x_bs, ld, trans, dst, x_bs, ld, batch, m, n, alpha, pair ? 1.0f : a,
+      rc = gemm_axpy_impl(mult, g_bs, m, xbuf[cur], x_bs, ld, trans, dst, x_bs, ld, batch, m, n, alpha, taken > 1 ? 1.0f : a,
                           last ? 1 : 0, last ? out_scale : 1.0f, stream, &sh_apply, (last && !tall) ? out_accum : 0.0f);
     }
     if (rc != MI_OK) return rc;

@@ -221,19 +221,31 @@ def newton_schulz(
     return _mT(X) if transpose else X
 
 
-def pair_schedule(coeffs: Sequence[tuple[float, float, float]], pairs: bool) -> list[int]:
-    """Group sizes of the single-call GPU driver: 2 = two steps on one Gram matrix, 1 = an ordinary step.
+def group_schedule(coeffs: Sequence[tuple[float, float, float]], mode: int) -> list[int]:
+    """Group sizes of the single-call GPU driver: g = g steps on one Gram matrix, 1 = an ordinary step.
 
-    Pairs alternate with single steps, starting with a pair; a pair needs quintic coefficients (c != 0) in both
-    of its steps.  ``pairs=False`` gives all ones.
+    ``mode`` 0: all ones.  1: pairs alternate with single steps, starting with a pair (5 steps: 2 + 1 + 2); a pair needs quintic
+    coefficients (c != 0) in both of its steps.  2: as 1, but the first three steps form one group when at least
+    two more steps follow, all three are quintic and ``(a_1 a_2)**2 <= 400`` (the factor by which the rounding
+    noise of the first Gram matrix has grown in the third); 5 steps: 3 + 2.
     """
-    groups, s, want_pair = [], 0, True
+    groups, s, want_group = [], 0, True
+    quintic = lambda k: coeffs[k][2] != 0.0
     while s < len(coeffs):
-        pair = pairs and want_pair and s + 1 < len(coeffs) and coeffs[s][2] != 0.0 and coeffs[s + 1][2] != 0.0
-        groups.append(2 if pair else 1)
-        s += groups[-1]
-        want_pair = not pair
+        size = 1
+        if mode and want_group and s + 1 < len(coeffs) and quintic(s) and quintic(s + 1):
+            size = 2
+            if mode == 2 and s == 0 and len(coeffs) >= 5 and quintic(2) and (coeffs[0][0] * coeffs[1][0]) ** 2 <= 400.0:
+                size = 3
+        groups.append(size)
+        s += size
+        want_group = size != 2  # a pair is followed by a single step; the opening triple may be followed by a pair
     return groups
+
+
+def pair_schedule(coeffs: Sequence[tuple[float, float, float]], pairs: bool) -> list[int]:
+    """:func:`group_schedule` restricted to pairs (mode 1) or single steps (mode 0)."""
+    return group_schedule(coeffs, 1 if pairs else 0)
 
 
 def _mirror_lower(mat: np.ndarray) -> np.ndarray:
@@ -248,7 +260,7 @@ def newton_schulz_shifted_bf16(
     custom_coefficient_sets=None,
     eps: float = 1e-15,
     normalize_in_double: bool = False,
-    pairs: bool | None = None,
+    pairs: bool | int | None = None,
 ) -> np.ndarray:
     """CPU model of the rounding schedule of the single-call GPU driver (``mi_newton_schulz_bf16``).
 
@@ -262,12 +274,14 @@ def newton_schulz_shifted_bf16(
     scalar (one pass over the float32 input instead of two).
 
     For wide matrices (m >= 1024 and n >= 2 m, or the short, very wide per-head shapes whose Gram matrix is summed
-    from K slices; ``pairs`` overrides the rule) the driver takes steps two at a time
-    on one Gram matrix (see :func:`pair_schedule`).  All factors are polynomials of A and commute, so with
-    q1 = e1 I + R1 (R1 = B' of the first step, e1 = a1 + b1 s + c1 s^2):
-        A2 = q1^2 A = s2 I + D2,  T' = R1 A' + e1 A' + s R1,  D2 = R1 T' + e1 T' + e1 s R1,  s2 = e1^2 s,
-        R2 = c2 D2^2 + (b2 + 2 c2 s2) D2,  e2 = a2 + b2 s2 + c2 s2^2,
-        X'' = e1 e2 X + S X,  S = R2 R1 + e2 R1 + e1 R2,
+    from K slices; ``pairs`` = False / True / 2 overrides the rule with mode 0 / 1 / 2 of :func:`group_schedule`)
+    the driver takes steps two -- at the start, for the large shapes, three -- at a time
+    on one Gram matrix.  All factors are polynomials of A and commute, so with A_k = s_k I + D_k,
+    q_k = e_k I + R_k (R_k = B' of step k, e_k = a_k + b_k s_k + c_k s_k^2) and the accumulated multiplier
+    q_k ... q_1 = alpha_k I + S_k:
+        T'_k = R_k D_k + e_k D_k + s_k R_k,  D_{k+1} = R_k T'_k + e_k T'_k + e_k s_k R_k,  s_{k+1} = e_k^2 s_k,
+        S_k = R_k S_{k-1} + e_k S_{k-1} + alpha_{k-1} R_k  (S_1 = R_1),  alpha_k = e_1 ... e_k,
+        X' = alpha_g X + S_g X  after the g steps of the group,
     each m x m product computed on its lower triangle, mirrored and rounded to bf16.
     This function reproduces those rounding points so that GPU results can be compared tightly.
     """
@@ -298,29 +312,31 @@ def newton_schulz_shifted_bf16(
     if pairs is None:
         batch = int(np.prod(x.shape[:-2])) if x.ndim == 3 else 1
         split_k_gram = m % 128 == 0 and m <= 256 and n % 512 == 0 and n >= 1024 and batch * (n // 512) <= 65535
-        pairs = split_k_gram or (m >= 1024 and n >= 2 * m)
+        mode = 1 if split_k_gram else 2 if (m >= 1024 and n >= 2 * m) else 0
+    else:
+        mode = int(pairs)  # False / True / 2
     eye = np.eye(m, dtype=np.float32)
     done = 0
-    for group in pair_schedule(coeffs, pairs):
+    for group in group_schedule(coeffs, mode):
         a, b, c = (f(v) for v in coeffs[done])
         s = sumsq / f(m)
         gram = round_to_bf16((r * r) * np.matmul(X, _mT(X)) - s * eye)
-        if group == 2:
-            a2, b2, c2 = (f(v) for v in coeffs[done + 1])
-            r1 = round_to_bf16(c * np.matmul(gram, gram) + (b + f(2.0) * c * s) * gram)
-            e1 = a + b * s + c * s * s
-            t = round_to_bf16(_mirror_lower(np.matmul(r1, gram) + e1 * gram + s * r1))
-            d2 = round_to_bf16(_mirror_lower(np.matmul(r1, t) + e1 * t + (e1 * s) * r1))
-            s2 = e1 * e1 * s
-            r2 = round_to_bf16(c2 * np.matmul(d2, d2) + (b2 + f(2.0) * c2 * s2) * d2)
-            e2 = a2 + b2 * s2 + c2 * s2 * s2
-            q = round_to_bf16(_mirror_lower(np.matmul(r2, r1) + e2 * r1 + e1 * r2))
-            Xn = (e1 * e2 * r) * X + r * np.matmul(q, X)
-        elif c != 0.0:
-            poly = round_to_bf16(c * np.matmul(gram, gram) + (b + f(2.0) * c * s) * gram)
-            Xn = ((a + b * s + c * s * s) * r) * X + r * np.matmul(poly, X)
-        else:
+        if group == 1 and c == 0.0:
             Xn = ((a + b * s) * r) * X + (b * r) * np.matmul(gram, X)
+        else:
+            # A_k = s_k I + D_k;  accumulated multiplier alpha I + S
+            D, sk, alpha, S = gram, s, f(1.0), None
+            for k in range(group):
+                ak, bk, ck = (f(v) for v in coeffs[done + k])
+                R = round_to_bf16(ck * np.matmul(D, D) + (bk + f(2.0) * ck * sk) * D)
+                e = ak + bk * sk + ck * sk * sk
+                S = R if k == 0 else round_to_bf16(_mirror_lower(np.matmul(R, S) + e * S + alpha * R))
+                if k + 1 < group:
+                    T = round_to_bf16(_mirror_lower(np.matmul(R, D) + e * D + sk * R))
+                    D = round_to_bf16(_mirror_lower(np.matmul(R, T) + e * T + (e * sk) * R))
+                    sk = e * e * sk
+                alpha = alpha * e
+            Xn = (alpha * r) * X + r * np.matmul(S, X)
         done += group
         r = np.ones_like(norm)  # from here on X is normalised
         sumsq = np.sum(Xn * Xn, axis=(-2, -1), keepdims=True, dtype=np.float32)

@@ -97,12 +97,13 @@ def test_paired_steps_match_oracle(gpu, forced_pairs, shape, kind, steps):
         assert rel_fro(model, single) > 1e-5
 
 
-def test_pair_rule_by_shape(gpu, monkeypatch):
-    """Wide matrices pair up by default, MI_NS_PAIRS=0 switches that off; both stay within tolerance."""
+def test_group_rule_by_shape(gpu, monkeypatch):
+    """Wide matrices take 5 quintic steps as 3 + 2 by default, as 2 + 1 + 2 under MI_NS_PAIRS=pairs, one at a time
+    under MI_NS_PAIRS=0; every variant stays within tolerance and follows its rounding model."""
     x = torch.randn(1024, 2560)
     want32 = O.newton_schulz(x.numpy(), 5, "quintic")
     outs = {}
-    for env in (None, "0"):
+    for env, mode in ((None, 2), ("pairs", 1), ("0", 0)):
         if env is None:
             monkeypatch.delenv("MI_NS_PAIRS", raising=False)
         else:
@@ -110,9 +111,14 @@ def test_pair_rule_by_shape(gpu, monkeypatch):
         with utils.fp32_matmul_precision("medium"):
             outs[env] = muon_utils.newton_schulz(x.to(gpu), steps=5, coefficient_type="quintic", use_syrk=True).cpu()
         assert rel_fro(outs[env], want32) <= TOL_FP32
-    assert rel_fro(outs[None], O.newton_schulz_shifted_bf16(x.numpy(), 5, "quintic", pairs=True)) <= 6e-3
-    assert rel_fro(outs["0"], O.newton_schulz_shifted_bf16(x.numpy(), 5, "quintic", pairs=False)) <= 6e-3
-    assert not torch.equal(outs[None], outs["0"])
+        assert rel_fro(outs[env], O.newton_schulz_shifted_bf16(x.numpy(), 5, "quintic", pairs=mode)) <= 6e-3
+    assert rel_fro(outs[None], O.newton_schulz_shifted_bf16(x.numpy(), 5, "quintic")) <= 6e-3  # the model's own rule
+    assert not torch.equal(outs[None], outs["pairs"]) and not torch.equal(outs["pairs"], outs["0"])
+    # polar_express opens with a large coefficient: no three steps at once there
+    monkeypatch.delenv("MI_NS_PAIRS", raising=False)
+    with utils.fp32_matmul_precision("medium"):
+        got = muon_utils.newton_schulz(x.to(gpu), steps=5, coefficient_type="polar_express", use_syrk=True).cpu()
+    assert rel_fro(got, O.newton_schulz_shifted_bf16(x.numpy(), 5, "polar_express", pairs=1)) <= 6e-3
 
 
 @pytest.mark.parametrize("shape", [(256, 512), (2, 128, 1024), (1024, 2048), (512, 256), (2, 1000, 504), (2048, 1024)])
@@ -145,18 +151,20 @@ def _spectrum_cases():
 
 
 @pytest.mark.parametrize("kind", ["simple", "quintic", "polar_express"])
-def test_paired_steps_are_as_accurate_as_single_steps(gpu, monkeypatch, kind):
+def test_grouped_steps_are_as_accurate_as_single_steps(gpu, monkeypatch, kind):
     """Ill-conditioned inputs are far from float32 under any bf16 schedule (the reference's included); what must
-    hold is that taking steps in pairs does not add to that."""
+    hold is that taking steps in groups (the driver's own rule: 3 + 2 or 2 + 1 + 2; pairs only) does not add to
+    that."""
     for name, x in _spectrum_cases():
         want32 = O.newton_schulz(x.numpy(), 5, kind, compute_dtype=np.float64)
         err = {}
-        for env in ("1", "0"):
+        for env in ("auto", "pairs", "0"):
             monkeypatch.setenv("MI_NS_PAIRS", env)
             with utils.fp32_matmul_precision("medium"):
                 got = muon_utils.newton_schulz(x.to(gpu), steps=5, coefficient_type=kind, use_syrk=True).cpu()
             err[env] = rel_fro(got, want32)
-        assert err["1"] <= 1.15 * err["0"] + 5e-4, (name, kind, err)
+        assert err["auto"] <= 1.15 * err["0"] + 5e-4, (name, kind, err)
+        assert err["pairs"] <= 1.15 * err["0"] + 5e-4, (name, kind, err)
 
 
 def test_fused_known_answers(gpu):

@@ -221,14 +221,21 @@ def test_shifted_schedule_model_is_the_same_iteration():
     assert O.pair_schedule([(1, 1, 1)] * 5, True) == [2, 1, 2] and O.pair_schedule([(1, 1, 1)] * 8, True) == [2, 1, 2, 1, 2]
     assert O.pair_schedule([(1, 1, 1)] * 4, True) == [2, 1, 1] and O.pair_schedule([(1, 1, 0)] * 3, True) == [1, 1, 1]
     assert O.pair_schedule([(1, 1, 1)] * 5, False) == [1] * 5
+    simple, pe = [(3.4445, -4.7750, 2.0315)], O.expand_coefficients(8, "polar_express")
+    assert O.group_schedule(simple * 5, 2) == [3, 2] and O.group_schedule(simple * 8, 2) == [3, 2, 1, 2]
+    assert O.group_schedule(simple * 4, 2) == [2, 1, 1] and O.group_schedule(simple * 6, 2) == [3, 2, 1]
+    assert O.group_schedule(pe[:5], 2) == [2, 1, 2]  # (a_1 a_2)^2 = 1113: no three steps at once
+    assert O.group_schedule(O.expand_coefficients(5, "quintic"), 2) == [3, 2]
     wide = rng.standard_normal((64, 256)).astype(np.float32)
     for kind, steps in (("simple", 5), ("quintic", 5), ("polar_express", 8), ("cubic5", 5)):
         try:
             O.round_to_bf16 = lambda v: np.asarray(v, dtype=np.float32)
             exact = O.newton_schulz_shifted_bf16(wide, steps, kind, pairs=True)
+            exact3 = O.newton_schulz_shifted_bf16(wide, steps, kind, pairs=2)
         finally:
             O.round_to_bf16 = saved
         np.testing.assert_allclose(exact, O.newton_schulz(wide, steps, kind), atol=2e-5)
+        np.testing.assert_allclose(exact3, O.newton_schulz(wide, steps, kind), atol=3e-5)
         hi = O.newton_schulz(wide, steps, kind, compute_dtype=np.float64)
         e_pair = np.linalg.norm(O.newton_schulz_shifted_bf16(wide, steps, kind, pairs=True) - hi) / np.linalg.norm(hi)
         e_single = np.linalg.norm(O.newton_schulz_shifted_bf16(wide, steps, kind, pairs=False) - hi) / np.linalg.norm(hi)
