@@ -28,8 +28,10 @@ for _p in (ROOT, os.path.join(ROOT, "emerging-optimizers_amd")):
 PEAK_BF16_TFLOPS = 2516.6  # MI355X dense bf16 MFMA: 256 CU x 2.4 GHz x 4096 FLOP/clk/CU
 # HBM-side bytes of one GEMM+AXPY at the headline shape (both launches), from two `rocprofv3 --pmc` runs of this file
 # (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for sumsq_kernel
-# of the same run, whose traffic is known (229 376 KiB read, 114 696 KiB written): factors 1.9994 and 0.9998.
-GEMM_AXPY_TRAFFIC_BYTES = int(((408472.6 + 146827.5) * 1.9994 + (98328.1 + 16392.0) * 0.9998) * 1024)
+# of the same run, whose traffic is known (229 376 KiB read, 114 696 KiB written): factors 1.9993 and 0.9998.
+GEMM_AXPY_TRAFFIC_BYTES = int(((406432.7 + 146832.3) * 1.9993 + (98328.0 + 16392.0) * 0.9998) * 1024)
+# The same for the lower-triangle kernel, averaged over its 16 launches per call (2 x X X^T, 14 m x m products).
+TRI_KERNEL_TRAFFIC_BYTES = int((128714.6 * 1.9993 + 32768.0 * 0.9998) * 1024)
 M, N, NS_STEPS = 4096, 14336, 5
 # Other benchmark configurations, timed with --workload (the default, "mlp", is the headline).
 WORKLOADS = {
@@ -344,9 +346,15 @@ def main():
     names = ["normalize_cast", "syrk_gram", "syrk_poly", "gemm_axpy"]
     per_kernel = {n: (ms_kind[i] / n_kind[i] if n_kind[i] else None) for i, n in enumerate(names)}
     gemm_ms = per_kernel["gemm_axpy"]
-    gemm_flop = 2.0 * M * M * N  # algorithmic FLOP of one GEMM+AXPY launch
-    achieved = gemm_flop / (gemm_ms * 1e-3) / 1e12 if gemm_ms else None
-
+    gemm_flop = 2.0 * M * M * N  # algorithmic FLOP of one GEMM+AXPY launch pair
+    gemm_tflops = gemm_flop / (gemm_ms * 1e-3) / 1e12 if gemm_ms else None
+    # The kernel with the largest share of the GPU time is the lower-triangle kernel (one rocprof row: 192 x 192
+    # tiles), which serves X X^T (m^2 n FLOP sym-halved) and every m x m product (m^3 FLOP): its launches are
+    # priced together, algorithmic FLOP per launch over the average launch duration.
+    tri_launches = n_kind[1] + n_kind[2]
+    tri_ms = (ms_kind[1] + ms_kind[2]) / tri_launches if tri_launches else None
+    tri_flop = (n_kind[1] * float(M) * M * N + n_kind[2] * float(M) ** 3) / tri_launches if tri_launches else None
+    achieved = tri_flop / (tri_ms * 1e-3) / 1e12 if tri_ms else None
     line = {
         "metric": "NS orthogonalize ms + TFLOP/s (% bf16 MFMA peak) at 4096x14336 bf16",
         "value": round(tflops, 2),
@@ -372,15 +380,19 @@ def main():
             "rel_fro_vs_fp32": round(rel, 6),
             "tolerance": 1e-2,
             "kernel_ms": {k: (round(v, 4) if v is not None else None) for k, v in per_kernel.items()},
+            "gemm_axpy_tflops": round(gemm_tflops, 1) if gemm_tflops else None,
+            "gemm_axpy_traffic_bytes": GEMM_AXPY_TRAFFIC_BYTES if (M, N) == (4096, 14336) else None,
         },
         "roofline": {
-            "kernel": "gemm_fast_kernel (X' = a X + B X, 2 m^2 n FLOP; 768 tiles of 256x256 + 256 tiles of 256x128)",
+            "kernel": "gemm_fast_kernel<FastCfg<192,...>, SYRK mode> (lower-triangle kernel: X X^T and the m x m products; "
+            f"{n_kind[1] // args.steps} + {n_kind[2] // args.steps} launches per call, sym-halved FLOP, average launch)",
             "bound": "mfma",
             "achieved": round(achieved, 2) if achieved else None,
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_BF16_TFLOPS, 4) if achieved else None,
-            "traffic": GEMM_AXPY_TRAFFIC_BYTES if (M, N) == (4096, 14336) else None,
+            "traffic": TRI_KERNEL_TRAFFIC_BYTES if ((M, N) == (4096, 14336) and schedule == [3, 2]) else None,
+            "avg_launch_ms": round(tri_ms, 4) if tri_ms else None,
         },
     }
     if rel > 1e-2:

@@ -427,8 +427,9 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, typename 
 // with 16 bytes per lane along rows; then the transposed tile is assembled the same way (2-byte LDS writes) and
 // written to the mirrored position.  A diagonal tile is assembled once from its lower half (value and mirror
 // image), so the stored result is symmetric bit for bit.  Tiles too large for the ring go in passes of RP rows.
-// Cin (the beta term) is fetched with the same row-wise 16-byte accesses into LDS first and picked up from
-// there in accumulator layout.  Every wavefront of the workgroup must call this (it contains barriers).
+// The addends (the beta terms) of a one-pass tile are read straight in accumulator layout (8 bytes per quad,
+// whole 32-byte sectors per row); a tile staged in passes fetches Cin with row-wise 16-byte accesses into LDS
+// first and picks it up from there.  Every wavefront of the workgroup must call this (it contains barriers).
 // Geometry of the staged SYRK epilogue.
 template <class C>
 struct SyrkStage {
@@ -438,30 +439,39 @@ struct SyrkStage {
   static constexpr int NPASS = TILE / RP;
   static constexpr int CPRW = TILE / 8;            // 16-byte chunks per tile row
   static constexpr int NCH = RP * CPRW / C::NT;    // chunks per thread and pass
-  // a one-pass tile may fetch its Cin rows into registers before the K loop (NCH x 4 registers per lane)
-  static constexpr bool CIN_EARLY = NPASS == 1 && NCH * 4 <= 80;
+  // a one-pass tile fetches its Cin values into registers before the K loop, in accumulator layout
+  // (one 8-byte quad per accumulator quad: NQUAD x 2 registers per lane)
+  static constexpr int NQUAD = C::FM * C::FN * (C::MI == 32 ? 4 : 1);
+  static constexpr bool CIN_EARLY = NPASS == 1 && NQUAD * 2 <= 80;
 };
-// Row-wise 16-byte loads of this thread's Cin chunks of a one-pass tile (issued before the K loop so that the
-// burst of all workgroups does not sit on the critical path at the end of the kernel).
+// This lane's addend values of a one-pass tile, in accumulator layout: quad (i, j, g) covers row
+// m0 + mw + i MI + (lane % MI), columns n0 + nw + j MI + 8 g + 4 (lane / MI) .. + 3 (g only for MI = 32).  One load
+// instruction touches MI rows with 32 contiguous bytes each -- whole 32-byte sectors, so nothing is fetched twice.
+// Issued before the K loop (first addend) or at the start of the epilogue (second), so that the burst of all
+// workgroups does not sit on the critical path.
 template <class C, bool GUARD>
-__device__ __forceinline__ void syrk_cin_prefetch(const GemmParams& p, int m0, int n0, int64_t batch,
-                                                  uint4 (&pre)[SyrkStage<C>::NCH]) {
-  using S = SyrkStage<C>;
-  const uint16_t* __restrict__ Cb = p.Cin + batch * p.c_bs;
+__device__ __forceinline__ void syrk_addend_fetch(const GemmParams& p, const uint16_t* __restrict__ Cb, int lane, int m_base,
+                                                  int n_base, uint2 (&pre)[SyrkStage<C>::NQUAD]) {
+  constexpr int MI = C::MI, G = MI == 32 ? 4 : 1;
+  const int frow = lane & (MI - 1), fk = lane / MI;
 #pragma unroll
-  for (int it = 0; it < S::NCH; ++it) {
-    const int c = threadIdx.x + it * C::NT, row = c / S::CPRW, c8 = c % S::CPRW;
-    const int m = m0 + row, n = n0 + c8 * 8;
-    pre[it] = make_uint4(0u, 0u, 0u, 0u);
-    if (!GUARD || (m < p.M && n < p.N)) pre[it] = *reinterpret_cast<const uint4*>(Cb + (int64_t)m * p.ldc + n);
-  }
+  for (int i = 0; i < C::FM; ++i)
+#pragma unroll
+    for (int j = 0; j < C::FN; ++j)
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const int m = m_base + i * MI + frow, n = n_base + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
+        uint2 v = make_uint2(0u, 0u);
+        if (!GUARD || (m < p.M && n < p.N)) v = *reinterpret_cast<const uint2*>(Cb + (int64_t)m * p.ldc + n);
+        pre[(i * C::FN + j) * G + g] = v;
+      }
 }
 
 template <class C, bool GUARD>
 __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename AccVec<C::MI>::type (&acc)[C::FM][C::FN],
                                                   char* lds, int lane, int wm, int wn, int m0, int n0, int64_t batch,
                                                   bool diag, float alpha, float beta, float beta2, float shift,
-                                                  const uint4 (&cin_pre)[SyrkStage<C>::CIN_EARLY ? SyrkStage<C>::NCH : 1]) {
+                                                  const uint2 (&cin_pre)[SyrkStage<C>::CIN_EARLY ? SyrkStage<C>::NQUAD : 1]) {
   using S = SyrkStage<C>;
   constexpr int TILE = S::TILE, LDT = S::LDT, MI = C::MI, G = MI == 32 ? 4 : 1, FM = C::FM, FN = C::FN;
   constexpr int RP = S::RP, NPASS = S::NPASS, CPRW = S::CPRW, NCH = S::NCH;
@@ -482,66 +492,21 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
   uint2 val[FM][FN][G];  // finished bf16 quads of this lane
   // ---- values: alpha * acc (+ beta * Cin) (+ beta2 * Cin2) (- shift on the diagonal), rounded to bf16 ----
   if constexpr (NPASS == 1) {
-    constexpr int h = 0;
-    // the second addend is requested first, so that its latency hides behind the staging of the first
-    uint4 c2[NCH];
-    if (use_c2) {
-#pragma unroll
-      for (int it = 0; it < NCH; ++it) {
-        const int c = tid + it * C::NT, row = c / CPRW, c8 = c % CPRW;
-        const int m = m0 + row, n = n0 + c8 * 8;
-        c2[it] = make_uint4(0u, 0u, 0u, 0u);
-        if (!GUARD || (m < p.M && n < p.N)) c2[it] = *reinterpret_cast<const uint4*>(Cb2 + (int64_t)m * p.ldc + n);
-      }
+    // Both addends arrive in accumulator layout: the first was requested before the K loop, the second is
+    // requested now and consumed after the first.
+    constexpr int NQ = S::NQUAD;
+    uint2 c2[NQ];
+    if (use_c2) syrk_addend_fetch<C, GUARD>(p, Cb2, lane, m0 + mw, n0 + nw, c2);
+    uint2 c1[S::CIN_EARLY ? 1 : NQ];
+    if constexpr (!S::CIN_EARLY) {
+      if (use_c) syrk_addend_fetch<C, GUARD>(p, Cb, lane, m0 + mw, n0 + nw, c1);
     }
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-      for (int j = 0; j < FN; ++j)
-#pragma unroll
-        for (int e = 0; e < 4 * G; ++e) acc[i][j][e] = alpha * acc[i][j][e];
-    // adds coef * (the tile staged in LDS) to this wavefront's accumulators
-    auto add_staged = [&](float coef) {
-#pragma unroll
-      for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-          for (int g = 0; g < G; ++g) {
-            const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
-            const uint2 raw = *reinterpret_cast<const uint2*>(lds + (ml * LDT + nl) * 2);
-            acc[i][j][4 * g + 0] = __builtin_fmaf(coef, __uint_as_float(raw.x << 16), acc[i][j][4 * g + 0]);
-            acc[i][j][4 * g + 1] = __builtin_fmaf(coef, __uint_as_float(raw.x & 0xffff0000u), acc[i][j][4 * g + 1]);
-            acc[i][j][4 * g + 2] = __builtin_fmaf(coef, __uint_as_float(raw.y << 16), acc[i][j][4 * g + 2]);
-            acc[i][j][4 * g + 3] = __builtin_fmaf(coef, __uint_as_float(raw.y & 0xffff0000u), acc[i][j][4 * g + 3]);
-          }
+    auto add = [&](f32x4_t& v, const uint2& raw, float coef) {
+      v[0] = __builtin_fmaf(coef, __uint_as_float(raw.x << 16), v[0]);
+      v[1] = __builtin_fmaf(coef, __uint_as_float(raw.x & 0xffff0000u), v[1]);
+      v[2] = __builtin_fmaf(coef, __uint_as_float(raw.y << 16), v[2]);
+      v[3] = __builtin_fmaf(coef, __uint_as_float(raw.y & 0xffff0000u), v[3]);
     };
-    if (use_c) {
-      __syncthreads();  // the ring is no longer read
-#pragma unroll
-      for (int it = 0; it < NCH; ++it) {
-        const int c = tid + it * C::NT, row = c / CPRW, c8 = c % CPRW;
-        const int m = m0 + row, n = n0 + c8 * 8;
-        uint4 v = make_uint4(0u, 0u, 0u, 0u);
-        if constexpr (S::CIN_EARLY)
-          v = cin_pre[it];  // fetched before the K loop
-        else if (!GUARD || (m < p.M && n < p.N))
-          v = *reinterpret_cast<const uint4*>(Cb + (int64_t)m * p.ldc + n);
-        *reinterpret_cast<uint4*>(lds + (row * LDT + c8 * 8) * 2) = v;
-      }
-      __syncthreads();
-      add_staged(beta);
-    }
-    if (use_c2) {
-      __syncthreads();
-#pragma unroll
-      for (int it = 0; it < NCH; ++it) {
-        const int c = tid + it * C::NT, row = c / CPRW, c8 = c % CPRW;
-        *reinterpret_cast<uint4*>(lds + (row * LDT + c8 * 8) * 2) = c2[it];
-      }
-      __syncthreads();
-      add_staged(beta2);
-    }
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
@@ -549,7 +514,17 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
 #pragma unroll
         for (int g = 0; g < G; ++g) {
           const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
-          f32x4_t v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+          const int q = (i * FN + j) * G + g;
+          f32x4_t v;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][4 * g + r];
+          if (use_c) {
+            if constexpr (S::CIN_EARLY)
+              add(v, cin_pre[q], beta);
+            else
+              add(v, c1[q], beta);
+          }
+          if (use_c2) add(v, c2[q], beta2);
           if (p.shift_mode == SHIFT_GRAM && diag) {
 #pragma unroll
             for (int r = 0; r < 4; ++r)
@@ -557,7 +532,6 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
           }
           val[i][j][g] = __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));
         }
-    (void)h;
   } else {
     // a tile staged in passes: Cin goes through LDS pass by pass, Cin2 (rare here) is read in accumulator layout
 #pragma unroll
@@ -903,11 +877,12 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
 #endif
   constexpr bool SYRK_STAGED = MODE == MODE_SYRK && !OUT_F32 && C::KSPLIT == 1 && C::NW == 4;
   constexpr bool CIN_EARLY = SYRK_STAGED && SyrkStage<C>::CIN_EARLY;
-  uint4 cin_pre[CIN_EARLY ? SyrkStage<C>::NCH : 1];
+  uint2 cin_pre[CIN_EARLY ? SyrkStage<C>::NQUAD : 1];
   if constexpr (CIN_EARLY) {
     // these loads are older than every direct-to-LDS load issued from here on, so the vmcnt waits of the K
     // loop cover them as well
-    if (p.Cin != nullptr) syrk_cin_prefetch<C, EDGE>(p, m0, n0, batch, cin_pre);
+    if (p.Cin != nullptr)
+      syrk_addend_fetch<C, EDGE>(p, p.Cin + batch * p.c_bs, lane, m0 + wm * C::TM, n0 + wn * C::TN, cin_pre);
   }
   // A wavefront none of whose outputs is ever stored (its rows or columns lie beyond the matrix, or its block is
   // strictly above the diagonal of a diagonal SYRK tile) keeps loading its share of the operand tiles and keeps

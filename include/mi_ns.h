@@ -121,11 +121,12 @@ size_t mi_frob_partials_len(int64_t batch, int64_t numel);
  * Two things differ from a literal step-by-step execution, neither of which changes the function computed:
  *  - the input is cast to bf16 by the pass that sums its squares, and 1 / norm enters the first two products
  *    as a device scalar (norms outside [1e-10, 1e10] are divided out before the cast instead);
- *  - for matrices with at least 1024 rows and twice as many columns, and for 128/256-row matrices at least four
- *    times as wide, consecutive quintic steps are taken two at a time on one Gram matrix (all factors are
- *    polynomials of X X^T and commute): 5 steps run as 2 + 1 + 2.  The environment variable MI_NS_PAIRS, read at
- *    every call (and by mi_newton_schulz_workspace_bytes), overrides this: "0" = one step at a time, "force" = pairs
- *    at every size.
+ *  - for matrices with at least 1024 rows and twice as many columns, consecutive quintic steps share one Gram
+ *    matrix (all factors are polynomials of X X^T and commute): the first three when at least two more follow and
+ *    (a_1 a_2)^2 <= 400, otherwise two at a time alternating with single steps, so 5 steps run as 3 + 2 or
+ *    2 + 1 + 2; 128/256-row matrices at least four times as wide run as 2 + 1 + 2.  The environment variable
+ *    MI_NS_PAIRS, read at every call (and by mi_newton_schulz_workspace_bytes), overrides this: "0" = one step at a
+ *    time, "pairs" = never three at once, "force" = pairs at every size.
  */
 int mi_newton_schulz_bf16(const float* x, float* out, int64_t batch, int64_t rows, int64_t cols,
                           const float* abc, int steps, float eps, int accumulate_fp64,

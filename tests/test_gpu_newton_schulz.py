@@ -150,7 +150,7 @@ def _spectrum_cases():
     yield "gaussian", torch.randn(m, n, generator=g)
 
 
-@pytest.mark.parametrize("kind", ["simple", "quintic", "polar_express"])
+@pytest.mark.parametrize("kind", ["simple", "quintic", "aol", "polar_express"])
 def test_grouped_steps_are_as_accurate_as_single_steps(gpu, monkeypatch, kind):
     """Ill-conditioned inputs are far from float32 under any bf16 schedule (the reference's included); what must
     hold is that taking steps in groups (the driver's own rule: 3 + 2 or 2 + 1 + 2; pairs only) does not add to
