@@ -855,13 +855,13 @@ __global__ void __launch_bounds__(256) gram_reduce_kernel(const float* __restric
 
 // ---------------------------------------------------------------------------------------------
 // 128 x 128 matrices (one attention head each): everything between the split-K Gram partials and the B X product
-// of a step -- or of a pair of steps -- in one launch.  One workgroup per matrix keeps up to four 128 x 128 bf16
+// of a step -- or of a group of two or three steps -- in one launch.  One workgroup per matrix keeps up to four 128 x 128 bf16
 // matrices in LDS (32 KB each, 16-byte chunks XOR-swizzled by row so that the 32 rows one fragment read touches
 // fall into different banks) and forms
 //   D  = r^2 sum_s partial_s - s I                       (what gram_reduce_kernel stores)
 //   R1 = c1 D^2 + (b1 + 2 c1 s) D                        single step: the result
-//   T' = R1 D + e1 D + s R1,  D2 = R1 T' + e1 T' + e1 s R1,  R2 = c2 D2^2 + (b2 + 2 c2 s2) D2,
-//   S  = R2 R1 + e2 R1 + e1 R2                           pair: the result
+//   and for a group of two or three steps the chain R_k, S_k, T'_k, D_{k+1} of SHIFT_GROUP_* (gemm_engine.hpp),
+//   whose last S is the result
 // with the rounding points of the separate kernels: float32 accumulation, one rounding to bf16 per matrix, the lower
 // triangle computed and mirrored.
 // ---------------------------------------------------------------------------------------------
@@ -925,9 +925,9 @@ struct ChainArgs {
   int nslots_in;
   float* shift_io;        // [batch], written
   const float* xscale;    // [batch] or null
-  float a1, b1, c1, a2, b2, c2;
-  int pair;
-  uint16_t* out;          // [batch][128][128] bf16: R1 (single step) or S (pair)
+  float co[3][3];         // (a, b, c) of the steps of the group
+  int group;              // 1, 2 or 3 steps on this Gram matrix
+  uint16_t* out;          // [batch][128][128] bf16: the multiplier S_g of X (R_1 for a single step)
 };
 
 // 16 wavefronts per workgroup, one per 32 x 32 block of the products; together they stream the float32 partials in
@@ -988,19 +988,39 @@ __global__ void __launch_bounds__(CH_THREADS) small_chain_kernel(ChainArgs a) {
     }
   }
   __syncthreads();
-  const float e1 = a.a1 + a.b1 * s + a.c1 * s * s;
-  // R1 = c1 D^2 + (b1 + 2 c1 s) D -> B1
-  chain_product(B0, B0, B0, nullptr, B1, a.c1, a.b1 + 2.0f * a.c1 * s, 0.0f, wave, lane);
-  const char* result = B1;
-  if (a.pair) {
-    const float s2 = e1 * e1 * s;
-    const float e2 = a.a2 + a.b2 * s2 + a.c2 * s2 * s2;
-    chain_product(B1, B0, B0, B1, B2, 1.0f, e1, s, wave, lane);                               // T' -> B2
-    chain_product(B1, B2, B2, B1, B3, 1.0f, e1, e1 * s, wave, lane);                          // D2 -> B3
-    chain_product(B3, B3, B3, nullptr, B0, a.c2, a.b2 + 2.0f * a.c2 * s2, 0.0f, wave, lane);  // R2 -> B0
-    chain_product(B0, B1, B1, B0, B2, 1.0f, e2, e1, wave, lane);                              // S  -> B2
-    result = B2;
+  // The steps of the group (SHIFT_GROUP_* in gemm_engine.hpp spells out the recursion); D_k stays in B0, the other
+  // three matrices are handed out and returned as what they hold dies.
+  char* pool[3] = {B1, B2, B3};
+  int free_n = 3;
+  char* D = B0;
+  char* S = nullptr;
+  float sk = s, before = 1.0f;
+#pragma unroll
+  for (int k = 0; k < 3; ++k) {
+    if (k >= a.group) break;
+    const float ak = a.co[k][0], bk = a.co[k][1], ck = a.co[k][2];
+    const float e = ak + bk * sk + ck * sk * sk;
+    char* R = pool[--free_n];
+    chain_product(D, D, D, nullptr, R, ck, bk + 2.0f * ck * sk, 0.0f, wave, lane);  // R_k
+    if (k == 0) {
+      S = R;
+    } else {
+      char* Sk = pool[--free_n];
+      chain_product(R, S, S, R, Sk, 1.0f, e, before, wave, lane);                   // S_k
+      pool[free_n++] = S;
+      S = Sk;
+    }
+    if (k + 1 < a.group) {
+      char* T = pool[--free_n];
+      chain_product(R, D, D, R, T, 1.0f, e, sk, wave, lane);                        // T'_k
+      chain_product(R, T, T, R, D, 1.0f, e, e * sk, wave, lane);                    // D_{k+1} over D_k
+      pool[free_n++] = T;
+      sk = e * e * sk;
+    }
+    if (k > 0) pool[free_n++] = R;
+    before *= e;
   }
+  const char* result = S;
   uint16_t* __restrict__ ob = a.out + b * (int64_t)(CH_M * CH_M);
   for (int c = tid; c < CH_M * (CH_M / 8); c += CH_THREADS) {
     const int row = c / (CH_M / 8), ch = c % (CH_M / 8);
@@ -1043,8 +1063,8 @@ static int small_gram(const uint16_t* X, int64_t batch, int64_t m, int64_t n, in
 
 // Partials, then everything up to the multiplier of the B X product in one launch (128-row matrices only).
 static int small_chain(const uint16_t* X, int64_t batch, int64_t n, int splits, float* partials, const float* slots_in,
-                       int nslots_in, float* shift_io, const float* xscale, const float* abc1, const float* abc2,
-                       uint16_t* out, hipStream_t stream) {
+                       int nslots_in, float* shift_io, const float* xscale, const float* abc, int group, uint16_t* out,
+                       hipStream_t stream) {
   int rc = small_gram_partials(X, batch, CH_M, n, splits, partials, stream);
   if (rc != MI_OK) return rc;
   ChainArgs a{};
@@ -1054,9 +1074,9 @@ static int small_chain(const uint16_t* X, int64_t batch, int64_t n, int splits, 
   a.nslots_in = nslots_in;
   a.shift_io = shift_io;
   a.xscale = xscale;
-  a.a1 = abc1[0], a.b1 = abc1[1], a.c1 = abc1[2];
-  a.pair = abc2 != nullptr;
-  if (abc2) a.a2 = abc2[0], a.b2 = abc2[1], a.c2 = abc2[2];
+  for (int k = 0; k < group; ++k)
+    for (int e = 0; e < 3; ++e) a.co[k][e] = abc[3 * k + e];
+  a.group = group;
   a.out = out;
   hipLaunchKernelGGL(small_chain_kernel, dim3((unsigned)batch), dim3(CH_THREADS), 0, stream, a);
   hipError_t e = hipGetLastError();
@@ -1085,10 +1105,9 @@ static int ns_pairs_enabled(int64_t m, int64_t n, int gram_splits) {
   const char* env = getenv("MI_NS_PAIRS");
   if (env && env[0] == '0') return 0;
   if (env && env[0] == 'f') return 1;
-  // (the split-K Gram path serves short matrices at least four times as wide as tall: a pair there trades two
-  // passes over X for four tiny products at the same number of launches)
-  if (gram_splits > 0) return 1;
-  if (m >= 1024 && n >= 2 * m) return (env && env[0] == 'p') ? 1 : 2;
+  // (the split-K Gram path serves short matrices at least four times as wide as tall: a group there trades passes
+  // over X for tiny products at no more launches)
+  if (gram_splits > 0 || (m >= 1024 && n >= 2 * m)) return (env && env[0] == 'p') ? 1 : 2;
   return 0;
 }
 
@@ -1208,23 +1227,22 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
     float alpha = b;
     int apply_mode = SHIFT_APPLY;
 #ifdef MI_HAS_SMALL_CFGS
-    const bool chain = w.gram_splits > 0 && m == CH_M && c != 0.0f && taken <= 2;
+    const bool chain = w.gram_splits > 0 && m == CH_M && c != 0.0f;
 #else
     const bool chain = false;
 #endif
     if (chain) {
 #ifdef MI_HAS_SMALL_CFGS
       // 128-row matrices: Gram partials, then one launch per matrix for everything up to the multiplier of X
-      uint16_t* dst_mult = taken == 2 ? reinterpret_cast<uint16_t*>(ws + w.t) : poly;
       {
         ProfScope prof(PROF_GRAM, stream);
         rc = small_chain(xbuf[cur], batch, n, w.gram_splits, reinterpret_cast<float*>(ws + w.gpart), slots, nslots, shift, xs,
-                         abc + 3 * s, taken == 2 ? abc + 3 * s + 3 : nullptr, dst_mult, stream);
+                         abc + 3 * s, taken, poly, stream);
       }
       if (rc != MI_OK) return rc;
-      mult = dst_mult;
+      mult = poly;
       alpha = 1.0f;
-      if (taken == 2) apply_mode = SHIFT_GROUP_APPLY;
+      if (taken > 1) apply_mode = SHIFT_GROUP_APPLY;
 #endif
     } else {
       // A' = X X^T - s I  (s = ||X||_F^2 / m from the partial sums the previous kernel left)

@@ -124,7 +124,7 @@ size_t mi_frob_partials_len(int64_t batch, int64_t numel);
  *  - for matrices with at least 1024 rows and twice as many columns, consecutive quintic steps share one Gram
  *    matrix (all factors are polynomials of X X^T and commute): the first three when at least two more follow and
  *    (a_1 a_2)^2 <= 400, otherwise two at a time alternating with single steps, so 5 steps run as 3 + 2 or
- *    2 + 1 + 2; 128/256-row matrices at least four times as wide run as 2 + 1 + 2.  The environment variable
+ *    2 + 1 + 2; the same holds for 128/256-row matrices at least four times as wide.  The environment variable
  *    MI_NS_PAIRS, read at every call (and by mi_newton_schulz_workspace_bytes), overrides this: "0" = one step at a
  *    time, "pairs" = never three at once, "force" = pairs at every size.
  */

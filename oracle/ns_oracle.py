@@ -312,7 +312,7 @@ def newton_schulz_shifted_bf16(
     if pairs is None:
         batch = int(np.prod(x.shape[:-2])) if x.ndim == 3 else 1
         split_k_gram = m % 128 == 0 and m <= 256 and n % 512 == 0 and n >= 1024 and batch * (n // 512) <= 65535
-        mode = 1 if split_k_gram else 2 if (m >= 1024 and n >= 2 * m) else 0
+        mode = 2 if (split_k_gram or (m >= 1024 and n >= 2 * m)) else 0
     else:
         mode = int(pairs)  # False / True / 2
     eye = np.eye(m, dtype=np.float32)
