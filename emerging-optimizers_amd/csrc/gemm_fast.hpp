@@ -489,7 +489,10 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
   const uint16_t* __restrict__ Cb2 = p.Cin2 ? p.Cin2 + batch * p.c_bs : nullptr;
   const bool use_c2 = beta2 != 0.0f && Cb2 != nullptr;
 
-  uint2 val[FM][FN][G];  // finished bf16 quads of this lane
+  // Finished bf16 quads of this lane.  A one-pass tile keeps them in registers; a tile staged in passes (a 256 x 256
+  // tile: 128 quads on top of 256 accumulators) finishes its float32 values in the accumulators instead and converts
+  // on the way to LDS, twice (tile and mirror image).
+  uint2 val[NPASS == 1 ? FM : 1][NPASS == 1 ? FN : 1][NPASS == 1 ? G : 1];
   // ---- values: alpha * acc (+ beta * Cin) (+ beta2 * Cin2) (- shift on the diagonal), rounded to bf16 ----
   if constexpr (NPASS == 1) {
     // Both addends arrive in accumulator layout: the first was requested before the K loop, the second is
@@ -578,11 +581,20 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
                 for (int r = 0; r < 4; ++r)
                   if (nl + r == ml) v[r] -= shift;
               }
-              val[i][j][g] = __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));
+#pragma unroll
+              for (int r = 0; r < 4; ++r) acc[i][j][4 * g + r] = v[r];
             }
       }
     }
   }
+  auto quad = [&](int i, int j, int g) -> uint2 {
+    if constexpr (NPASS == 1) {
+      return val[i][j][g];
+    } else {
+      const f32x4_t v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+      return __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));
+    }
+  };
   auto elem = [&](const uint2& q, int r) -> uint16_t {
     return (uint16_t)(r == 0 ? (q.x & 0xffffu) : r == 1 ? (q.x >> 16) : r == 2 ? (q.y & 0xffffu) : (q.y >> 16));
   };
@@ -609,11 +621,12 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
         for (int g = 0; g < G; ++g) {
           const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
           if (!mirror_in_tile) {
-            if (mw / RP == h) *reinterpret_cast<uint2*>(lds + ((ml - h * RP) * LDT + nl) * 2) = val[i][j][g];
-          } else {
+            if (mw / RP == h) *reinterpret_cast<uint2*>(lds + ((ml - h * RP) * LDT + nl) * 2) = quad(i, j, g);
+          } else if (mw / RP == h || nw / RP == h) {
+            const uint2 q4 = quad(i, j, g);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              const uint16_t e = elem(val[i][j][g], r);
+              const uint16_t e = elem(q4, r);
               if (mw / RP == h && nl + r <= ml) *reinterpret_cast<uint16_t*>(lds + ((ml - h * RP) * LDT + nl + r) * 2) = e;
               if (nw / RP == h && nl + r < ml) *reinterpret_cast<uint16_t*>(lds + ((nl + r - h * RP) * LDT + ml) * 2) = e;
             }
@@ -635,9 +648,10 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
 #pragma unroll
             for (int g = 0; g < G; ++g) {
               const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
+              const uint2 q4 = quad(i, j, g);
 #pragma unroll
               for (int r = 0; r < 4; ++r)
-                *reinterpret_cast<uint16_t*>(lds + ((nl + r - h * RP) * LDT + ml) * 2) = elem(val[i][j][g], r);
+                *reinterpret_cast<uint16_t*>(lds + ((nl + r - h * RP) * LDT + ml) * 2) = elem(q4, r);
             }
       }
       __syncthreads();
