@@ -295,6 +295,21 @@ def test_llama_shapes_within_tolerance(gpu, shape):
     assert rel_fro(got_t.T, got) < 5e-3
 
 
+@pytest.mark.parametrize("shape", [(1024, 2048), (1024, 8192), (2048, 8192), (1536, 4096), (3072, 8192), (2, 2048, 4096),
+                                   (8192, 2048), (1000, 2104)])
+@pytest.mark.parametrize("kind,steps", [("simple", 5), ("quintic", 5), ("polar_express", 8), ("deepseekv4", 10)])
+def test_wide_shapes_grouped_by_default(gpu, shape, kind, steps):
+    """Shapes that take several steps per Gram matrix by the driver's own rule (tile edges, batches, tall inputs,
+    long schedules: 3+2, 2+1+2+1+2, 3+2+1+2+1+1), against float32 torch on the GPU."""
+    x = (torch.randn(*shape, generator=torch.Generator().manual_seed(sum(shape))) * 1e-2).to(gpu)
+    coeffs = O.expand_coefficients(steps, kind)
+    ref = ns_fp32_torch(x, coeffs)
+    with utils.fp32_matmul_precision("medium"):
+        got = muon_utils.newton_schulz(x, steps=steps, coefficient_type=kind, use_syrk=True)
+    errs = [rel_fro(got[i], ref[i]) for i in range(shape[0])] if len(shape) == 3 else [rel_fro(got, ref)]
+    assert max(errs) <= TOL_FP32, errs
+
+
 def test_quintic_default_at_headline_shape(gpu):
     x = llama_grad((4096, 14336), seed=7).to(gpu)
     coeffs = muon_utils._COEFFICIENT_SETS["quintic"]
