@@ -375,6 +375,7 @@ def main():
             "tflops_full_count": round(f_full / (ms_per_step * 1e-3) / 1e12, 2),
             "schedule": "+".join(map(str, schedule)) + " (steps of one group share one Gram matrix)",
             "tflops_executed": round(f_exec / (ms_per_step * 1e-3) / 1e12, 2),
+            "pct_of_bf16_mfma_peak_executed": round(100.0 * f_exec / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 2),
             "launches_per_call": {n: n_kind[i] // args.steps for i, n in enumerate(["normalize_cast", "syrk_gram", "syrk_poly", "gemm_axpy"])},
             "pct_of_bf16_mfma_peak": round(100.0 * tflops / PEAK_BF16_TFLOPS, 2),
             "rel_fro_vs_fp32": round(rel, 6),
