@@ -1420,6 +1420,23 @@ size_t mi_newton_schulz_workspace_bytes(int64_t batch, int64_t rows, int64_t col
   return ns_layout(batch, rows, cols).total;
 }
 
+int mi_newton_schulz_schedule(int64_t batch, int64_t rows, int64_t cols, const float* abc, int steps, int* groups,
+                              int max_groups) {
+  if (batch <= 0 || rows <= 0 || cols <= 0 || steps < 0 || (steps > 0 && !abc) || !groups || max_groups < 0)
+    return fail(MI_ERR_BAD_ARG, "mi_newton_schulz_schedule: bad argument");
+  const NsWorkspace w = ns_layout(batch, rows, cols);
+  int count = 0;
+  bool want_group = true;
+  for (int s = 0; s < steps;) {
+    const int taken = ns_group_size(w.pairs, abc, steps, s, want_group);
+    want_group = taken != 2;
+    if (count < max_groups) groups[count] = taken;
+    ++count;
+    s += taken;
+  }
+  return count;
+}
+
 int mi_newton_schulz_bf16(const float* x, float* out, int64_t batch, int64_t rows, int64_t cols, const float* abc,
                           int steps, float eps, int accumulate_fp64, float out_scale, void* workspace,
                           size_t workspace_bytes, void* stream) {

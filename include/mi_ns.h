@@ -134,6 +134,15 @@ int mi_newton_schulz_bf16(const float* x, float* out, int64_t batch, int64_t row
 size_t mi_newton_schulz_workspace_bytes(int64_t batch, int64_t rows, int64_t cols);
 
 /*
+ * How mi_newton_schulz_bf16 would group the steps of a call with these arguments (pure host code, no GPU needed):
+ * writes the group sizes (1 = an ordinary step, 2 or 3 = that many steps on one Gram matrix) to groups[0..] and
+ * returns their number (which may exceed max_groups; only max_groups entries are written), or a negative error
+ * code.  No counterpart in the reference, whose loop (muon_utils.py:264-272) always takes one step at a time.
+ */
+int mi_newton_schulz_schedule(int64_t batch, int64_t rows, int64_t cols, const float* abc, int steps, int* groups,
+                              int max_groups);
+
+/*
  * One fused Muon update of a float32 parameter batch: momentum, Nesterov direction, Newton-Schulz
  * orthogonalisation and the weight update, without materialising the direction or the update in HBM:
  *   momentum <- momentum + (1 - beta) (grad - momentum)                 buf.lerp_(grad, 1 - beta)

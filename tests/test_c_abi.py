@@ -97,3 +97,32 @@ def test_python_validation_messages_cpu():
     with pytest.raises(RuntimeError, match="GPU only"):
         triton_kernels.tsyrk_ex(torch.randn(8, 8).to(bf))
     assert triton_kernels.can_use_batched_tsyrk(torch.randn(2, 16, 16).to(bf)) is False  # not on the GPU
+
+
+@pytest.mark.parametrize("env", [None, "0", "pairs", "force"])
+def test_step_grouping_rule_matches_the_oracle_model(monkeypatch, env):
+    """The host-side rule of the driver (which steps share a Gram matrix) against the oracle's restatement of it,
+    over shapes on both sides of every threshold and every coefficient family."""
+    from oracle import ns_oracle as O
+
+    if env is None:
+        monkeypatch.delenv("MI_NS_PAIRS", raising=False)
+    else:
+        monkeypatch.setenv("MI_NS_PAIRS", env)
+    lib = _hip.lib()
+    shapes = [(1, 4096, 14336), (1, 14336, 4096), (8, 4096, 14336), (1, 4096, 4096), (1, 4096, 8184), (1, 4096, 8192),
+              (1, 1024, 2048), (1, 1016, 4096), (32, 128, 4096), (2, 256, 1536), (4, 128, 1000), (1, 384, 4096), (1, 8, 16)]
+    cases = [("simple", 5), ("quintic", 5), ("quintic", 4), ("quintic", 3), ("polar_express", 8), ("cans", 5), ("aol", 5),
+             ("deepseekv4", 10), ("cubic5", 5), ("simple", 1), ("simple", 2)]
+    for batch, rows, cols in shapes:
+        m, n = min(rows, cols), max(rows, cols)
+        split_k = m % 128 == 0 and m <= 256 and n % 512 == 0 and n >= 1024 and batch * (n // 512) <= 65535
+        rule = 2 if (split_k or (m >= 1024 and n >= 2 * m)) else 0
+        mode = {None: rule, "0": 0, "pairs": min(rule, 1), "force": 1}[env]
+        for kind, steps in cases:
+            coeffs = O.expand_coefficients(steps, kind)
+            abc = (ctypes.c_float * (3 * steps))(*[v for c in coeffs for v in c])
+            out = (ctypes.c_int * 16)()
+            count = lib.mi_newton_schulz_schedule(batch, rows, cols, abc, steps, out, 16)
+            assert list(out[:count]) == O.group_schedule(coeffs, mode), (env, batch, rows, cols, kind, steps)
+    assert lib.mi_newton_schulz_schedule(1, 64, 64, None, 5, (ctypes.c_int * 4)(), 4) == _hip.MI_ERR_BAD_ARG
