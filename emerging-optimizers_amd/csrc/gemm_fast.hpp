@@ -281,7 +281,6 @@ __device__ __forceinline__ bf16x8_t fast_frag16_ks(uint32_t tile_lds, uint32_t S
   const uint32_t a1 = (((S + (uint32_t)(2 * r + 8) * 16u) & (ROWB - 1)) | R) + tile_lds + (uint32_t)(32 * q + 4) * ROWB;
   const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(uintptr_t)a0);
   const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(uintptr_t)a1);
-  typedef short s16x8_t __attribute__((ext_vector_type(8)));
   return __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 }
 
@@ -473,7 +472,7 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
                                                   bool diag, float alpha, float beta, float beta2, float shift,
                                                   const uint2 (&cin_pre)[SyrkStage<C>::CIN_EARLY ? SyrkStage<C>::NQUAD : 1]) {
   using S = SyrkStage<C>;
-  constexpr int TILE = S::TILE, LDT = S::LDT, MI = C::MI, G = MI == 32 ? 4 : 1, FM = C::FM, FN = C::FN;
+  constexpr int LDT = S::LDT, MI = C::MI, G = MI == 32 ? 4 : 1, FM = C::FM, FN = C::FN;
   constexpr int RP = S::RP, NPASS = S::NPASS, CPRW = S::CPRW, NCH = S::NCH;
   static_assert(RP * LDT * 2 <= S::RING, "staging pass exceeds the ring");
   static_assert(RP % C::TM == 0 && RP % C::TN == 0, "a wavefront's block must fall into one pass");
