@@ -93,7 +93,12 @@ using CfgSyrk192 = FastCfg<192, 2, 2, 64, 3, MI_SYRK192_KSPLIT>;
 // Batched small matrices (per-head shapes, 128 rows): GEMM+AXPY tile 128 x 256 (wavefronts of 128 x 64) and a
 // 128 x 128 tile (wavefronts of 64 x 64) for the split-K Gram partials.
 using CfgM128 = FastCfg<128, 1, 4, 64, 2, 1, 256, 16>;
-using CfgT128 = FastCfg<128, 2, 2, 64, 3, 1, 128, 16>;
+#ifndef MI_T128_NS
+#define MI_T128_NS 3
+#endif
+using CfgT128 = FastCfg<128, 2, 2, 64, MI_T128_NS, 1, 128, 16>;
+// The same tile with a two-slot ring (64 KB): two workgroups share a CU, so one's epilogue overlaps the other's K loop.
+using CfgT128x2 = FastCfg<128, 2, 2, 64, 2, 1, 128, 16>;
 using CfgBig = FastCfg<256, 2, 2, 64, 2, 1, 256, 16>;     // wavefronts of 128 x 128
 #ifndef MI_HALFN_NS
 #define MI_HALFN_NS 3
@@ -423,12 +428,15 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, typename 
 // SYRK-mode epilogue through LDS.  The accumulator layout gives a lane one output row and 4-column groups, i.e.
 // 8-byte pieces of 16 different rows per store instruction, and the mirrored tile would go out as single bf16
 // values.  Here the finished bf16 tile is assembled in LDS (row-major, rows padded by 16 bytes) and written
-// with 16 bytes per lane along rows; then the transposed tile is assembled the same way (2-byte LDS writes) and
-// written to the mirrored position.  A diagonal tile is assembled once from its lower half (value and mirror
-// image), so the stored result is symmetric bit for bit.  Tiles too large for the ring go in passes of RP rows.
-// The addends (the beta terms) of a one-pass tile are read straight in accumulator layout (8 bytes per quad,
-// whole 32-byte sectors per row); a tile staged in passes fetches Cin with row-wise 16-byte accesses into LDS
-// first and picks it up from there.  Every wavefront of the workgroup must call this (it contains barriers).
+// with 16 bytes per lane along rows; the mirror image is formed from the same staged rows with the LDS transpose
+// read (4 x 4 blocks of bf16 transposed in flight) and also leaves with 16 bytes per lane along (mirrored) rows.
+// A diagonal tile is made symmetric in LDS first: the wavefronts on the diagonal stage the lower half of their
+// block and fill its upper half with transposed 4 x 4 blocks; the block below the diagonal is written like any
+// other and mirrored into the tile's upper right.  The stored result is therefore symmetric bit for bit.
+// Tiles too large for the ring go in passes of RP rows.
+// The addends (the beta terms) are read straight in accumulator layout (8 bytes per quad, whole 32-byte sectors
+// per row); a one-pass tile requests the first one before the K loop.
+// Every wavefront of the workgroup must call this (it contains barriers).
 // Geometry of the staged SYRK epilogue.
 template <class C>
 struct SyrkStage {
@@ -489,8 +497,7 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
   const bool use_c2 = beta2 != 0.0f && Cb2 != nullptr;
 
   // Finished bf16 quads of this lane.  A one-pass tile keeps them in registers; a tile staged in passes (a 256 x 256
-  // tile: 128 quads on top of 256 accumulators) finishes its float32 values in the accumulators instead and converts
-  // on the way to LDS, twice (tile and mirror image).
+  // tile: 128 quads on top of 256 accumulators) finishes each quad on its way to LDS.
   uint2 val[NPASS == 1 ? FM : 1][NPASS == 1 ? FN : 1][NPASS == 1 ? G : 1];
   // ---- values: alpha * acc (+ beta * Cin) (+ beta2 * Cin2) (- shift on the diagonal), rounded to bf16 ----
   if constexpr (NPASS == 1) {
@@ -534,127 +541,142 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
           }
           val[i][j][g] = __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));
         }
-  } else {
-    // a tile staged in passes: Cin goes through LDS pass by pass, Cin2 (rare here) is read in accumulator layout
-#pragma unroll
-    for (int h = 0; h < NPASS; ++h) {
-      if (use_c) {
-        __syncthreads();  // the ring (or the previous pass) is no longer read
-#pragma unroll
-        for (int it = 0; it < NCH; ++it) {
-          const int c = tid + it * C::NT, row = c / CPRW, c8 = c % CPRW;
-          const int m = m0 + h * RP + row, n = n0 + c8 * 8;
-          uint4 v = make_uint4(0u, 0u, 0u, 0u);
-          if (!GUARD || (m < p.M && n < p.N)) v = *reinterpret_cast<const uint4*>(Cb + (int64_t)m * p.ldc + n);
-          *reinterpret_cast<uint4*>(lds + (row * LDT + c8 * 8) * 2) = v;
-        }
-        __syncthreads();
-      }
-      if (mw / RP == h) {
-#pragma unroll
-        for (int i = 0; i < FM; ++i)
-#pragma unroll
-          for (int j = 0; j < FN; ++j)
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-              const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
-              f32x4_t v;
-#pragma unroll
-              for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][4 * g + r];
-              if (use_c) {
-                const uint2 raw = *reinterpret_cast<const uint2*>(lds + ((ml - h * RP) * LDT + nl) * 2);
-                v[0] = __builtin_fmaf(beta, __uint_as_float(raw.x << 16), v[0]);
-                v[1] = __builtin_fmaf(beta, __uint_as_float(raw.x & 0xffff0000u), v[1]);
-                v[2] = __builtin_fmaf(beta, __uint_as_float(raw.y << 16), v[2]);
-                v[3] = __builtin_fmaf(beta, __uint_as_float(raw.y & 0xffff0000u), v[3]);
-              }
-              if (use_c2 && (!GUARD || (m0 + ml < p.M && n0 + nl < p.N))) {
-                const uint2 raw = *reinterpret_cast<const uint2*>(Cb2 + (int64_t)(m0 + ml) * p.ldc + n0 + nl);
-                v[0] = __builtin_fmaf(beta2, __uint_as_float(raw.x << 16), v[0]);
-                v[1] = __builtin_fmaf(beta2, __uint_as_float(raw.x & 0xffff0000u), v[1]);
-                v[2] = __builtin_fmaf(beta2, __uint_as_float(raw.y << 16), v[2]);
-                v[3] = __builtin_fmaf(beta2, __uint_as_float(raw.y & 0xffff0000u), v[3]);
-              }
-              if (p.shift_mode == SHIFT_GRAM && diag) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                  if (nl + r == ml) v[r] -= shift;
-              }
-#pragma unroll
-              for (int r = 0; r < 4; ++r) acc[i][j][4 * g + r] = v[r];
-            }
-      }
-    }
   }
+  // finished bf16 quad (i, j, g) of this lane; a tile staged in passes reads its addends here, in accumulator layout
+  // (fetching them a fragment row ahead into registers was tried: it spills and is slower)
   auto quad = [&](int i, int j, int g) -> uint2 {
     if constexpr (NPASS == 1) {
       return val[i][j][g];
     } else {
-      const f32x4_t v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+      const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
+      auto add = [&](f32x4_t& v, const uint2& raw, float coef) {
+        v[0] = __builtin_fmaf(coef, __uint_as_float(raw.x << 16), v[0]);
+        v[1] = __builtin_fmaf(coef, __uint_as_float(raw.x & 0xffff0000u), v[1]);
+        v[2] = __builtin_fmaf(coef, __uint_as_float(raw.y << 16), v[2]);
+        v[3] = __builtin_fmaf(coef, __uint_as_float(raw.y & 0xffff0000u), v[3]);
+      };
+      f32x4_t v;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][4 * g + r];
+      if (!GUARD || (m0 + ml < p.M && n0 + nl < p.N)) {
+        if (use_c) add(v, *reinterpret_cast<const uint2*>(Cb + (int64_t)(m0 + ml) * p.ldc + n0 + nl), beta);
+        if (use_c2) add(v, *reinterpret_cast<const uint2*>(Cb2 + (int64_t)(m0 + ml) * p.ldc + n0 + nl), beta2);
+      }
+      if (p.shift_mode == SHIFT_GRAM && diag) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (nl + r == ml) v[r] -= shift;
+      }
       return __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));
     }
   };
   auto elem = [&](const uint2& q, int r) -> uint16_t {
     return (uint16_t)(r == 0 ? (q.x & 0xffffu) : r == 1 ? (q.x >> 16) : r == 2 ? (q.y & 0xffffu) : (q.y >> 16));
   };
-  // row-wise write-out of one assembled pass: LDS rows [0, RP) -> global rows grow0 + row, columns gcol0 ..
-  auto write_out = [&](int grow0, int gcol0, int row_limit, int col_limit) {
+  typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)lds;  // LDS byte address
+  auto tr_read = [&](uint32_t byte_off) -> uint2 {
+    return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(uintptr_t)(lds_base + byte_off)));
+  };
+  const bool sym = diag && !p.skip_upper;  // diagonal tile: the lower half and its mirror image make the tile
+  const int wave = tid >> 6, l16 = lane & 15;
+  // Transposed write-out of staged rows [r_lo, r_lo + ROWS) x columns [0, CCOLS): a unit is 4 columns x 32 rows;
+  // each 16-lane group transposes one unit with two LDS transpose reads (source lane L fetches the 4 columns at
+  // row 8 (L % 4) + L / 4, then 4 rows further down) and ends up with 16 bytes of a mirrored row per lane.
+  auto mirror_out = [&](auto rows_c, auto ccols_c, int r_lo, int grow0, int gcol0) {
+    constexpr int ROWS = decltype(rows_c)::value, CCOLS = decltype(ccols_c)::value;
+    static_assert(ROWS % 32 == 0 && CCOLS % 4 == 0, "units of 4 columns x 32 rows");
+    constexpr int NB = ROWS / 32, UNITS = CCOLS / 4 * NB, ITER = (UNITS + 15) / 16;
 #pragma unroll
-    for (int it = 0; it < NCH; ++it) {
-      const int c = tid + it * C::NT, row = c / CPRW, c8 = c % CPRW;
-      const int gr = grow0 + row, gc = gcol0 + c8 * 8;
-      const uint4 v = *reinterpret_cast<const uint4*>(lds + (row * LDT + c8 * 8) * 2);
-      if (!GUARD || (gr < row_limit && gc < col_limit)) *reinterpret_cast<uint4*>(ob + (int64_t)gr * p.ldo + gc) = v;
+    for (int it = 0; it < ITER; ++it) {
+      const int unit = it * 16 + wave * 4 + (lane >> 4);
+      const bool on = UNITS % 16 == 0 || unit < UNITS;
+      const int u = UNITS % 16 == 0 ? unit : min(unit, UNITS - 1);
+      const int cq = u / NB, rb = u % NB;
+      const uint32_t a0 = (uint32_t)(((r_lo + 32 * rb + 8 * (l16 & 3) + (l16 >> 2)) * LDT + 4 * cq) * 2);
+      const uint2 t0 = tr_read(a0), t1 = tr_read(a0 + 4 * LDT * 2);
+      const int gr = grow0 + 4 * cq + (l16 & 3), gc = gcol0 + 32 * rb + 8 * (l16 >> 2);
+      if (on && (!GUARD || (gr < p.N && gc < p.M)))
+        *reinterpret_cast<uint4*>(ob + (int64_t)gr * p.ldo + gc) = make_uint4(t0.x, t0.y, t1.x, t1.y);
     }
   };
-  const bool mirror_in_tile = diag && !p.skip_upper;  // diagonal tile: lower half + its mirror image make the tile
-  // ---- the tile itself ----
-#pragma unroll
   for (int h = 0; h < NPASS; ++h) {
     __syncthreads();  // previous readers of the staging area are done
+    // ---- this pass's rows, row-major ----
+    if (mw / RP == h) {
+      if (!sym || wm > wn) {
 #pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-      for (int j = 0; j < FN; ++j)
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-          const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
-          if (!mirror_in_tile) {
-            if (mw / RP == h) *reinterpret_cast<uint2*>(lds + ((ml - h * RP) * LDT + nl) * 2) = quad(i, j, g);
-          } else if (mw / RP == h || nw / RP == h) {
-            const uint2 q4 = quad(i, j, g);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const uint16_t e = elem(q4, r);
-              if (mw / RP == h && nl + r <= ml) *reinterpret_cast<uint16_t*>(lds + ((ml - h * RP) * LDT + nl + r) * 2) = e;
-              if (nw / RP == h && nl + r < ml) *reinterpret_cast<uint16_t*>(lds + ((nl + r - h * RP) * LDT + ml) * 2) = e;
-            }
-          }
-        }
-    __syncthreads();
-    write_out(m0 + h * RP, n0, p.M, p.N);
-  }
-  // ---- the mirrored tile ----
-  if (!diag && !p.skip_upper) {
-#pragma unroll
-    for (int h = 0; h < NPASS; ++h) {
-      __syncthreads();
-      if (nw / RP == h) {
-#pragma unroll
-        for (int i = 0; i < FM; ++i)
+        for (int i = 0; i < FM; ++i) {
 #pragma unroll
           for (int j = 0; j < FN; ++j)
 #pragma unroll
             for (int g = 0; g < G; ++g) {
               const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
-              const uint2 q4 = quad(i, j, g);
-#pragma unroll
-              for (int r = 0; r < 4; ++r)
-                *reinterpret_cast<uint16_t*>(lds + ((nl + r - h * RP) * LDT + ml) * 2) = elem(q4, r);
+              *reinterpret_cast<uint2*>(lds + ((ml - h * RP) * LDT + nl) * 2) = quad(i, j, g);
             }
+        }
+      } else if (wm == wn) {
+        // block on the diagonal: quads below the diagonal's 4 x 4 blocks go in whole, a quad inside such a block
+        // puts its lower elements at both positions; the rest of the upper half is filled in below
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+#pragma unroll
+          for (int j = 0; j <= i; ++j)
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+              const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
+              if (j < i || nl < (ml & ~3)) {
+                *reinterpret_cast<uint2*>(lds + ((ml - h * RP) * LDT + nl) * 2) = quad(i, j, g);
+              } else if (nl == (ml & ~3)) {
+                const uint2 q4 = quad(i, j, g);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                  const uint16_t e = elem(q4, r);
+                  if (nl + r <= ml) *reinterpret_cast<uint16_t*>(lds + ((ml - h * RP) * LDT + nl + r) * 2) = e;
+                  if (nl + r < ml) *reinterpret_cast<uint16_t*>(lds + ((nl + r - h * RP) * LDT + ml) * 2) = e;
+                }
+              }
+            }
+        }
       }
+    }
+    if (sym) {
       __syncthreads();
-      write_out(n0 + h * RP, m0, p.N, p.M);
+      if (wm == wn && mw / RP == h) {
+        // upper 4 x 4 blocks of the diagonal block <- transposed lower ones (16 blocks per transpose read)
+        constexpr int NB4 = C::TM / 4;
+        static_assert(NB4 * NB4 % 16 == 0, "blocks must fill whole transpose reads");
+        const int rowbase = mw - h * RP, colbase = nw;
+        for (int it = 0; it < NB4 * NB4 / 16; ++it) {
+          const int ids = it * 16 + 4 * (lane >> 4) + (lane & 3);  // block this lane fetches a row of
+          const uint2 t =
+              tr_read((uint32_t)(((rowbase + 4 * (ids / NB4) + (l16 >> 2)) * LDT + colbase + 4 * (ids % NB4)) * 2));
+          const int idr = it * 16 + (lane >> 2), br = idr / NB4, bc = idr % NB4;  // block this lane receives a column of
+          if (br > bc) *reinterpret_cast<uint2*>(lds + ((rowbase + 4 * bc + (lane & 3)) * LDT + colbase + 4 * br) * 2) = t;
+        }
+      }
+    }
+    __syncthreads();
+    // ---- row-wise write-out: LDS rows [0, RP) -> global rows m0 + h RP + row ----
+#pragma unroll
+    for (int it = 0; it < NCH; ++it) {
+      const int c = tid + it * C::NT, row = c / CPRW, c8 = c % CPRW;
+      const int gr = m0 + h * RP + row, gc = n0 + c8 * 8;
+      const uint4 v = *reinterpret_cast<const uint4*>(lds + (row * LDT + c8 * 8) * 2);
+      // a diagonal tile holds nothing right of the diagonal block of a row: that part comes from the mirror image
+      const bool held = !sym || c8 * 8 < ((h * RP + row) / C::TM + 1) * C::TM;
+      if (held && (!GUARD || (gr < p.M && gc < p.N))) *reinterpret_cast<uint4*>(ob + (int64_t)gr * p.ldo + gc) = v;
+    }
+    // ---- the mirror image, straight from the staged rows ----
+    if (!p.skip_upper) {
+      if (!diag) {
+        mirror_out(std::integral_constant<int, RP>{}, std::integral_constant<int, C::TILE_M>{}, 0, n0, m0 + h * RP);
+      } else if ((h + 1) * RP > C::TM) {
+        // blocks below the diagonal blocks (rows from TM on, columns before TM) go to the upper right of the tile
+        constexpr int LO = NPASS == 1 ? C::TM : 0;  // first such row of the staged pass
+        static_assert(NPASS == 1 || RP == C::TM, "a pass is the tile or one block row");
+        mirror_out(std::integral_constant<int, C::TM>{}, std::integral_constant<int, C::TM>{}, LO, n0, m0 + h * RP + LO);
+      }
     }
   }
 }

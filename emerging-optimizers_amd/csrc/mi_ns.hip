@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -140,30 +141,52 @@ static int num_cus() {
 }
 
 // Tile choice of the fast path by modelled time: rounds of workgroups over the CUs times the cost of one tile.
-// Measured on this part (SYRK n = 1024 .. 4096, batch 1 .. 16, K 1024 .. 14336; GEMM m = 1024 .. 4096):
-//  * SYRK: 192 x 192 tiles (253 lower-triangle workgroups at 4096 rows = one round on 256 CUs) were never slower than
-//    256 x 256 tiles, batched or not; 128 x 128 tiles cost about 1.4x per FLOP but win whenever 192-tiles cannot fill the
-//    chip or waste most of a round (2048 rows: 66 vs 136 workgroups; 2 x 3072 rows: 272 vs 600).
+// Measured on this part (SYRK n = 1024 .. 8192, batch 1 .. 16, K 1024 .. 14336; GEMM m = 1024 .. 4096).
 //  * GEMM: 256 x 128 tiles cost about 1.27x per FLOP of 256 x 256 tiles and win when the latter leave CUs idle
 //    (1024 x 4096: 64 tiles).
-enum SyrkTile { SYRK_TILE_128, SYRK_TILE_192 };
-static SyrkTile pick_syrk_tile(int64_t n, int64_t batch) {
-#if defined(MI_HAS_SMALL_CFGS) && defined(MI_FORCE_SYRK128)
-  if (MI_FORCE_SYRK128) return SYRK_TILE_128;  // tuning builds only
+// Tile of the lower-triangle kernel.  Modelled time of a launch = rounds x (start-up + epilogue + k-tiles x time per
+// 64-deep k-tile), in microseconds, fitted to measurements on this part (256 CUs, all busy):
+//   192 x 192 (one workgroup per CU)             12.6 + 0.80 kt
+//   256 x 256 (one per CU, two-pass epilogue)    29.7 + 1.30 kt   needs n % 256 == 0
+//   128 x 128, two-slot ring (two per CU)         9.2 + s kt per pair of tiles, s = 0.74 (kt <= 32) .. 0.85 (kt >= 128:
+//                                                 long runs of MFMA work from two workgroups lower the clock),
+//                                                 needs n % 128 == 0
+//   128 x 128, three-slot ring (one per CU)       9.0 + 0.44 kt (0.31 kt when the tiles do not fill the CUs: the
+//                                                 clock rises), needs n % 128 == 0
+// Short K or few tiles favour the small tiles (their epilogue is short and, two to a CU, hidden), long K the
+// 192 x 192 tile, and row counts that 192 divides badly (1792 = 7 x 256) the 256 x 256 tile.
+enum SyrkTile { SYRK_TILE_128, SYRK_TILE_128X2, SYRK_TILE_192, SYRK_TILE_256 };
+static SyrkTile pick_syrk_tile(int64_t n, int64_t batch, int64_t k) {
+#if defined(MI_FORCE_SYRK_TILE)  // tuning builds only: 128, 1282, 192 or 256
+  if (MI_FORCE_SYRK_TILE == 192) return SYRK_TILE_192;
+  if (MI_FORCE_SYRK_TILE == 256 && n % 256 == 0) return SYRK_TILE_256;
+  if (MI_FORCE_SYRK_TILE == 128 && n % 128 == 0) return SYRK_TILE_128;
+  if (MI_FORCE_SYRK_TILE == 1282 && n % 128 == 0) return SYRK_TILE_128X2;
 #endif
 #ifdef MI_HAS_SMALL_CFGS
   const int64_t cus = num_cus();
-  auto rounds = [&](int64_t tile) {
+  const double kt = (double)ceil_div(k, 64);
+  auto tiles = [&](int64_t tile) {
     const int64_t t = ceil_div(n, tile);
-    return ceil_div(t * (t + 1) / 2 * batch, cus);
+    return t * (t + 1) / 2 * batch;
   };
-  const double cost192 = (double)rounds(192) * 192.0 * 192.0;
-  const double cost128 = (double)rounds(128) * 128.0 * 128.0 * 1.4;
-  if (n % 128 == 0 && cost128 < cost192) return SYRK_TILE_128;
+  SyrkTile best = SYRK_TILE_192;
+  double best_cost = (double)ceil_div(tiles(192), cus) * (12.6 + 0.80 * kt);
+  auto offer = [&](SyrkTile t, double cost) {
+    if (cost < best_cost) best = t, best_cost = cost;
+  };
+  if (n % 256 == 0) offer(SYRK_TILE_256, (double)ceil_div(tiles(256), cus) * (29.7 + 1.30 * kt));
+  if (n % 128 == 0) {
+    const int64_t t128 = tiles(128);
+    const double s2 = 0.74 + 0.11 * std::min(std::max(kt - 32.0, 0.0) / 96.0, 1.0);
+    offer(SYRK_TILE_128X2, (double)ceil_div(t128, 2 * cus) * (9.2 + s2 * kt));
+    offer(SYRK_TILE_128, (double)ceil_div(t128, cus) * (9.0 + (t128 <= cus ? 0.31 : 0.44) * kt));
+  }
+  return best;
 #else
-  (void)n; (void)batch;
-#endif
+  (void)n; (void)batch; (void)k;
   return SYRK_TILE_192;
+#endif
 }
 // 256 x 128 instead of 256 x 256 GEMM tiles for the whole product?
 static bool gemm_prefers_half_tiles(int64_t m, int64_t n, int64_t batch) {
@@ -179,10 +202,18 @@ static int launch_class(TileClass tc, const GemmParams& p, int64_t batch, hipStr
   const bool k_ok = p.K % 64 == 0 && p.K >= 64;
   if (k_ok && p.M >= 1024 && p.N >= 1024) {
     if constexpr (MODE == MODE_SYRK && !P_KS && !Q_KS) {
+      switch (pick_syrk_tile(p.M, batch, p.K)) {
 #ifdef MI_HAS_SMALL_CFGS
-      if (pick_syrk_tile(p.M, batch) == SYRK_TILE_128) return launch_fast<CfgT128, false, false, MODE, OUT_F32>(p, batch, stream);
+        case SYRK_TILE_128:
+          return launch_fast<CfgT128, false, false, MODE, OUT_F32>(p, batch, stream);
+        case SYRK_TILE_128X2:
+          return launch_fast<CfgT128x2, false, false, MODE, OUT_F32>(p, batch, stream);
 #endif
-      return launch_fast<CfgSyrk192, false, false, MODE, OUT_F32>(p, batch, stream);
+        case SYRK_TILE_256:
+          return launch_fast<CfgBig, false, false, MODE, OUT_F32>(p, batch, stream);
+        default:
+          return launch_fast<CfgSyrk192, false, false, MODE, OUT_F32>(p, batch, stream);
+      }
     }
     if constexpr (MODE == MODE_GEMM && !P_KS && Q_KS) {
       if (p.M % 256 == 0 && p.N % 256 == 0 && gemm_prefers_half_tiles(p.M, p.N, batch))

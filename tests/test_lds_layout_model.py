@@ -141,3 +141,158 @@ def test_compact_transpose_read_address_equals_direct_formula(rows):
                     col, kb = wb + 16 * r + 4 * (i16 & 3), 32 * q + 8 * g + (i16 >> 2)
                     ref = [k * rowb + (((col >> 3) + ks_rot(16, k)) & (ch - 1)) * 16 + (col & 7) * 2 for k in (kb, kb + 4)]
                     assert [a0, a1] == ref
+
+
+# ---- SYRK-mode epilogue: tile assembled row-major in LDS, mirror image formed with the LDS transpose read ----
+#
+# Restates `syrk_epilogue_lds` lane by lane: staging of the accumulator quads, the in-LDS fill of the upper 4 x 4
+# blocks of a diagonal wavefront block, the row-wise write-out and the transposed write-out.  The check is that
+# global memory ends up holding exactly the lower-triangle values and their mirror image, every element written
+# once, for every tile shape the library instantiates.
+
+
+def tr_read(lds, addr_of_lane):
+    """ds_read_b64_tr_b16: result lane i, element e <- source lane 4e + i/4, element i%4 (per 16-lane group)."""
+    out = []
+    for lane in range(64):
+        grp, i = lane & ~15, lane & 15
+        out.append([lds.get(addr_of_lane[grp + 4 * e + i // 4] + 2 * (i % 4)) for e in range(4)])
+    return out
+
+
+def syrk_epilogue_model(tile, mi, npass, diag, skip_upper=False):
+    tm = tile // 2
+    ldt, rp = tile + 8, tile // npass
+    g_cnt = 4 if mi == 32 else 1
+    fm = tm // mi
+    sym, mirror = diag and not skip_upper, not skip_upper
+    m0, n0 = (tile, tile) if diag else (2 * tile, 0)
+    out = {}
+
+    def value(ml, nl):  # what the accumulators of the wavefront owning (ml, nl) hold
+        return ("v", ml, nl)
+
+    def store(row, col, vals):
+        for t, v in enumerate(vals):
+            assert (row, col + t) not in out, "element written twice"
+            out[(row, col + t)] = v
+
+    for h in range(npass):
+        lds = {}
+
+        def put(row, col, v):
+            assert 0 <= row < rp and 0 <= col < tile
+            lds[(row * ldt + col) * 2] = v
+
+        # staging
+        for wave in range(4):
+            wm, wn = wave // 2, wave % 2
+            mw, nw = wm * tm, wn * tm
+            if mw // rp != h:
+                continue
+            for lane in range(64):
+                frow, fk = lane & (mi - 1), lane // mi
+                for i in range(fm):
+                    for j in range(fm):
+                        for g in range(g_cnt):
+                            ml, nl = mw + i * mi + frow, nw + j * mi + (8 * g if mi == 32 else 0) + 4 * fk
+                            quad = [value(ml, nl + r) for r in range(4)]
+                            if not sym or wm > wn:
+                                for r in range(4):
+                                    put(ml - h * rp, nl + r, quad[r])
+                            elif wm == wn:
+                                if i > j or (i == j and nl < (ml & ~3)):
+                                    for r in range(4):
+                                        put(ml - h * rp, nl + r, quad[r])
+                                elif i == j and nl == (ml & ~3):
+                                    for r in range(4):
+                                        if nl + r <= ml:
+                                            put(ml - h * rp, nl + r, quad[r])
+                                        if nl + r < ml:
+                                            put(nl + r - h * rp, ml, quad[r])
+        # upper 4 x 4 blocks of a diagonal wavefront block
+        if sym:
+            for wave in (0, 3):
+                mw = (wave // 2) * tm
+                if mw // rp != h:
+                    continue
+                nb4 = tm // 4
+                assert nb4 * nb4 % 16 == 0
+                rowbase, colbase = mw - h * rp, mw
+                for it in range(nb4 * nb4 // 16):
+                    addr = []
+                    for lane in range(64):
+                        ids = it * 16 + 4 * (lane // 16) + (lane % 4)
+                        brs, bcs, e = ids // nb4, ids % nb4, (lane % 16) // 4
+                        addr.append(((rowbase + 4 * brs + e) * ldt + colbase + 4 * bcs) * 2)
+                    got = tr_read(lds, addr)
+                    for lane in range(64):
+                        idr = it * 16 + lane // 4
+                        br, bc, r = idr // nb4, idr % nb4, lane % 4
+                        if br > bc:
+                            for t in range(4):
+                                put(rowbase + 4 * bc + r, colbase + 4 * br + t, got[lane][t])
+        # row-wise write-out
+        cprw = tile // 8
+        assert rp * cprw % 256 == 0
+        for it in range(rp * cprw // 256):
+            for tid in range(256):
+                c = tid + it * 256
+                row, c8 = c // cprw, c % cprw
+                ml = h * rp + row
+                if sym and c8 * 8 >= (ml // tm + 1) * tm:
+                    continue
+                store(m0 + ml, n0 + c8 * 8, [lds[(row * ldt + c8 * 8 + t) * 2] for t in range(8)])
+        # transposed write-out
+        if mirror:
+            if sym:
+                lo, hi = max(tm, h * rp), min(tile, (h + 1) * rp)
+                r_lo, rows, ccols = lo - h * rp, max(hi - lo, 0), tm
+            else:
+                r_lo, rows, ccols = 0, rp, tile
+            assert rows % 32 == 0
+            nb = rows // 32
+            units = (ccols // 4) * nb
+            for it in range((units + 15) // 16):
+                for wave in range(4):
+                    addr0, meta = [], []
+                    for lane in range(64):
+                        unit = it * 16 + wave * 4 + lane // 16
+                        on = unit < units
+                        u = min(unit, max(units - 1, 0))
+                        cq, rb = (u // nb, u % nb) if nb else (0, 0)
+                        L = lane % 16
+                        addr0.append(((r_lo + 32 * rb + 8 * (L % 4) + L // 4) * ldt + 4 * cq) * 2)
+                        meta.append((on, cq, rb, L // 4, L % 4))
+                    if units == 0:
+                        continue
+                    t0 = tr_read(lds, addr0)
+                    t1 = tr_read(lds, [a + 4 * ldt * 2 for a in addr0])
+                    for lane in range(64):
+                        on, cq, rb, q, r = meta[lane]
+                        if on:
+                            store(n0 + 4 * cq + r, m0 + h * rp + r_lo + 32 * rb + 8 * q, t0[lane] + t1[lane])
+    return out, (m0, n0)
+
+
+@pytest.mark.parametrize("tile,mi,npass", [(192, 16, 1), (256, 16, 2), (128, 16, 1), (256, 32, 2), (192, 32, 1)])
+@pytest.mark.parametrize("diag", [False, True])
+def test_syrk_epilogue_writes_the_tile_and_its_mirror_image(tile, mi, npass, diag):
+    if mi == 32 and (tile // 2) % 32:
+        pytest.skip("a 96-row wavefront block is not a multiple of the 32 x 32 MFMA tile")
+    out, (m0, n0) = syrk_epilogue_model(tile, mi, npass, diag)
+    expect = {}
+    for a in range(tile):
+        for b in range(tile):
+            if diag:
+                expect[(m0 + a, n0 + b)] = ("v", max(a, b), min(a, b))
+            else:
+                expect[(m0 + a, n0 + b)] = ("v", a, b)
+                expect[(n0 + b, m0 + a)] = ("v", a, b)
+    assert out == expect
+
+
+@pytest.mark.parametrize("tile,npass", [(192, 1), (256, 2)])
+def test_syrk_epilogue_lower_only(tile, npass):
+    out, (m0, n0) = syrk_epilogue_model(tile, 16, npass, diag=False, skip_upper=True)
+    assert out == {(m0 + a, n0 + b): ("v", a, b) for a in range(tile) for b in range(tile)}
