@@ -1,0 +1,117 @@
+"""Static check of the compiled gfx950 kernels: no accumulator-register traffic next to the MFMA instructions.
+
+The fast kernels issue their MFMAs as inline assembly with the accumulators tied in place (AGPRs), so the compiler
+neither sees an MFMA nor inserts the wait states an MFMA result needs before a VALU or memory instruction may read
+it.  That is safe only while the register allocator keeps every accumulator where it is for the whole K loop and
+the first read of an accumulator follows the drain (three ``s_nop 7``) after the loop.  A change elsewhere in a
+kernel (register pressure in the epilogue, for instance) can make the allocator swap or spill accumulator registers
+inside the loop; the result is then wrong in a few elements only.  This test compiles the library to assembly and
+rejects, for every fast kernel,
+  * any ``v_accvgpr_*`` move or AGPR spill inside an innermost loop that contains MFMAs,
+  * any such instruction between an MFMA and the drain that follows it.
+No GPU is involved.
+"""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "emerging-optimizers_amd", "csrc")
+FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-Wno-unused-command-line-argument", "--cuda-device-only", "-S"]
+
+ACC_TRAFFIC = re.compile(r"^\s*(v_accvgpr_\w+|scratch_(store|load)\w*\s+(off,\s*)?a\[|scratch_load\w*\s+a\[)")
+
+
+def instructions(lines):
+    """(index, text) of the lines that are instructions or labels (comments, directives and asm markers dropped)."""
+    out = []
+    for i, raw in enumerate(lines):
+        t = raw.split(";")[0].strip()
+        if not t or t.startswith(".") and not t.endswith(":") or t.startswith(";;"):
+            continue
+        out.append((i, t))
+    return out
+
+
+def accumulator_hazards(lines):
+    ins = instructions(lines)
+    text = [t for _, t in ins]
+    label_at = {t[:-1]: k for k, t in enumerate(text) if t.endswith(":")}
+    bad = []
+    # innermost loops (a branch back to an earlier label with no other loop inside)
+    loops = []
+    for k, t in enumerate(text):
+        m = re.match(r"s_cbranch_\w+\s+(\S+)|s_branch\s+(\S+)", t)
+        if m:
+            target = label_at.get(m.group(1) or m.group(2))
+            if target is not None and target <= k:
+                loops.append((target, k))
+    for lo, hi in loops:
+        if any((a, b) != (lo, hi) and lo <= a and b <= hi for a, b in loops):
+            continue
+        body = text[lo:hi]
+        if any(x.startswith("v_mfma") for x in body):
+            bad += [f"in MFMA loop: {x}" for x in body if ACC_TRAFFIC.match(x)]
+    # between an MFMA and the drain (or the next MFMA)
+    for k, t in enumerate(text):
+        if not t.startswith("v_mfma"):
+            continue
+        for x in text[k + 1:k + 13]:
+            if x.startswith("v_mfma") or x.startswith("s_nop 7"):
+                break
+            if ACC_TRAFFIC.match(x):
+                bad.append(f"after MFMA, before the drain: {x}")
+    return bad
+
+
+def test_detector_flags_swaps_and_spills():
+    swap = """
+.LBB0_1:
+	v_accvgpr_read_b32 v66, a220
+	v_accvgpr_mov_b32 a220, a0
+	;;#ASMSTART
+	v_mfma_f32_16x16x32_bf16 a[0:3], v[14:17], v[46:49], a[0:3]
+	;;#ASMEND
+	s_cbranch_scc1 .LBB0_1
+""".splitlines()
+    assert len(accumulator_hazards(swap)) == 2
+    spill = """
+	v_mfma_f32_16x16x32_bf16 a[0:3], v[14:17], v[46:49], a[0:3]
+	scratch_store_dwordx4 off, a[232:235], off offset:100 ; 16-byte Folded Spill
+	s_nop 7
+	v_accvgpr_read_b32 v1, a0
+""".splitlines()
+    assert accumulator_hazards(spill) == ["after MFMA, before the drain: scratch_store_dwordx4 off, a[232:235], off offset:100"]
+    clean = """
+.LBB0_1:
+	v_mfma_f32_16x16x32_bf16 a[0:3], v[14:17], v[46:49], a[0:3]
+	ds_read_b64_tr_b16 v[118:119], v66
+	s_cbranch_scc1 .LBB0_1
+	s_nop 7
+	v_accvgpr_read_b32 v1, a0
+""".splitlines()
+    assert accumulator_hazards(clean) == []
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="hipcc not available")
+def test_no_accumulator_traffic_next_to_mfma(tmp_path):
+    asm = tmp_path / "mi_ns.s"
+    subprocess.run(["hipcc", *FLAGS, "mi_ns.hip", "-o", str(asm)], cwd=CSRC, check=True, capture_output=True, timeout=900)
+    kernels, name = {}, None
+    for line in asm.read_text().splitlines():
+        m = re.match(r"^(_ZN2mi\S+):\s", line)
+        if m:
+            name = m.group(1)
+            kernels[name] = []
+        elif name:
+            kernels[name].append(line)
+            if "s_endpgm" in line:
+                name = None
+    fast = {n: ls for n, ls in kernels.items() if "gemm_fast_kernel" in n or "small_chain_kernel" in n}
+    assert len(fast) >= 20 and all(any("v_mfma" in x for x in ls) for ls in fast.values())
+    report = {n: accumulator_hazards(ls) for n, ls in fast.items()}
+    report = {n: b for n, b in report.items() if b}
+    assert not report, "\n".join(f"{n}: {len(b)} hazards, e.g. {b[0]}" for n, b in report.items())
