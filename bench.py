@@ -28,10 +28,10 @@ for _p in (ROOT, os.path.join(ROOT, "emerging-optimizers_amd")):
 PEAK_BF16_TFLOPS = 2516.6  # MI355X dense bf16 MFMA: 256 CU x 2.4 GHz x 4096 FLOP/clk/CU
 # HBM-side bytes of one GEMM+AXPY at the headline shape (both launches), from two `rocprofv3 --pmc` runs of this file
 # (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same counter reads for sumsq_kernel
-# of the same run, whose traffic is known (229 376 KiB read, 114 696 KiB written): factors 1.9993 and 0.9998.
-GEMM_AXPY_TRAFFIC_BYTES = int(((406432.7 + 146832.3) * 1.9993 + (98328.0 + 16392.0) * 0.9998) * 1024)
+# of the same run, whose traffic is known (229 376 KiB read, 114 696 KiB written): factors 1.9994 and 0.9998.
+GEMM_AXPY_TRAFFIC_BYTES = int(((405915.0 + 146831.8) * 1.9994 + (98328.0 + 16392.0) * 0.9998) * 1024)
 # The same for the lower-triangle kernel, averaged over its 16 launches per call (2 x X X^T, 14 m x m products).
-TRI_KERNEL_TRAFFIC_BYTES = int((128714.6 * 1.9993 + 32768.0 * 0.9998) * 1024)
+TRI_KERNEL_TRAFFIC_BYTES = int((128715.5 * 1.9994 + 32768.1 * 0.9998) * 1024)
 M, N, NS_STEPS = 4096, 14336, 5
 # Other benchmark configurations, timed with --workload (the default, "mlp", is the headline).
 WORKLOADS = {
