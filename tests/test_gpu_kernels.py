@@ -41,7 +41,7 @@ def test_syrk_integer_exact(gpu, fn, n, k, trans):
 
 
 @pytest.mark.parametrize("fn", SYRK_2D)
-@pytest.mark.parametrize("n,alpha", [(128, 0.5), (256, 0.25), (1024, 0.25)])
+@pytest.mark.parametrize("n,alpha", [(128, 0.5), (256, 0.25), (1024, 0.25), (5120, 0.25)])  # 5120: 256 x 256 tiles
 @pytest.mark.parametrize("trans", [False, True])
 def test_syrk_addmm_integer_exact(gpu, fn, n, alpha, trans):
     s = _int_bf16((n, n), -3, 3, gpu)
@@ -84,7 +84,8 @@ def test_syrk_skip_upper_triangle(gpu):
     assert torch.equal(torch.tril(d.float()), torch.tril(ref.float()))
 
 
-@pytest.mark.parametrize("b,n,k", [(2, 128, 128), (4, 256, 64), (8, 16, 128), (2, 1024, 64), (3, 40, 24)])
+# (8, 1024, 256): 128 x 128 tiles two to a CU; (8, 1792, 4096): 256 x 256 tiles, then 128 x 128 with addend
+@pytest.mark.parametrize("b,n,k", [(2, 128, 128), (4, 256, 64), (8, 16, 128), (2, 1024, 64), (3, 40, 24), (8, 1024, 256), (8, 1792, 4096)])
 @pytest.mark.parametrize("trans", [False, True])
 def test_batched_syrk_integer_exact(gpu, b, n, k, trans):
     a = _int_bf16((b, k, n) if trans else (b, n, k), -3, 3, gpu)
