@@ -485,6 +485,7 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
   static_assert(RP * LDT * 2 <= S::RING, "staging pass exceeds the ring");
   static_assert(RP % C::TM == 0 && RP % C::TN == 0, "a wavefront's block must fall into one pass");
   static_assert(C::KSPLIT == 1 && C::TILE_M == C::TILE_N, "square tiles, one K group");
+  static_assert(C::WGM == 2 && C::WGN == 2 && C::TM == C::TN, "2 x 2 wavefronts with square blocks: the diagonal blocks are (0,0) and (1,1)");
   static_assert(RP * CPRW % C::NT == 0, "write-out must divide evenly");
   const int tid = threadIdx.x;
   const int frow = lane & (MI - 1), fk = lane / MI;
