@@ -202,18 +202,21 @@ static int launch_class(TileClass tc, const GemmParams& p, int64_t batch, hipStr
   const bool k_ok = p.K % 64 == 0 && p.K >= 64;
   if (k_ok && p.M >= 1024 && p.N >= 1024) {
     if constexpr (MODE == MODE_SYRK && !P_KS && !Q_KS) {
-      switch (pick_syrk_tile(p.M, batch, p.K)) {
+      auto launch_tile = [&](const GemmParams& q, int64_t b) {
+        switch (pick_syrk_tile(q.M, b, q.K)) {
 #ifdef MI_HAS_SMALL_CFGS
-        case SYRK_TILE_128:
-          return launch_fast<CfgT128, false, false, MODE, OUT_F32>(p, batch, stream);
-        case SYRK_TILE_128X2:
-          return launch_fast<CfgT128x2, false, false, MODE, OUT_F32>(p, batch, stream);
+          case SYRK_TILE_128:
+            return launch_fast<CfgT128, false, false, MODE, OUT_F32>(q, b, stream);
+          case SYRK_TILE_128X2:
+            return launch_fast<CfgT128x2, false, false, MODE, OUT_F32>(q, b, stream);
 #endif
-        case SYRK_TILE_256:
-          return launch_fast<CfgBig, false, false, MODE, OUT_F32>(p, batch, stream);
-        default:
-          return launch_fast<CfgSyrk192, false, false, MODE, OUT_F32>(p, batch, stream);
-      }
+          case SYRK_TILE_256:
+            return launch_fast<CfgBig, false, false, MODE, OUT_F32>(q, b, stream);
+          default:
+            return launch_fast<CfgSyrk192, false, false, MODE, OUT_F32>(q, b, stream);
+        }
+      };
+      return launch_tile(p, batch);
     }
     if constexpr (MODE == MODE_GEMM && !P_KS && Q_KS) {
       if (p.M % 256 == 0 && p.N % 256 == 0 && gemm_prefers_half_tiles(p.M, p.N, batch))

@@ -84,8 +84,10 @@ def test_syrk_skip_upper_triangle(gpu):
     assert torch.equal(torch.tril(d.float()), torch.tril(ref.float()))
 
 
-# (8, 1024, 256): 128 x 128 tiles two to a CU; (8, 1792, 4096): 256 x 256 tiles, then 128 x 128 with addend
-@pytest.mark.parametrize("b,n,k", [(2, 128, 128), (4, 256, 64), (8, 16, 128), (2, 1024, 64), (3, 40, 24), (8, 1024, 256), (8, 1792, 4096)])
+# (8, 1024, 256): 128 x 128 tiles two to a CU; (8, 1792, 4096): 256 x 256 tiles, then 128 x 128 with addend;
+# (4, 2048, 2048): 544 tiles of 128 x 128, more than one round of two per CU
+@pytest.mark.parametrize("b,n,k", [(2, 128, 128), (4, 256, 64), (8, 16, 128), (2, 1024, 64), (3, 40, 24), (8, 1024, 256), (8, 1792, 4096),
+                                   (4, 2048, 2048)])
 @pytest.mark.parametrize("trans", [False, True])
 def test_batched_syrk_integer_exact(gpu, b, n, k, trans):
     a = _int_bf16((b, k, n) if trans else (b, n, k), -3, 3, gpu)
