@@ -61,6 +61,7 @@ struct GemmParams {
   const float* xscale;
   float* slots_out;          // GEMM mode: per-workgroup sum of squares of the output,
   int slot_stride, slot_base;  //   at slots_out[batch * slot_stride + slot_base + blockIdx.x]
+  int slot_capacity;         // host side only: floats reserved per batch entry behind slots_out (0: not checked)
 };
 
 // Consecutive steps can share one Gram matrix, because every factor involved is a polynomial of it and they all

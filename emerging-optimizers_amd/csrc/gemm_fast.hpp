@@ -34,19 +34,15 @@ __device__ __forceinline__ void static_for(F&& f) {
   static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
-// Compile-time shape of one fast-kernel variant.
-template <int TILE_M_, int WGM_, int WGN_, int BK_, int NS_, int KSPLIT_ = 1, int TILE_N_ = TILE_M_, int MI_ = 32>
+// Compile-time shape of one fast-kernel variant.  The MFMA is v_mfma_f32_16x16x32_bf16 throughout: of the two bf16
+// shapes (same peak) it moves a quarter of the accumulator registers per instruction and draws less power per FLOP
+// on random operands, which is what bounds the clock on this part.
+template <int TILE_M_, int WGM_, int WGN_, int BK_, int NS_, int TILE_N_ = TILE_M_>
 struct FastCfg {
-  // MFMA shape: MI = 32 -> v_mfma_f32_32x32x16_bf16, MI = 16 -> v_mfma_f32_16x16x32_bf16 (KI = k per MFMA).
-  // Both do 16 K FLOP per pass; on random operands the 16 x 16 shape draws less power per FLOP (it moves a
-  // quarter of the accumulator registers per instruction), which is what bounds the clock on this part.
-  static constexpr int MI = MI_, KI = MI_ == 32 ? 16 : 32;
+  static constexpr int MI = 16, KI = 32;                     // MFMA tile rows / k per MFMA
   static constexpr int TILE_M = TILE_M_, TILE_N = TILE_N_;  // workgroup tile: rows of P x rows of Q
   static constexpr int TILE = TILE_M_;                      // (SYRK uses square tiles)
-  // KSPLIT groups of WGM x WGN wavefronts each cover the whole tile and take alternate 16-wide k-steps; their
-  // accumulators are added through LDS after the K loop (two wavefronts per SIMD with large wave tiles).
-  static constexpr int KSPLIT = KSPLIT_;
-  static constexpr int WGM = WGM_, WGN = WGN_, NWG = WGM * WGN, NW = NWG * KSPLIT, NT = NW * 64;
+  static constexpr int WGM = WGM_, WGN = WGN_, NW = WGM * WGN, NT = NW * 64;
   static constexpr int TM = TILE_M / WGM, TN = TILE_N / WGN, FM = TM / MI, FN = TN / MI;
   static constexpr int BK = BK_;                       // k extent of one ring slot
   static constexpr int NS = NS_;                       // ring slots
@@ -57,67 +53,28 @@ struct FastCfg {
   static constexpr int CPR = BK / 8;                   // 16-byte chunks per K-contiguous LDS row
   static constexpr int ROWS_PER_KB = 1024 / (BK * 2);  // K-contiguous rows covered by one 1 KB load
   static_assert(BK == 32 || BK == 64, "ring slot depth");
-  static_assert(KSPLIT == 1 || KSPLIT == 2, "at most two K groups");
-  static_assert(MI == 32 || MI == 16, "MFMA shape");
-  static_assert((BK / KI) % (2 * KSPLIT) == 0, "each K group needs an even number of k-steps per tile");
+  static_assert((BK / KI) % 2 == 0, "an even number of k-steps per tile");
   static_assert(TM % MI == 0 && TN % MI == 0, "wave tile must be a multiple of the MFMA tile");
   static_assert(P_BYTES % (1024 * NW) == 0 && Q_BYTES % (1024 * NW) == 0,
                 "tiles must split evenly over the wavefronts' 1 KB loads");
   static_assert(NS * SLOT_BYTES <= 160 * 1024 - 256, "ring exceeds the 160 KB LDS");
 };
-#ifndef MI_SHAPE
-#define MI_SHAPE 16
-#endif
-#if MI_SHAPE == 32
-// MFMA-bound default: 256 x 256 tile, 8 wavefronts (2 per SIMD) of 128 x 64, two 64 KB slots.
-#ifndef MI_BIG_WGN
-#define MI_BIG_WGN 4
-#endif
-#ifndef MI_BIG_BK
-#define MI_BIG_BK 64
-#define MI_BIG_NS 2
-#endif
-using CfgBig = FastCfg<256, 2, MI_BIG_WGN, MI_BIG_BK, MI_BIG_NS>;
-// Half-width tile for the last partial round of a GEMM: 256 x 128, wavefronts of 128 x 32.
-using CfgHalfN = FastCfg<256, 2, 4, 64, 2, 1, 128>;
-// SYRK on ~4096-row Gram matrices: 192 x 192 tiles give 22 * 23 / 2 = 253 lower-triangle tiles, one per
-// CU in a single round (256 x 256 tiles would give 136 and leave 47 % of the CUs idle).
-// 2 K-groups x 4 wavefronts of 96 x 96, three 48 KB slots (two K tiles in flight).
-#ifndef MI_SYRK192_KSPLIT
-#define MI_SYRK192_KSPLIT 2
-#endif
-using CfgSyrk192 = FastCfg<192, 2, 2, 64, 3, MI_SYRK192_KSPLIT>;
-#else
-// 16 x 16 x 32 MFMA variants: one wavefront per SIMD (4 per workgroup), accumulators in 256 / 128 / 144 registers.
-#define MI_HAS_SMALL_CFGS 1
+// One wavefront per SIMD (4 per workgroup), accumulators in 256 / 128 / 144 registers.
 // Batched small matrices (per-head shapes, 128 rows): GEMM+AXPY tile 128 x 256 (wavefronts of 128 x 64) and a
 // 128 x 128 tile (wavefronts of 64 x 64) for the split-K Gram partials.
-using CfgM128 = FastCfg<128, 1, 4, 64, 2, 1, 256, 16>;
-#ifndef MI_T128_NS
-#define MI_T128_NS 3
-#endif
-using CfgT128 = FastCfg<128, 2, 2, 64, MI_T128_NS, 1, 128, 16>;
+using CfgM128 = FastCfg<128, 1, 4, 64, 2, 256>;
+using CfgT128 = FastCfg<128, 2, 2, 64, 3, 128>;
 // The same tile with a two-slot ring (64 KB): two workgroups share a CU, so one's epilogue overlaps the other's K loop.
-using CfgT128x2 = FastCfg<128, 2, 2, 64, 2, 1, 128, 16>;
-using CfgBig = FastCfg<256, 2, 2, 64, 2, 1, 256, 16>;     // wavefronts of 128 x 128
-#ifndef MI_HALFN_NS
-#define MI_HALFN_NS 3
-#endif
-using CfgHalfN = FastCfg<256, 2, 2, 64, MI_HALFN_NS, 1, 128, 16>;   // wavefronts of 128 x 64
-using CfgSyrk192 = FastCfg<192, 2, 2, 64, 3, 1, 192, 16>;  // wavefronts of 96 x 96
-#endif
+using CfgT128x2 = FastCfg<128, 2, 2, 64, 2, 128>;
+using CfgBig = FastCfg<256, 2, 2, 64, 2, 256>;      // wavefronts of 128 x 128
+using CfgHalfN = FastCfg<256, 2, 2, 64, 3, 128>;    // wavefronts of 128 x 64
+using CfgSyrk192 = FastCfg<192, 2, 2, 64, 3, 192>;  // wavefronts of 96 x 96
 
-template <int MI> struct AccVec { typedef f32x16_t type; };
-template <> struct AccVec<16> { typedef f32x4_t type; };
 
-// Rotation (in 16-byte chunks) of k-row k of a K-strided LDS tile.  It is chosen per MFMA shape so that the
-// k-rows which one pass of the transpose read touches (32 lanes) fall on disjoint banks:
-//   MI = 32: a pass reads 4 k-rows x 64 B  -> 64 B per k
-//   MI = 16: a pass reads 4 k-rows x 32 B at k and at k + 8 -> 32 B per k inside an 8-row group, 128 B per group
-template <int MI>
-__device__ __forceinline__ int ks_rot(int k) {
-  return MI == 32 ? 4 * k : 2 * (k & 7) + 8 * (k >> 3);
-}
+// Rotation (in 16-byte chunks) of k-row k of a K-strided LDS tile, chosen so that the k-rows which one pass of the
+// transpose read touches (32 lanes: 4 k-rows x 32 B at k and at k + 8) fall on disjoint banks: 32 B per k inside an
+// 8-row group, 128 B per group.
+__device__ __forceinline__ int ks_rot(int k) { return 2 * (k & 7) + 8 * (k >> 3); }
 
 // Direct-to-LDS load: every lane fetches 16 bytes from its own global address; the wavefront's 1 KB lands
 // at LDS byte address `lds_addr` + 16 * lane (`lds_addr` is wave-uniform and travels in M0).  Written as inline assembly so
@@ -126,9 +83,7 @@ __device__ __forceinline__ int ks_rot(int k) {
 // (M0 is a reserved register: the compiler never keeps a value in it across statements, so it is not
 // listed as clobbered.)
 __device__ __forceinline__ void dma16(const uint16_t* g, uint32_t lds_addr) {
-#ifndef MI_ABLATE_LOADS
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(g) : "memory");
-#endif
 }
 
 // XOR swizzle of the K-contiguous LDS tile: chunk c of row r is stored at slot kc_slot(r, c) of its row, so
@@ -142,9 +97,7 @@ __device__ __forceinline__ int kc_slot(int row, int c) {
 // offset: the blocks of one tile differ only in the base, so a handful of offset registers serve all loads
 // of an operand and the per-load address arithmetic runs on the scalar unit.
 __device__ __forceinline__ void dma16_sv(uint64_t sbase, uint32_t voff, uint32_t lds_addr) {
-#ifndef MI_ABLATE_LOADS
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(sbase) : "memory");
-#endif
 }
 
 // Direct-to-LDS loads of one operand tile (ROWS rows of the operand x BK along k).  The tile is cut into
@@ -160,12 +113,13 @@ struct FastLoader {
   static constexpr int KS_CHUNKS = ROWS / 8;          // 16-byte chunks per k-row of the K-strided layout
   static constexpr int KS_ROWS_PER_KB = 512 / ROWS;   // k-rows covered by one 1 KB load
   // period of the swizzle phase in the block index
-  static constexpr int PERIOD = KS ? (C::MI == 32 ? (KS_CHUNKS / (4 * KS_ROWS_PER_KB) > 0 ? KS_CHUNKS / (4 * KS_ROWS_PER_KB) : 1)
-                                                  : (KS_CHUNKS / KS_ROWS_PER_KB > 0 ? KS_CHUNKS / KS_ROWS_PER_KB : 1))
-                                   : (C::BK == 64 ? 2 : 1);
+  static constexpr int PERIOD = KS ? (KS_CHUNKS / KS_ROWS_PER_KB > 0 ? KS_CHUNKS / KS_ROWS_PER_KB : 1) : (C::BK == 64 ? 2 : 1);
   static constexpr bool PERIODIC = LPT % PERIOD == 0;  // then the phase of load i is i % PERIOD for every wavefront
   static constexpr int NV = CLAMP ? 1 : (PERIODIC ? (PERIOD < LPT ? PERIOD : LPT) : LPT);
   static_assert(!KS || ROWS == 256 || ROWS == 128, "K-strided LDS layout is laid out for 128/256-wide tiles");
+  // (a K-strided tile at the edge of its operand would need clamping along the contiguous dimension, which a
+  // 16-byte load cannot do per element: the launcher never sends such a tile here)
+  static_assert(!(KS && CLAMP), "edge tiles of K-strided operands are not served by the fast kernel");
 
   const uint16_t* gp[CLAMP ? LPT : 1];  // CLAMP: per-load pointers
   uint32_t voff[NV];                    // !CLAMP: per-lane byte offsets inside a block
@@ -181,7 +135,7 @@ struct FastLoader {
       return (int64_t)lr * ld + c * 8;
     } else {
       const int kr = lane / KS_CHUNKS;
-      const int c = ((lane % KS_CHUNKS) - ks_rot<C::MI>(KS_ROWS_PER_KB * b + kr)) & (KS_CHUNKS - 1);
+      const int c = ((lane % KS_CHUNKS) - ks_rot(KS_ROWS_PER_KB * b + kr)) & (KS_CHUNKS - 1);
       return (int64_t)kr * ld + c * 8;
     }
   }
@@ -191,19 +145,13 @@ struct FastLoader {
 #pragma unroll
       for (int i = 0; i < LPT; ++i) {
         const int b = wave * LPT + i;  // 1 KB block index inside the tile
-        if (!KS) {
-          const int row = C::ROWS_PER_KB * b + lane / C::CPR;
-          const int c = kc_slot<C::BK>(row, lane % C::CPR);
-          int gr = row0 + row;
-          gr = gr < rows_valid ? gr : rows_valid - 1;
-          gp[i] = opbase + (int64_t)gr * ld + c * 8;
-        } else {
-          const int k = KS_ROWS_PER_KB * b + lane / KS_CHUNKS;
-          const int c = ((lane % KS_CHUNKS) - ks_rot<C::MI>(k)) & (KS_CHUNKS - 1);
-          gp[i] = opbase + (int64_t)k * ld + row0 + c * 8;
-        }
+        const int row = C::ROWS_PER_KB * b + lane / C::CPR;
+        const int c = kc_slot<C::BK>(row, lane % C::CPR);
+        int gr = row0 + row;
+        gr = gr < rows_valid ? gr : rows_valid - 1;
+        gp[i] = opbase + (int64_t)gr * ld + c * 8;
       }
-      step = KS ? (int64_t)C::BK * ld : C::BK;
+      step = C::BK;
     } else {
       const int b0 = wave * LPT;
 #pragma unroll
@@ -232,44 +180,18 @@ struct FastLoader {
   }
 };
 
-// MFMA fragment (8 bf16 along k per lane) for MI consecutive rows starting at `row_base`, k-step q (KI k each).
-//   MI = 32: lane l -> row l % 32, k = 16 q + 8 (l / 32) .. +7
-//   MI = 16: lane l -> row l % 16, k = 32 q + 8 (l / 16) .. +7
-// K-strided tiles are read with the LDS transpose read: its 16 lanes fetch 4 k-rows x 16 rows (8 bytes per
-// lane: 4 consecutive rows at one k) and every lane receives the 4 k-values of its own row.
-template <class C, bool KS, int ROWS>
+// MFMA fragment (8 bf16 along k per lane) of a K-contiguous tile for 16 consecutive rows starting at `row_base`,
+// k-step q (32 k each): lane l -> row l % 16, k = 32 q + 8 (l / 16) .. +7.
+template <class C>
 __device__ __forceinline__ bf16x8_t fast_frag(const char* tile, int row_base, int q, int lane) {
-  constexpr int KS_CHUNKS = ROWS / 8, KS_ROW_BYTES = ROWS * 2, MI = C::MI;
-  const int kgrp = MI == 32 ? (lane >> 5) : (lane >> 4);  // which 8-wide k group of the k-step this lane feeds
-  if (!KS) {
-    const int row = row_base + (lane & (MI - 1));
-    const int c = kc_slot<C::BK>(row, (C::KI / 8) * q + kgrp);
-    return *reinterpret_cast<const bf16x8_t*>(tile + row * (C::BK * 2) + c * 16);
-  } else {
-    const int i16 = lane & 15;
-    const int col = row_base + (MI == 32 ? 16 * ((lane >> 4) & 1) : 0) + 4 * (i16 & 3);
-    const int kb = C::KI * q + 8 * kgrp + (i16 >> 2);
-    s16x4_t lo, hi;
-    {
-      const int k = kb;
-      const int slot = ((col >> 3) + ks_rot<MI>(k)) & (KS_CHUNKS - 1);
-      lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (s16x4_t __attribute__((address_space(3)))*)(tile + k * KS_ROW_BYTES + slot * 16 + (col & 7) * 2));
-    }
-    {
-      const int k = kb + 4;
-      const int slot = ((col >> 3) + ks_rot<MI>(k)) & (KS_CHUNKS - 1);
-      hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (s16x4_t __attribute__((address_space(3)))*)(tile + k * KS_ROW_BYTES + slot * 16 + (col & 7) * 2));
-    }
-    typedef short s16x8_t __attribute__((ext_vector_type(8)));
-    s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(bf16x8_t, both);
-  }
+  const int row = row_base + (lane & 15);
+  const int c = kc_slot<C::BK>(row, (C::KI / 8) * q + (lane >> 4));
+  return *reinterpret_cast<const bf16x8_t*>(tile + row * (C::BK * 2) + c * 16);
 }
 
-// K-strided fragment of the 16 x 16 x 32 shape from two per-lane constants (see ks16_consts): the LDS address of
-// every transpose read is ((S + c) & rowmask | R) + constant, i.e. two VALU operations next to the read instead
+// K-strided tiles are read with the LDS transpose read: its 16 lanes fetch 4 k-rows x 16 rows (8 bytes per lane: 4
+// consecutive rows at one k) and every lane receives the 4 k-values of its own row.  The fragment is formed from two
+// per-lane constants (see ks16_consts): the LDS address of every transpose read is ((S + c) & rowmask | R) + constant, i.e. two VALU operations next to the read instead
 // of one address register per (fragment, k-half, k-step, ring slot) kept alive across the whole K loop.
 template <int ROWS>
 __device__ __forceinline__ void ks16_consts(int lane, int wave_row_base, uint32_t& S, uint32_t& R) {
@@ -302,39 +224,34 @@ __device__ __forceinline__ void mfma_drain() { asm volatile("s_nop 7\n\ts_nop 7\
 // own L2, so id % 8 names the XCD and id / 8 the position in that XCD's queue.  Each XCD gets a contiguous
 // range of tile columns (all tile rows), walked in blocks of XCD_BLOCK_M tile rows: the ~32 tiles an XCD
 // works on at one time then form a compact block that shares P row-panels and Q column-panels in L2.
-#ifndef MI_XCD_BLOCK_M
-#define MI_XCD_BLOCK_M 8
-#endif
+constexpr int XCD_BLOCK_M = 8;
 __device__ __forceinline__ void gemm_tile_of(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
   constexpr int XCDS = 8;
-  const int total = tiles_m * tiles_n;
-  if (MI_XCD_BLOCK_M == 0 || tiles_n % XCDS != 0 || tiles_m % MI_XCD_BLOCK_M != 0) {
+  if (tiles_n % XCDS != 0 || tiles_m % XCD_BLOCK_M != 0) {
     tm = pid % tiles_m;
     tn = pid / tiles_m;
     return;
   }
-  (void)total;
   const int xcd = pid % XCDS, local = pid / XCDS;
   const int cols_per_xcd = tiles_n / XCDS;
-  const int block = MI_XCD_BLOCK_M * cols_per_xcd;  // tiles in one row-block of this XCD's column range
+  const int block = XCD_BLOCK_M * cols_per_xcd;  // tiles in one row-block of this XCD's column range
   const int rb = local / block, r = local % block;
-  tm = rb * MI_XCD_BLOCK_M + r % MI_XCD_BLOCK_M;
-  tn = xcd * cols_per_xcd + r / MI_XCD_BLOCK_M;
+  tm = rb * XCD_BLOCK_M + r % XCD_BLOCK_M;
+  tn = xcd * cols_per_xcd + r / XCD_BLOCK_M;
 }
 
 // GEMM-mode epilogue through LDS.  In the MFMA accumulator layout a lane owns one output row and scattered
 // 4-column groups, so direct global accesses touch 32 rows per instruction.  Here every wavefront parks one
 // 32-row block of its accumulators in its own LDS region (float32, rows padded by 16 bytes against bank
 // conflicts), then re-reads it so that 8 consecutive lanes cover 64 consecutive columns of one row: the
-// Cin loads and the stores become 16-byte-per-lane, 128-byte-per-row accesses.  (MI = rows of one MFMA tile,
-// G = 4-column groups a lane holds per MFMA tile: 4 for the 32 x 32 shape, 1 for 16 x 16.)  No workgroup barrier is
-// needed between the passes: a wavefront only touches its own region and LDS operations of one wavefront
+// Cin loads and the stores become 16-byte-per-lane, 128-byte-per-row accesses.  (MI = rows of one MFMA tile.)
+// No workgroup barrier is needed between the passes: a wavefront only touches its own region and LDS operations of one wavefront
 // complete in order.
 template <class C, bool OUT_F32, bool GUARD>
-__device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, typename AccVec<C::MI>::type (&acc)[C::FM][C::FN], char* lds, int wave,
+__device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x4_t (&acc)[C::FM][C::FN], char* lds, int wave,
                                                   int lane, int m_base, int n_base, int64_t batch, float alpha,
                                                   float beta, float* red) {
-  constexpr int TN = C::TN, ROWB = TN * 4 + 16, MI = C::MI, G = MI == 32 ? 4 : 1;
+  constexpr int TN = C::TN, ROWB = TN * 4 + 16, MI = C::MI;
   constexpr int LPR = TN / 8;    // lanes per output row (8 columns each)
   constexpr int RPI = 64 / LPR;  // rows per read iteration
   static_assert(MI % RPI == 0 && 64 % LPR == 0, "wave tile width must be 32, 64 or 128");
@@ -371,10 +288,9 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, typename 
     char* reg = lds + (wave * NREG + i % NREG) * (MI * ROWB);
 #pragma unroll
     for (int j = 0; j < C::FN; ++j)
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        f32x4_t v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-        *reinterpret_cast<f32x4_t*>(reg + frow * ROWB + (j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk) * 4) = v;
+{
+        const f32x4_t v = acc[i][j];
+        *reinterpret_cast<f32x4_t*>(reg + frow * ROWB + (j * MI + 4 * fk) * 4) = v;
       }
 #pragma unroll
     for (int t = 0; t < NIT; ++t) {
@@ -448,43 +364,42 @@ struct SyrkStage {
   static constexpr int NCH = RP * CPRW / C::NT;    // chunks per thread and pass
   // a one-pass tile fetches its Cin values into registers before the K loop, in accumulator layout
   // (one 8-byte quad per accumulator quad: NQUAD x 2 registers per lane)
-  static constexpr int NQUAD = C::FM * C::FN * (C::MI == 32 ? 4 : 1);
+  static constexpr int NQUAD = C::FM * C::FN;
   static constexpr bool CIN_EARLY = NPASS == 1 && NQUAD * 2 <= 80;
 };
-// This lane's addend values of a one-pass tile, in accumulator layout: quad (i, j, g) covers row
-// m0 + mw + i MI + (lane % MI), columns n0 + nw + j MI + 8 g + 4 (lane / MI) .. + 3 (g only for MI = 32).  One load
+// This lane's addend values of a one-pass tile, in accumulator layout: quad (i, j) covers row
+// m0 + mw + 16 i + (lane % 16), columns n0 + nw + 16 j + 4 (lane / 16) .. + 3.  One load
 // instruction touches MI rows with 32 contiguous bytes each -- whole 32-byte sectors, so nothing is fetched twice.
 // Issued before the K loop (first addend) or at the start of the epilogue (second), so that the burst of all
 // workgroups does not sit on the critical path.
 template <class C, bool GUARD>
 __device__ __forceinline__ void syrk_addend_fetch(const GemmParams& p, const uint16_t* __restrict__ Cb, int lane, int m_base,
                                                   int n_base, uint2 (&pre)[SyrkStage<C>::NQUAD]) {
-  constexpr int MI = C::MI, G = MI == 32 ? 4 : 1;
+  constexpr int MI = C::MI;
   const int frow = lane & (MI - 1), fk = lane / MI;
 #pragma unroll
   for (int i = 0; i < C::FM; ++i)
 #pragma unroll
     for (int j = 0; j < C::FN; ++j)
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        const int m = m_base + i * MI + frow, n = n_base + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
+{
+        const int m = m_base + i * MI + frow, n = n_base + j * MI + 4 * fk;
         uint2 v = make_uint2(0u, 0u);
         if (!GUARD || (m < p.M && n < p.N)) v = *reinterpret_cast<const uint2*>(Cb + (int64_t)m * p.ldc + n);
-        pre[(i * C::FN + j) * G + g] = v;
+        pre[i * C::FN + j] = v;
       }
 }
 
 template <class C, bool GUARD>
-__device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename AccVec<C::MI>::type (&acc)[C::FM][C::FN],
+__device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, f32x4_t (&acc)[C::FM][C::FN],
                                                   char* lds, int lane, int wm, int wn, int m0, int n0, int64_t batch,
                                                   bool diag, float alpha, float beta, float beta2, float shift,
                                                   const uint2 (&cin_pre)[SyrkStage<C>::CIN_EARLY ? SyrkStage<C>::NQUAD : 1]) {
   using S = SyrkStage<C>;
-  constexpr int LDT = S::LDT, MI = C::MI, G = MI == 32 ? 4 : 1, FM = C::FM, FN = C::FN;
+  constexpr int LDT = S::LDT, MI = C::MI, FM = C::FM, FN = C::FN;
   constexpr int RP = S::RP, NPASS = S::NPASS, CPRW = S::CPRW, NCH = S::NCH;
   static_assert(RP * LDT * 2 <= S::RING, "staging pass exceeds the ring");
   static_assert(RP % C::TM == 0 && RP % C::TN == 0, "a wavefront's block must fall into one pass");
-  static_assert(C::KSPLIT == 1 && C::TILE_M == C::TILE_N, "square tiles, one K group");
+  static_assert(C::TILE_M == C::TILE_N, "square tiles");
   static_assert(C::WGM == 2 && C::WGN == 2 && C::TM == C::TN, "2 x 2 wavefronts with square blocks: the diagonal blocks are (0,0) and (1,1)");
   static_assert(RP * CPRW % C::NT == 0, "write-out must divide evenly");
   const int tid = threadIdx.x;
@@ -499,7 +414,7 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
 
   // Finished bf16 quads of this lane.  A one-pass tile keeps them in registers; a tile staged in passes (a 256 x 256
   // tile: 128 quads on top of 256 accumulators) finishes each quad on its way to LDS.
-  uint2 val[NPASS == 1 ? FM : 1][NPASS == 1 ? FN : 1][NPASS == 1 ? G : 1];
+  uint2 val[NPASS == 1 ? FM : 1][NPASS == 1 ? FN : 1];
   // ---- values: alpha * acc (+ beta * Cin) (+ beta2 * Cin2) (- shift on the diagonal), rounded to bf16 ----
   if constexpr (NPASS == 1) {
     // Both addends arrive in accumulator layout: the first was requested before the K loop, the second is
@@ -521,13 +436,12 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
     for (int i = 0; i < FM; ++i)
 #pragma unroll
       for (int j = 0; j < FN; ++j)
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-          const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
-          const int q = (i * FN + j) * G + g;
+{
+          const int ml = mw + i * MI + frow, nl = nw + j * MI + 4 * fk;
+          const int q = i * FN + j;
           f32x4_t v;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][4 * g + r];
+          for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][r];
           if (use_c) {
             if constexpr (S::CIN_EARLY)
               add(v, cin_pre[q], beta);
@@ -540,16 +454,16 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
             for (int r = 0; r < 4; ++r)
               if (nl + r == ml) v[r] -= shift;
           }
-          val[i][j][g] = __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));
+          val[i][j] = __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));
         }
   }
-  // finished bf16 quad (i, j, g) of this lane; a tile staged in passes reads its addends here, in accumulator layout
+  // finished bf16 quad (i, j) of this lane; a tile staged in passes reads its addends here, in accumulator layout
   // (fetching them a fragment row ahead into registers was tried: it spills and is slower)
-  auto quad = [&](int i, int j, int g) -> uint2 {
+  auto quad = [&](int i, int j) -> uint2 {
     if constexpr (NPASS == 1) {
-      return val[i][j][g];
+      return val[i][j];
     } else {
-      const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
+      const int ml = mw + i * MI + frow, nl = nw + j * MI + 4 * fk;
       auto add = [&](f32x4_t& v, const uint2& raw, float coef) {
         v[0] = __builtin_fmaf(coef, __uint_as_float(raw.x << 16), v[0]);
         v[1] = __builtin_fmaf(coef, __uint_as_float(raw.x & 0xffff0000u), v[1]);
@@ -558,7 +472,7 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
       };
       f32x4_t v;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][4 * g + r];
+      for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][r];
       if (!GUARD || (m0 + ml < p.M && n0 + nl < p.N)) {
         if (use_c) add(v, *reinterpret_cast<const uint2*>(Cb + (int64_t)(m0 + ml) * p.ldc + n0 + nl), beta);
         if (use_c2) add(v, *reinterpret_cast<const uint2*>(Cb2 + (int64_t)(m0 + ml) * p.ldc + n0 + nl), beta2);
@@ -610,10 +524,9 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
         for (int i = 0; i < FM; ++i) {
 #pragma unroll
           for (int j = 0; j < FN; ++j)
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-              const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
-              *reinterpret_cast<uint2*>(lds + ((ml - h * RP) * LDT + nl) * 2) = quad(i, j, g);
+{
+              const int ml = mw + i * MI + frow, nl = nw + j * MI + 4 * fk;
+              *reinterpret_cast<uint2*>(lds + ((ml - h * RP) * LDT + nl) * 2) = quad(i, j);
             }
         }
       } else if (wm == wn) {
@@ -623,13 +536,12 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
         for (int i = 0; i < FM; ++i) {
 #pragma unroll
           for (int j = 0; j <= i; ++j)
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-              const int ml = mw + i * MI + frow, nl = nw + j * MI + (MI == 32 ? 8 * g : 0) + 4 * fk;
+{
+              const int ml = mw + i * MI + frow, nl = nw + j * MI + 4 * fk;
               if (j < i || nl < (ml & ~3)) {
-                *reinterpret_cast<uint2*>(lds + ((ml - h * RP) * LDT + nl) * 2) = quad(i, j, g);
+                *reinterpret_cast<uint2*>(lds + ((ml - h * RP) * LDT + nl) * 2) = quad(i, j);
               } else if (nl == (ml & ~3)) {
-                const uint2 q4 = quad(i, j, g);
+                const uint2 q4 = quad(i, j);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                   const uint16_t e = elem(q4, r);
@@ -664,8 +576,9 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, typename 
       const int c = tid + it * C::NT, row = c / CPRW, c8 = c % CPRW;
       const int gr = m0 + h * RP + row, gc = n0 + c8 * 8;
       const uint4 v = *reinterpret_cast<const uint4*>(lds + (row * LDT + c8 * 8) * 2);
-      // a diagonal tile holds nothing right of the diagonal block of a row: that part comes from the mirror image
-      const bool held = !sym || c8 * 8 < ((h * RP + row) / C::TM + 1) * C::TM;
+      // a diagonal tile holds nothing right of the diagonal block of a row (the wavefront that owns that block sits
+      // the product out): that part comes from the mirror image, or stays unwritten when the upper triangle is skipped
+      const bool held = !diag || c8 * 8 < ((h * RP + row) / C::TM + 1) * C::TM;
       if (held && (!GUARD || (gr < p.M && gc < p.N))) *reinterpret_cast<uint4*>(ob + (int64_t)gr * p.ldo + gc) = v;
     }
     // ---- the mirror image, straight from the staged rows ----
@@ -696,8 +609,7 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: everything derived from it stays in SGPRs
-  const int kgroup = wave / C::NWG, wig = wave % C::NWG;  // K group and position inside it
-  const int wm = wig % C::WGM, wn = wig / C::WGM;
+  const int wm = wave % C::WGM, wn = wave / C::WGM;
   const int64_t batch = blockIdx.y;
   int tm, tn;
   if (MODE == MODE_SYRK) {
@@ -724,8 +636,8 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   lp.init(p.P + p_off, p.ldp, m0, p.M, wave, lane);
   lq.init(p.Q + q_off, p.ldq, n0, p.N, wave, lane);
 
-  constexpr int MI = C::MI, ACC_N = MI == 32 ? 16 : 4;
-  typename AccVec<MI>::type acc[FM][FN];
+  constexpr int MI = C::MI, ACC_N = 4;
+  f32x4_t acc[FM][FN];
 #pragma unroll
   for (int i = 0; i < FM; ++i)
 #pragma unroll
@@ -734,7 +646,7 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
       for (int e = 0; e < ACC_N; ++e) acc[i][j][e] = 0.0f;
 
   const int nk = p.K / C::BK;
-  constexpr int NQ = C::BK / C::KI / C::KSPLIT;  // k-steps of one tile that this wavefront multiplies
+  constexpr int NQ = C::BK / C::KI;  // k-steps of one tile
   constexpr int LOADS_PER_TILE = C::LPT_P + C::LPT_Q;  // per thread, both operands
   static_assert(NQ % 2 == 0, "fragment buffer parity assumes an even number of k-steps per tile");
   static_assert((NS - 1) * LOADS_PER_TILE < 64, "vmcnt is a 6-bit counter");
@@ -752,33 +664,27 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   // tile before its barrier): the CU's single address unit then sees an even stream instead of a burst from
   // all wavefronts at once, and the tile still has NS-2 whole tile times to land.  With two slots there is no
   // slack for that and the whole tile goes out in the k-step after the barrier.
-#ifdef MI_TIMING
-  long long t_load = 0, t_bar = 0;
-#endif
   constexpr int UNITS = FM + FN, MMAS = FM * FN;  // fragment reads / MFMAs per k-step
   constexpr int UPS = (UNITS + MMAS - 1) / MMAS;  // fragment reads per slot
   constexpr int PARTS = (NS >= 3 && LOADS_PER_TILE % NQ == 0) ? NQ : 1;
   constexpr int PL = LOADS_PER_TILE / PARTS;      // loads per part
   constexpr int DPS = (PL + MMAS - 1) / MMAS;     // loads per slot (1 unless a part outnumbers the MFMAs)
   bf16x8_t fp[2][FM], fq[2][FN];
-  uint32_t ks_sp = 0, ks_rp = 0, ks_sq = 0, ks_rq = 0;  // 16 x 16 shape: lane constants of the K-strided reads
-  if constexpr (MI == 16 && P_KS) ks16_consts<C::TILE_M>(lane, wm * C::TM, ks_sp, ks_rp);
-  if constexpr (MI == 16 && Q_KS) ks16_consts<C::TILE_N>(lane, wn * C::TN, ks_sq, ks_rq);
+  uint32_t ks_sp = 0, ks_rp = 0, ks_sq = 0, ks_rq = 0;  // lane constants of the K-strided reads
+  if constexpr (P_KS) ks16_consts<C::TILE_M>(lane, wm * C::TM, ks_sp, ks_rp);
+  if constexpr (Q_KS) ks16_consts<C::TILE_N>(lane, wn * C::TN, ks_sq, ks_rq);
   auto lds_of = [&](const char* ptr) { return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)ptr; };
   auto read_unit = [&](const char* st, int q, int buf, int r) {
-#ifdef MI_ABLATE_READS
-    if (q >= 0) return;  // debug build: fragments keep their start-up contents
-#endif
     if (r < FM) {
-      if constexpr (MI == 16 && P_KS)
-        fp[buf][r] = fast_frag16_ks<C::TILE_M>(lds_of(st), ks_sp, ks_rp, r, q * C::KSPLIT + kgroup);
+      if constexpr (P_KS)
+        fp[buf][r] = fast_frag16_ks<C::TILE_M>(lds_of(st), ks_sp, ks_rp, r, q);
       else
-        fp[buf][r] = fast_frag<C, P_KS, C::TILE_M>(st, wm * C::TM + r * MI, q * C::KSPLIT + kgroup, lane);
+        fp[buf][r] = fast_frag<C>(st, wm * C::TM + r * MI, q, lane);
     } else {
-      if constexpr (MI == 16 && Q_KS)
-        fq[buf][r - FM] = fast_frag16_ks<C::TILE_N>(lds_of(st + P_BYTES), ks_sq, ks_rq, r - FM, q * C::KSPLIT + kgroup);
+      if constexpr (Q_KS)
+        fq[buf][r - FM] = fast_frag16_ks<C::TILE_N>(lds_of(st + P_BYTES), ks_sq, ks_rq, r - FM, q);
       else
-        fq[buf][r - FM] = fast_frag<C, Q_KS, C::TILE_N>(st + P_BYTES, wn * C::TN + (r - FM) * MI, q * C::KSPLIT + kgroup, lane);
+        fq[buf][r - FM] = fast_frag<C>(st + P_BYTES, wn * C::TN + (r - FM) * MI, q, lane);
     }
   };
   auto fetch = [&](const char* st, int q, int buf) {
@@ -806,22 +712,16 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   auto k_step = [&](auto read_flag, auto part, int buf, const char* rd_tile, int rd_q, int ld_slot) {
     constexpr bool READ = decltype(read_flag)::value;
     constexpr int PART = decltype(part)::value;
-    if constexpr (MI == 16 && (P_KS || Q_KS)) {
+    if constexpr (P_KS || Q_KS) {
       // keep the address arithmetic of the transpose reads next to them (it would otherwise be hoisted out of
       // the K loop, one register per read)
       asm volatile("" : "+v"(ks_sp), "+v"(ks_rp), "+v"(ks_sq), "+v"(ks_rq));
     }
-#ifdef MI_SETPRIO
-    __builtin_amdgcn_s_setprio(MI_SETPRIO);
-#endif
     static_for<MMAS>([&](auto xc) {
       // P fragment i stays for FN MFMAs in a row; the Q fragments are walked forth and back, so that one of the
       // two operands is always the same as in the previous MFMA (measurably less power than changing both)
       constexpr int x = decltype(xc)::value, i = x / FN, j = (i & 1) ? FN - 1 - x % FN : x % FN;
-      if constexpr (MI == 32)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fq[buf][j], fp[buf][i], acc[i][j], 0, 0, 0);
-      else
-        mfma16_inplace(acc[i][j], fq[buf][j], fp[buf][i]);
+      mfma16_inplace(acc[i][j], fq[buf][j], fp[buf][i]);
       if constexpr (READ) {
         static_for<UPS>([&](auto uc) {
           constexpr int u = decltype(uc)::value;
@@ -836,17 +736,12 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
           if constexpr ((PL <= MMAS ? e * MMAS / PL : e / DPS) == x) issue_one(ld_slot, PART * PL + e);
         });
       }
-#ifndef MI_NO_SCHED_INTERLEAVE
       __builtin_amdgcn_sched_barrier(0);
-#endif
     });
     if (PART == PARTS - 1) {
       lp.advance();
       lq.advance();
     }
-#ifdef MI_SETPRIO
-    __builtin_amdgcn_s_setprio(0);
-#endif
   };
   // `steady` (a compile-time flag) marks tiles in the middle of the K loop: tile kt+NS exists (so the vacated
   // slot is refilled and NS-2 younger tiles stay in flight at the wait), and the tile body is branch free.
@@ -864,23 +759,9 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
         k_step(std::true_type{}, std::integral_constant<int, -1>{}, q & 1, cur, q + 1, 0);
       }
     }
-#ifdef MI_TIMING
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
-    const long long tw0 = __builtin_readcyclecounter();
-#endif
     // own loads of tile kt+1 have landed; own reads of `cur` are done
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(STEADY ? (NS - 2) * LOADS_PER_TILE : 0, 0));
-#ifdef MI_TIMING
-    const long long tw1 = __builtin_readcyclecounter();
-#endif
-#ifndef MI_ABLATE_BARRIER
     __syncthreads();
-#endif
-#ifdef MI_TIMING
-    const long long tw2 = __builtin_readcyclecounter();
-    t_load += tw1 - tw0;
-    t_bar += tw2 - tw1;
-#endif
     if (STEADY) {
       k_step(std::true_type{}, std::integral_constant<int, 0>{}, (NQ - 1) & 1, nxt, 0, cur_slot);
     } else {
@@ -891,9 +772,6 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   };
   static_assert(NQ <= 4, "k_tile spells out at most three k-steps before the barrier");
 
-#ifdef MI_TIMING
-  const long long t_start = __builtin_readcyclecounter();
-#endif
   // prologue: tiles 0 .. NS-2 and part 0 of tile NS-1 in flight, wait for tile 0
 #pragma unroll
   for (int t = 0; t < NS - 1; ++t)
@@ -904,14 +782,7 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   else
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
   __syncthreads();
-#ifdef MI_ABLATE_READS
-#pragma unroll
-  for (int r = 0; r < UNITS; ++r) {
-    if (r < FM) fp[0][r] = fp[1][r] = fast_frag<C, P_KS, C::TILE_M>(ring[0], wm * C::TM + r * MI, kgroup, lane);
-    else fq[0][r - FM] = fq[1][r - FM] = fast_frag<C, Q_KS, C::TILE_N>(ring[0] + P_BYTES, wn * C::TN + (r - FM) * MI, kgroup, lane);
-  }
-#endif
-  constexpr bool SYRK_STAGED = MODE == MODE_SYRK && !OUT_F32 && C::KSPLIT == 1 && C::NW == 4;
+  constexpr bool SYRK_STAGED = MODE == MODE_SYRK && !OUT_F32 && C::NW == 4;
   constexpr bool CIN_EARLY = SYRK_STAGED && SyrkStage<C>::CIN_EARLY;
   uint2 cin_pre[CIN_EARLY ? SyrkStage<C>::NQUAD : 1];
   if constexpr (CIN_EARLY) {
@@ -931,9 +802,7 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
       const int cur_slot = kt % NS, prev_slot = (cur_slot + NS - 1) % NS;
       if (PARTS > 1 && kt + NS - 1 < nk) issue_parts(prev_slot, 1, PARTS);
       __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
-#ifndef MI_ABLATE_BARRIER
       __syncthreads();
-#endif
       if (kt + NS < nk) issue_parts(cur_slot, 0, 1);
     }
   } else {
@@ -950,41 +819,7 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
     }
   }
 
-  if constexpr (MI == 16) mfma_drain();
-  if constexpr (C::KSPLIT == 2) {
-    // Sum the two K groups: group 1 parks its accumulators in the ring (lane-linear, conflict free),
-    // group 0 adds them and carries on with the epilogue alone.
-    static_assert(C::KSPLIT == 1 || C::NWG * FM * FN * ACC_N * 256 <= NS * C::SLOT_BYTES, "accumulators exceed the ring");
-    __syncthreads();  // all fragment reads of the ring are done
-    char* park = &ring[0][0] + wig * (FM * FN * ACC_N * 256);
-    if (kgroup == 1) {
-#pragma unroll
-      for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-          for (int g = 0; g < ACC_N / 4; ++g) {
-            f32x4_t v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-            *reinterpret_cast<f32x4_t*>(park + ((i * FN + j) * (ACC_N / 4) + g) * 1024 + lane * 16) = v;
-          }
-    }
-    __syncthreads();
-    if (kgroup == 0) {
-#pragma unroll
-      for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-          for (int g = 0; g < ACC_N / 4; ++g) {
-            const f32x4_t v = *reinterpret_cast<const f32x4_t*>(park + ((i * FN + j) * (ACC_N / 4) + g) * 1024 + lane * 16);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) acc[i][j][4 * g + r] += v[r];
-          }
-    }
-  }
-#ifdef MI_TIMING
-  const long long t_loop = __builtin_readcyclecounter();
-#endif
+  mfma_drain();
   const Scalars sc = resolve_shift<NT>(p, batch, red);
   const float alpha = sc.alpha, beta = sc.beta, beta2 = sc.beta2, shift = sc.shift;
   const bool diag = (MODE == MODE_SYRK) && (tm == tn);
@@ -995,23 +830,9 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   } else if constexpr (SYRK_STAGED) {
     syrk_epilogue_lds<C, EDGE>(p, acc, &ring[0][0], lane, wm, wn, m0, n0, batch, diag, alpha, beta, beta2, shift, cin_pre);
   } else {
-    static_assert(C::KSPLIT == 1 || MODE == MODE_SYRK, "the K-group variant is wired for SYRK only");
-    // (SYRK never takes the per-workgroup sum at the end of tile_epilogue, so group 1 may simply skip it)
-    if (C::KSPLIT == 1 || kgroup == 0)
-      tile_epilogue<MODE, OUT_F32, EDGE, FM, FN, NT, MI>(p, acc, m0 + wm * C::TM, n0 + wn * C::TN, lane, batch, diag, alpha,
-                                                     beta, shift, red, beta2);
+    tile_epilogue<MODE, OUT_F32, EDGE, FM, FN, NT, MI>(p, acc, m0 + wm * C::TM, n0 + wn * C::TN, lane, batch, diag, alpha, beta, shift,
+                                                       red, beta2);
   }
-#ifdef MI_TIMING
-  if (p.slots_in && lane == 0) {  // debug build only: slots_in doubles as the timing dump
-    __builtin_amdgcn_s_waitcnt(0);
-    const long long t_end = __builtin_readcyclecounter();
-    long long* dump = (long long*)p.slots_in + ((long long)blockIdx.x * C::NW + wave) * 4;
-    dump[0] = t_load;
-    dump[1] = t_bar;
-    dump[2] = t_loop - t_start;
-    dump[3] = t_end - t_loop;
-  }
-#endif
 }
 
 }  // namespace mi

@@ -1,0 +1,31 @@
+// Host-side launchers of the tile engine.  The kernels are compiled in several translation units (one per kernel
+// family, so that they build in parallel); each defines the launchers of its family by explicit instantiation of the
+// templates in launch_impl.hpp, and the rest of the library only sees the declarations below.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "gemm_fast.hpp"
+
+namespace mi {
+
+// Records the text behind mi_last_error() for this host thread and returns `code`.
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+// What the last launch_one / launch_fast call on this thread launched: workgroups per batch entry and the tile shape.
+struct LastLaunch {
+  int tiles, tile_m, tile_n, fast;
+};
+extern thread_local LastLaunch g_last_launch;
+
+// General kernel (gemm_engine.hpp): any multiple-of-8 shape, K tails, both operand layouts.
+template <int BM, int BN, int BK, int WGM, int WGN, bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
+int launch_one(const GemmParams& p, int64_t batch, hipStream_t stream);
+
+// Fast kernel (gemm_fast.hpp): K a multiple of the ring-slot depth; tiles that overhang the matrix only for the
+// lower-triangle product of K-contiguous operands; anything else is refused with MI_ERR_UNSUPPORTED_SHAPE before
+// a kernel is launched.
+template <class C, bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
+int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream);
+
+}  // namespace mi

@@ -1,0 +1,76 @@
+// Definitions of the launchers declared in launch.hpp; included by the translation units that instantiate kernels.
+#pragma once
+#include "../../include/mi_ns.h"
+#include "launch.hpp"
+
+namespace mi {
+
+// Per-workgroup partial sums go to slots_out[batch * slot_stride + slot_base + workgroup]: refuse a launch whose
+// workgroups would write past the capacity the caller reserved (checked before anything is launched).
+static inline int check_slots(const GemmParams& q, int64_t tiles) {
+  if (q.slots_out != nullptr && q.slot_capacity > 0 && (q.slot_base + tiles > q.slot_capacity || q.slot_stride > q.slot_capacity))
+    return fail(MI_ERR_WORKSPACE, "internal: %lld partial-sum slots exceed the %d reserved", (long long)(q.slot_base + tiles),
+                q.slot_capacity);
+  return MI_OK;
+}
+
+template <int BM, int BN, int BK, int WGM, int WGN, bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
+int launch_one(const GemmParams& p, int64_t batch, hipStream_t stream) {
+  auto kern = gemm_bf16_kernel<BM, BN, BK, WGM, WGN, P_KS, Q_KS, MODE, OUT_F32>;
+  constexpr int LDS_BYTES = 2 * (BM + BN) * BK * 2;
+  static bool attr_set = false;  // benign race: setting the attribute twice is harmless
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "hipFuncSetAttribute(%d B LDS): %s", LDS_BYTES, hipGetErrorString(e));
+    attr_set = true;
+  }
+  GemmParams q = p;
+  q.tiles_m = (p.M + BM - 1) / BM;
+  q.tiles_n = (p.N + BN - 1) / BN;
+  const int64_t tiles = (MODE == MODE_SYRK) ? (int64_t)q.tiles_m * (q.tiles_m + 1) / 2 : (int64_t)q.tiles_m * q.tiles_n;
+  if (tiles <= 0 || batch <= 0) return MI_OK;
+  if (batch > 65535) return fail(MI_ERR_UNSUPPORTED_SHAPE, "batch %lld exceeds the grid limit 65535", (long long)batch);
+  if (q.slot_stride == 0) q.slot_stride = (int)tiles;
+  if (int rc = check_slots(q, tiles)) return rc;
+  g_last_launch = LastLaunch{(int)tiles, BM, BN, 0};
+  dim3 grid((unsigned)tiles, (unsigned)batch, 1), block(WGM * WGN * 64, 1, 1);
+  hipLaunchKernelGGL(kern, grid, block, LDS_BYTES, stream, q);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+  return MI_OK;
+}
+
+template <class C, bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
+int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream) {
+  // the K loop of the fast kernel has no tail, and its loaders trust these extents
+  if (p.K < C::BK || p.K % C::BK != 0)
+    return fail(MI_ERR_UNSUPPORTED_SHAPE, "internal: K = %d is not a multiple of %d", p.K, C::BK);
+  if (p.M <= 0 || p.N <= 0 || batch <= 0) return MI_OK;
+  GemmParams q = p;
+  q.tiles_m = (p.M + C::TILE_M - 1) / C::TILE_M;
+  q.tiles_n = (p.N + C::TILE_N - 1) / C::TILE_N;
+  int64_t tiles = (MODE == MODE_SYRK) ? (int64_t)q.tiles_m * (q.tiles_m + 1) / 2 : (int64_t)q.tiles_m * q.tiles_n;
+  if (MODE == MODE_SYRK) tiles = (tiles + 7) / 8 * 8;  // XCD-chunked enumeration: grid padded to a multiple of 8
+  if (batch > 65535) return fail(MI_ERR_UNSUPPORTED_SHAPE, "batch %lld exceeds the grid limit 65535", (long long)batch);
+  if (q.slot_stride == 0) q.slot_stride = (int)tiles;
+  if (int rc = check_slots(q, tiles)) return rc;
+  dim3 grid((unsigned)tiles, (unsigned)batch, 1), block(C::NT, 1, 1);
+  const bool edge = (p.M % C::TILE_M) != 0 || (p.N % C::TILE_N) != 0;
+  // Only the lower-triangle product of K-contiguous operands has a variant for tiles that overhang the matrix
+  // (rows clamped in the loaders, guarded epilogue).
+  constexpr bool HAS_EDGE_VARIANT = MODE == MODE_SYRK && !P_KS && !Q_KS;
+  if (edge) {
+    if constexpr (HAS_EDGE_VARIANT)
+      hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, true>), grid, block, 0, stream, q);
+    else
+      return fail(MI_ERR_UNSUPPORTED_SHAPE, "internal: %d x %d is not a whole number of %d x %d tiles", p.M, p.N, C::TILE_M, C::TILE_N);
+  } else {
+    hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, false>), grid, block, 0, stream, q);
+  }
+  g_last_launch = LastLaunch{(int)tiles, C::TILE_M, C::TILE_N, 1};
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+  return MI_OK;
+}
+
+}  // namespace mi

@@ -11,14 +11,14 @@
 #include <string>
 #include <vector>
 
-#include "gemm_engine.hpp"
-#include "gemm_fast.hpp"
+#include "launch.hpp"
 
 namespace mi {
 
 static thread_local std::string g_last_error;
+thread_local LastLaunch g_last_launch = {0, 0, 0, 0};
 
-static int fail(int code, const char* fmt, ...) {
+int fail(int code, const char* fmt, ...) {
   char buf[512];
   va_list ap;
   va_start(ap, fmt);
@@ -74,56 +74,6 @@ static TileClass pick_class(int64_t extent) {
   return TILE_SMALL;
 }
 
-// Number of workgroups (per batch entry) the last launch_class call on this thread used.
-static thread_local int g_last_tiles = 0;
-
-template <int BM, int BN, int BK, int WGM, int WGN, bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
-static int launch_one(const GemmParams& p, int64_t batch, hipStream_t stream) {
-  auto kern = gemm_bf16_kernel<BM, BN, BK, WGM, WGN, P_KS, Q_KS, MODE, OUT_F32>;
-  constexpr int LDS_BYTES = 2 * (BM + BN) * BK * 2;
-  static bool attr_set = false;  // benign race: setting the attribute twice is harmless
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-    if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "hipFuncSetAttribute(%d B LDS): %s", LDS_BYTES, hipGetErrorString(e));
-    attr_set = true;
-  }
-  GemmParams q = p;
-  q.tiles_m = (p.M + BM - 1) / BM;
-  q.tiles_n = (p.N + BN - 1) / BN;
-  int64_t tiles = (MODE == MODE_SYRK) ? (int64_t)q.tiles_m * (q.tiles_m + 1) / 2 : (int64_t)q.tiles_m * q.tiles_n;
-  if (tiles <= 0 || batch <= 0) return MI_OK;
-  if (batch > 65535) return fail(MI_ERR_UNSUPPORTED_SHAPE, "batch %lld exceeds the grid limit 65535", (long long)batch);
-  g_last_tiles = (int)tiles;
-  if (q.slot_stride == 0) q.slot_stride = (int)tiles;
-  dim3 grid((unsigned)tiles, (unsigned)batch, 1), block(WGM * WGN * 64, 1, 1);
-  hipLaunchKernelGGL(kern, grid, block, LDS_BYTES, stream, q);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
-  return MI_OK;
-}
-
-template <class C, bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
-static int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream) {
-  GemmParams q = p;
-  q.tiles_m = (p.M + C::TILE_M - 1) / C::TILE_M;
-  q.tiles_n = (p.N + C::TILE_N - 1) / C::TILE_N;
-  int64_t tiles = (MODE == MODE_SYRK) ? (int64_t)q.tiles_m * (q.tiles_m + 1) / 2 : (int64_t)q.tiles_m * q.tiles_n;
-  if (MODE == MODE_SYRK) tiles = (tiles + 7) / 8 * 8;  // XCD-chunked enumeration: grid padded to a multiple of 8
-  if (batch > 65535) return fail(MI_ERR_UNSUPPORTED_SHAPE, "batch %lld exceeds the grid limit 65535", (long long)batch);
-  g_last_tiles = (int)tiles;
-  if (q.slot_stride == 0) q.slot_stride = (int)tiles;
-  dim3 grid((unsigned)tiles, (unsigned)batch, 1), block(C::NT, 1, 1);
-  const bool edge = (p.M % C::TILE_M) != 0 || (p.N % C::TILE_N) != 0;
-  if (edge)
-    hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, true>), grid, block, 0, stream, q);
-  else
-    hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, false>), grid, block, 0, stream, q);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
-  return MI_OK;
-}
-
 static int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Device-wide compute units (workgroups that run concurrently at one fast-kernel workgroup per CU).
@@ -155,23 +105,18 @@ static int num_cus() {
 //                                                 clock rises), needs n % 128 == 0
 // Short K or few tiles favour the small tiles (their epilogue is short and, two to a CU, hidden), long K the
 // 192 x 192 tile, and row counts that 192 divides badly (1792 = 7 x 256) the 256 x 256 tile.
-enum SyrkTile { SYRK_TILE_128, SYRK_TILE_128X2, SYRK_TILE_192, SYRK_TILE_256 };
-static SyrkTile pick_syrk_tile(int64_t n, int64_t batch, int64_t k) {
-#if defined(MI_FORCE_SYRK_TILE)  // tuning builds only: 128, 1282, 192 or 256
-  if (MI_FORCE_SYRK_TILE == 192) return SYRK_TILE_192;
-  if (MI_FORCE_SYRK_TILE == 256 && n % 256 == 0) return SYRK_TILE_256;
-  if (MI_FORCE_SYRK_TILE == 128 && n % 128 == 0) return SYRK_TILE_128;
-  if (MI_FORCE_SYRK_TILE == 1282 && n % 128 == 0) return SYRK_TILE_128X2;
-#endif
-#ifdef MI_HAS_SMALL_CFGS
+enum SyrkTile { SYRK_TILE_NONE, SYRK_TILE_128, SYRK_TILE_128X2, SYRK_TILE_192, SYRK_TILE_256 };
+// `k_strided`: the operand is stored transposed; its LDS layout exists for 128- and 256-row tiles only, and not for
+// tiles that overhang the matrix, so there may be no fast tile at all.
+static SyrkTile pick_syrk_tile(int64_t n, int64_t batch, int64_t k, bool k_strided) {
   const int64_t cus = num_cus();
   const double kt = (double)ceil_div(k, 64);
   auto tiles = [&](int64_t tile) {
     const int64_t t = ceil_div(n, tile);
     return t * (t + 1) / 2 * batch;
   };
-  SyrkTile best = SYRK_TILE_192;
-  double best_cost = (double)ceil_div(tiles(192), cus) * (12.6 + 0.80 * kt);
+  SyrkTile best = k_strided ? SYRK_TILE_NONE : SYRK_TILE_192;
+  double best_cost = k_strided ? 1e30 : (double)ceil_div(tiles(192), cus) * (12.6 + 0.80 * kt);
   auto offer = [&](SyrkTile t, double cost) {
     if (cost < best_cost) best = t, best_cost = cost;
   };
@@ -183,16 +128,9 @@ static SyrkTile pick_syrk_tile(int64_t n, int64_t batch, int64_t k) {
     offer(SYRK_TILE_128, (double)ceil_div(t128, cus) * (9.0 + (t128 <= cus ? 0.31 : 0.44) * kt));
   }
   return best;
-#else
-  (void)n; (void)batch; (void)k;
-  return SYRK_TILE_192;
-#endif
 }
 // 256 x 128 instead of 256 x 256 GEMM tiles for the whole product?
 static bool gemm_prefers_half_tiles(int64_t m, int64_t n, int64_t batch) {
-#if defined(MI_FORCE_GEMM_HALF)
-  if (MI_FORCE_GEMM_HALF) return true;  // tuning builds only
-#endif
   const int64_t cus = num_cus(), tiles = (m / 256) * (n / 256) * batch;
   return (double)ceil_div(2 * tiles, cus) * 0.5 * 1.27 < (double)ceil_div(tiles, cus);
 }
@@ -201,36 +139,35 @@ template <bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
 static int launch_class(TileClass tc, const GemmParams& p, int64_t batch, hipStream_t stream) {
   const bool k_ok = p.K % 64 == 0 && p.K >= 64;
   if (k_ok && p.M >= 1024 && p.N >= 1024) {
-    if constexpr (MODE == MODE_SYRK && !P_KS && !Q_KS) {
-      auto launch_tile = [&](const GemmParams& q, int64_t b) {
-        switch (pick_syrk_tile(q.M, b, q.K)) {
-#ifdef MI_HAS_SMALL_CFGS
-          case SYRK_TILE_128:
-            return launch_fast<CfgT128, false, false, MODE, OUT_F32>(q, b, stream);
-          case SYRK_TILE_128X2:
-            return launch_fast<CfgT128x2, false, false, MODE, OUT_F32>(q, b, stream);
-#endif
-          case SYRK_TILE_256:
-            return launch_fast<CfgBig, false, false, MODE, OUT_F32>(q, b, stream);
-          default:
-            return launch_fast<CfgSyrk192, false, false, MODE, OUT_F32>(q, b, stream);
-        }
-      };
-      return launch_tile(p, batch);
+    if constexpr (MODE == MODE_SYRK) {
+      static_assert(P_KS == Q_KS, "the lower-triangle product reads one operand in one layout");
+      switch (pick_syrk_tile(p.M, batch, p.K, P_KS)) {
+        case SYRK_TILE_128:
+          return launch_fast<CfgT128, P_KS, Q_KS, MODE, OUT_F32>(p, batch, stream);
+        case SYRK_TILE_128X2:
+          return launch_fast<CfgT128x2, P_KS, Q_KS, MODE, OUT_F32>(p, batch, stream);
+        case SYRK_TILE_256:
+          return launch_fast<CfgBig, P_KS, Q_KS, MODE, OUT_F32>(p, batch, stream);
+        case SYRK_TILE_192:
+          if constexpr (!P_KS) return launch_fast<CfgSyrk192, false, false, MODE, OUT_F32>(p, batch, stream);
+          break;
+        default:
+          break;  // no fast tile for this shape: the general kernel below
+      }
     }
     if constexpr (MODE == MODE_GEMM && !P_KS && Q_KS) {
       if (p.M % 256 == 0 && p.N % 256 == 0 && gemm_prefers_half_tiles(p.M, p.N, batch))
         return launch_fast<CfgHalfN, false, true, MODE, OUT_F32>(p, batch, stream);
     }
-    if (p.M % 256 == 0 && p.N % 256 == 0) return launch_fast<CfgBig, P_KS, Q_KS, MODE, OUT_F32>(p, batch, stream);
+    if constexpr (MODE == MODE_GEMM) {
+      if (p.M % 256 == 0 && p.N % 256 == 0) return launch_fast<CfgBig, P_KS, Q_KS, MODE, OUT_F32>(p, batch, stream);
+    }
   }
-#ifdef MI_HAS_SMALL_CFGS
   if constexpr (MODE == MODE_GEMM && !P_KS && Q_KS) {
     // short, wide products (per-head shapes): 128 x 256 tiles keep the direct-to-LDS loads and the coalesced epilogue
     if (k_ok && p.M % 128 == 0 && p.M < 1024 && p.N % 256 == 0 && p.N >= 256)
       return launch_fast<CfgM128, false, true, MODE, OUT_F32>(p, batch, stream);
   }
-#endif
   switch (tc) {
     case TILE_BIG:
       return launch_one<256, 256, 64, 2, 2, P_KS, Q_KS, MODE, OUT_F32>(p, batch, stream);
@@ -252,6 +189,7 @@ struct ShiftArgs {
   const float* group_abc = nullptr;  // SHIFT_GROUP_*: (a, b, c) of the steps of the group, 3 floats each
   int group_size = 0, stage = 0;
   const float* xscale = nullptr;  // first group of steps on an unnormalised X
+  int slot_capacity = 0;          // floats reserved per batch entry behind slots_out
   void apply(GemmParams& p) const {
     p.shift_mode = mode;
     p.xscale = xscale;
@@ -267,6 +205,7 @@ struct ShiftArgs {
     p.slots_out = slots_out;
     p.slot_stride = 0;  // filled in by the launcher
     p.slot_base = 0;
+    p.slot_capacity = slot_capacity;
   }
 };
 
@@ -310,9 +249,6 @@ static int syrk_impl(const void* A, int64_t batch, int64_t n, int64_t k, int64_t
   p.out_scale = 1.0f;
   p.skip_upper = skip_upper ? 1 : 0;
   if (sh) sh->apply(p);
-#ifdef MI_TIMING
-  p.slots_in = reinterpret_cast<const float*>(getenv("MI_TIMING_PTR") ? strtoull(getenv("MI_TIMING_PTR"), nullptr, 0) : 0ull);
-#endif
   TileClass tc = pick_class(n);
   return a_trans ? launch_class<true, true, MODE_SYRK, false>(tc, p, batch, stream)
                  : launch_class<false, false, MODE_SYRK, false>(tc, p, batch, stream);
@@ -348,9 +284,6 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
   p.out_scale = out_scale;
   p.out_accum = out_fp32 ? out_accum : 0.0f;
   if (sh) sh->apply(p);
-#ifdef MI_TIMING
-  p.slots_in = reinterpret_cast<const float*>(getenv("MI_TIMING_PTR") ? strtoull(getenv("MI_TIMING_PTR"), nullptr, 0) : 0ull);
-#endif
   TileClass tc = pick_class(m);
   if (!x_trans) {
     // OUT (m x n): P = Bm rows (K-contiguous), Q[j][k] = X[k][j] (K-strided).
@@ -365,7 +298,6 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
     // Tile-count quantisation: T full 256 x 256 tiles over C compute units leave a last round that is at
     // most half full when 0 < T mod C <= C/2.  If that remainder is a whole number of tile columns, those
     // columns are computed as 256 x 128 tiles instead (twice as many workgroups, one short round).
-#ifndef MI_NO_GEMM_SPLIT
     if (batch == 1 && m % 256 == 0 && n % 256 == 0 && m >= 1024 && n >= 1024 && m % 64 == 0) {
       const int64_t tm = m / 256, tn = n / 256, cus = num_cus();
       const int64_t rem = (tm * tn) % cus;
@@ -387,11 +319,10 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
         if (rc != MI_OK) return rc;
         rc = out_fp32 ? launch_fast<CfgHalfN, false, true, MODE_GEMM, true>(pt, batch, stream)
                       : launch_fast<CfgHalfN, false, true, MODE_GEMM, false>(pt, batch, stream);
-        g_last_tiles = tiles_main + tiles_tail;
+        g_last_launch.tiles = tiles_main + tiles_tail;
         return rc;
       }
     }
-#endif
     return out_fp32 ? launch_class<false, true, MODE_GEMM, true>(tc, p, batch, stream)
                     : launch_class<false, true, MODE_GEMM, false>(tc, p, batch, stream);
   }
@@ -849,15 +780,10 @@ static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, in
 // The slice length is fixed (512 columns), so the number of slices -- and with it the order of the float32
 // additions -- depends on the shape of one matrix only: a batched call and per-matrix calls agree bit for bit.
 static int small_gram_splits(int64_t batch, int64_t m, int64_t n) {
-#ifdef MI_HAS_SMALL_CFGS
   if (m % 128 != 0 || m > 256 || n % 512 != 0 || n < 1024) return 0;
   const int64_t splits = n / 512;
   if (batch * splits > 65535) return 0;
   return (int)splits;
-#else
-  (void)batch; (void)m; (void)n;
-  return 0;
-#endif
 }
 
 __global__ void __launch_bounds__(256) gram_reduce_kernel(const float* __restrict__ partials, int splits, int m,
@@ -1062,7 +988,6 @@ __global__ void __launch_bounds__(CH_THREADS) small_chain_kernel(ChainArgs a) {
   }
 }
 
-#ifdef MI_HAS_SMALL_CFGS
 // Split-K partial Gram matrices: the K range is cut into `splits` slices that run as extra batch entries.
 static int small_gram_partials(const uint16_t* X, int64_t batch, int64_t m, int64_t n, int splits, float* partials,
                                hipStream_t stream) {
@@ -1117,7 +1042,6 @@ static int small_chain(const uint16_t* X, int64_t batch, int64_t n, int splits, 
   if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "small_chain launch failed: %s", hipGetErrorString(e));
   return MI_OK;
 }
-#endif
 
 static size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
@@ -1209,7 +1133,13 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
   if (rows % 8 || cols % 8)
     return fail(MI_ERR_UNSUPPORTED_SHAPE, "rows and cols must be multiples of 8, got %lld x %lld", (long long)rows, (long long)cols);
   if (batch == 0 || rows == 0 || cols == 0) return MI_OK;
+  // Everything that can be refused is refused here, before the first kernel: the fused optimizer update changes the
+  // momentum buffer in its first pass, and an error after that would leave the state half updated.
+  if (batch > 65535) return fail(MI_ERR_UNSUPPORTED_SHAPE, "batch %lld exceeds the grid limit 65535", (long long)batch);
+  if (!aligned16(x) || !aligned16(out)) return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_newton_schulz_bf16: tensors must be 16-byte aligned");
+  if (rows > (1 << 30) || cols > (1 << 30)) return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_newton_schulz_bf16: extent too large");
   const NsWorkspace w = ns_layout(batch, rows, cols);
+  if (w.max_slots > INT32_MAX) return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_newton_schulz_bf16: matrix too large");
   if (!workspace || workspace_bytes < w.total)
     return fail(MI_ERR_WORKSPACE, "workspace too small: need %zu bytes, got %zu", w.total, workspace_bytes);
   if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(MI_ERR_WORKSPACE, "workspace must be 256-byte aligned");
@@ -1260,13 +1190,8 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
     const uint16_t* mult = gram;
     float alpha = b;
     int apply_mode = SHIFT_APPLY;
-#ifdef MI_HAS_SMALL_CFGS
     const bool chain = w.gram_splits > 0 && m == CH_M && c != 0.0f;
-#else
-    const bool chain = false;
-#endif
     if (chain) {
-#ifdef MI_HAS_SMALL_CFGS
       // 128-row matrices: Gram partials, then one launch per matrix for everything up to the multiplier of X
       {
         ProfScope prof(PROF_GRAM, stream);
@@ -1277,19 +1202,16 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
       mult = poly;
       alpha = 1.0f;
       if (taken > 1) apply_mode = SHIFT_GROUP_APPLY;
-#endif
     } else {
       // A' = X X^T - s I  (s = ||X||_F^2 / m from the partial sums the previous kernel left)
       ShiftArgs sh_gram{SHIFT_GRAM, b, c, slots, nslots, shift, nullptr};
       sh_gram.xscale = xs;
       {
         ProfScope prof(PROF_GRAM, stream);
-#ifdef MI_HAS_SMALL_CFGS
         if (w.gram_splits > 0)
           rc = small_gram(xbuf[cur], batch, m, n, w.gram_splits, reinterpret_cast<float*>(ws + w.gpart), slots, nslots, shift,
                           gram, stream, xs);
         else
-#endif
           rc = syrk_impl(xbuf[cur], batch, m, n, x_bs, ld, trans, nullptr, 0, m, 1.0f, 0.0f, gram, g_bs, m, 0, stream, &sh_gram);
       }
       if (rc != MI_OK) return rc;
@@ -1360,14 +1282,14 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
     sh_apply.group_size = taken;
     sh_apply.stage = taken - 1;
     sh_apply.xscale = xs;
+    sh_apply.slot_capacity = (int)w.max_slots;
     {
       ProfScope prof(PROF_APPLY, stream);
       rc = gemm_axpy_impl(mult, g_bs, m, xbuf[cur], x_bs, ld, trans, dst, x_bs, ld, batch, m, n, alpha, taken > 1 ? 1.0f : a,
                           last ? 1 : 0, last ? out_scale : 1.0f, stream, &sh_apply, (last && !tall) ? out_accum : 0.0f);
     }
     if (rc != MI_OK) return rc;
-    nslots = g_last_tiles;
-    if (nslots > w.max_slots) return fail(MI_ERR_WORKSPACE, "internal: %d partial-sum slots exceed the %lld reserved", nslots, (long long)w.max_slots);
+    nslots = g_last_launch.tiles;
     cur ^= 1;
     s += taken;
   }
@@ -1382,9 +1304,10 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
 }
 
 
+#pragma GCC visibility push(default)
 extern "C" {
 
-int mi_version(void) { return 100; }
+int mi_version(void) { return 200; }
 
 const char* mi_last_error(void) { return g_last_error.c_str(); }
 
@@ -1491,4 +1414,13 @@ int mi_muon_update_bf16(float* param, const float* grad, float* momentum, int64_
                  param_decay);
 }
 
+int mi_debug_last_launch(int* tiles, int* tile_m, int* tile_n, int* fast) {
+  if (tiles) *tiles = g_last_launch.tiles;
+  if (tile_m) *tile_m = g_last_launch.tile_m;
+  if (tile_n) *tile_n = g_last_launch.tile_n;
+  if (fast) *fast = g_last_launch.fast;
+  return MI_OK;
+}
+
 }  // extern "C"
+#pragma GCC visibility pop

@@ -49,6 +49,7 @@ EXPORTS = (
     ),
     ("mi_profile_begin", _int, ()),
     ("mi_profile_end", _int, (_vp, _vp)),
+    ("mi_debug_last_launch", _int, (_vp, _vp, _vp, _vp)),
 )
 
 _lock = threading.Lock()
@@ -87,6 +88,13 @@ def lib() -> ctypes.CDLL:
     if _lib is None:
         raise RuntimeError(f"HIP extension unavailable: {_load_error}")
     return _lib
+
+
+def last_launch() -> dict:
+    """Tile shape and workgroup count of the last product this thread launched (see ``mi_debug_last_launch``)."""
+    vals = [ctypes.c_int(0) for _ in range(4)]
+    check(lib().mi_debug_last_launch(*[ctypes.byref(v) for v in vals]))
+    return dict(zip(("tiles", "tile_m", "tile_n", "fast"), (v.value for v in vals)))
 
 
 def last_error() -> str:

@@ -52,6 +52,8 @@ const char* mi_last_error(void);
  * C[b] is (n, n), must be symmetric, may be NULL iff beta == 0.  D[b] is (n, n) row-major.
  * Only lower-triangle tiles are computed; every strictly-lower element is also stored at its
  * mirrored position unless skip_upper != 0, so D[b] is bitwise symmetric (syrk.py:221-224).
+ * With skip_upper != 0 the diagonal and everything below it are stored; an element above the diagonal is either
+ * left untouched or, where it shares a diagonal block with stored elements, holds its correct value.
  * D may alias neither A nor C.
  */
 int mi_syrk_bf16(const void* A, int64_t batch, int64_t n, int64_t k,
@@ -174,6 +176,14 @@ int mi_muon_update_bf16(float* param, const float* grad, float* momentum, int64_
  */
 int mi_profile_begin(void);
 int mi_profile_end(float* ms_by_kind, int* launches_by_kind);
+
+/*
+ * What the last product launched from this host thread used (for tests that must know which kernel variant served
+ * a shape; the reference's tests check its autotuner's config pruning instead,
+ * tests/test_triton_kernels.py:90-125): workgroups per batch entry, tile rows and columns, and whether it was the
+ * direct-to-LDS kernel (1) or the general one (0).  Any pointer may be NULL.
+ */
+int mi_debug_last_launch(int* tiles, int* tile_m, int* tile_n, int* fast);
 
 #ifdef __cplusplus
 }

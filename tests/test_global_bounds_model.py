@@ -1,0 +1,460 @@
+"""Host model of every GLOBAL address the direct-to-LDS kernels touch (emerging-optimizers_amd/csrc/gemm_fast.hpp with
+its launcher, launch_impl.hpp, and the tile enumerations of gemm_engine.hpp).
+
+The fast kernel's loaders have no bounds checks of their own: a tile that lies wholly inside its operand is fetched
+through precomputed lane offsets, and only the lower-triangle product of K-contiguous operands has a variant with
+clamped rows for tiles that overhang the matrix.  Whether a launch is safe is therefore decided on the host.  This
+model replays, for every tile configuration x operand layout x product the library instantiates,
+  * the launcher's decisions (tile counts, the padded lower-triangle grid, edge variant or refusal),
+  * workgroup id -> tile (``tri_block_decode`` with the XCD chunking, ``gemm_tile_of``),
+  * every 16-byte operand load of every wavefront for the first and the last K tile (``FastLoader``),
+  * the addend loads and every store of both epilogues (row-wise and mirrored write-out, GEMM staging),
+  * the per-workgroup partial-sum slot,
+over a grid of shapes (multiples of 8 on both sides of every tile size, batches, split-K slices, the tail split of
+the wide GEMM) and asserts that each access lies inside the matrix it belongs to.  It also checks that the tile
+enumerations visit every tile exactly once.  No GPU is involved.
+"""
+
+import itertools
+
+import numpy as np
+import pytest
+
+NW, BK, MI = 4, 64, 16
+LANES = np.arange(64)
+
+# name -> (TILE_M, TILE_N, WGM, WGN, ring slots)
+CFGS = {
+    "CfgM128": (128, 256, 1, 4, 2),
+    "CfgT128": (128, 128, 2, 2, 3),
+    "CfgT128x2": (128, 128, 2, 2, 2),
+    "CfgBig": (256, 256, 2, 2, 2),
+    "CfgHalfN": (256, 128, 2, 2, 3),
+    "CfgSyrk192": (192, 192, 2, 2, 3),
+}
+# (cfg, P K-strided, Q K-strided, mode) exactly as the inst_*.hip files instantiate them
+INSTANCES = [
+    ("CfgSyrk192", False, False, "syrk"), ("CfgT128", False, False, "syrk"), ("CfgBig", False, False, "syrk"),
+    ("CfgT128x2", False, False, "syrk"), ("CfgBig", True, True, "syrk"), ("CfgT128", True, True, "syrk"),
+    ("CfgT128x2", True, True, "syrk"), ("CfgBig", False, True, "gemm"), ("CfgHalfN", False, True, "gemm"),
+    ("CfgM128", False, True, "gemm"), ("CfgBig", False, False, "gemm"), ("CfgT128", False, False, "gemm"),
+]
+
+
+def kc_slot(row, c):
+    return c ^ ((row >> 1) & 7)
+
+
+def ks_rot(k):
+    return 2 * (k & 7) + 8 * (k >> 3)
+
+
+# ------------------------------------------------------------------ tile enumerations
+def tri_block_decode(s, T, block=6):
+    r = 0
+    while (r + 1) * (r + 2) // 2 <= s:
+        r += 1
+    bi = r // block
+    row0 = bi * block
+    h = min(T - row0, block)
+    u = s - row0 * (row0 + 1) // 2
+    rect = h * block
+    if u < bi * rect:
+        bj, v = divmod(u, rect)
+        return row0 + v // block, bj * block + v % block
+    u -= bi * rect
+    lr = 0
+    while (lr + 1) * (lr + 2) // 2 <= u:
+        lr += 1
+    return row0 + lr, row0 + (u - lr * (lr + 1) // 2)
+
+
+def gemm_tile_of(pid, tiles_m, tiles_n, xcds=8, block_m=8):
+    if tiles_n % xcds != 0 or tiles_m % block_m != 0:
+        return pid % tiles_m, pid // tiles_m
+    xcd, local = pid % xcds, pid // xcds
+    cols_per_xcd = tiles_n // xcds
+    block = block_m * cols_per_xcd
+    rb, r = divmod(local, block)
+    return rb * block_m + r % block_m, xcd * cols_per_xcd + r // block_m
+
+
+def syrk_grid_tiles(tiles_m):
+    """Workgroup id -> tile of the padded lower-triangle grid (None: padding workgroup that exits at once)."""
+    total = tiles_m * (tiles_m + 1) // 2
+    grid = (total + 7) // 8 * 8
+    per_xcd = grid // 8
+    out = []
+    for bid in range(grid):
+        s = (bid % 8) * per_xcd + bid // 8
+        out.append(tri_block_decode(s, tiles_m) if s < total else None)
+    return out
+
+
+@pytest.mark.parametrize("tiles_m", list(range(1, 70)))
+def test_lower_triangle_grid_visits_every_tile_once(tiles_m):
+    seen = [t for t in syrk_grid_tiles(tiles_m) if t is not None]
+    assert sorted(seen) == [(i, j) for i in range(tiles_m) for j in range(i + 1)]
+
+
+@pytest.mark.parametrize("tiles_m,tiles_n", [(4, 9), (8, 16), (16, 48), (16, 56), (8, 32), (1, 2), (3, 3), (16, 8), (24, 40), (7, 16)])
+def test_gemm_grid_visits_every_tile_once(tiles_m, tiles_n):
+    seen = [gemm_tile_of(pid, tiles_m, tiles_n) for pid in range(tiles_m * tiles_n)]
+    assert sorted(seen) == [(i, j) for i in range(tiles_m) for j in range(tiles_n)]
+
+
+# ------------------------------------------------------------------ operand loads
+class Matrix:
+    """A row-major (rows x cols) matrix inside a batch; every access must name an in-range row and a run of columns
+    that ends inside the row."""
+
+    def __init__(self, name, rows, cols, ld=None):
+        self.name, self.rows, self.cols, self.ld = name, rows, cols, cols if ld is None else ld
+
+    def check(self, rows, cols, width, what):
+        rows, cols = np.asarray(rows), np.asarray(cols)
+        ok = (rows >= 0) & (rows < self.rows) & (cols >= 0) & (cols + width <= self.cols)
+        assert ok.all(), f"{what}: {self.name}[{rows[~ok][:4]}, {cols[~ok][:4]} + {width}] outside {self.rows} x {self.cols}"
+
+
+def loader_accesses(rows_tile, ks, clamp, row0, rows_valid, kt, wave):
+    """(row, k) of the first element of every 16-byte load that `wave` issues for K tile `kt` of one operand tile
+    (rows = the operand's row index, k = its position along K), as FastLoader computes them."""
+    lpt = rows_tile * BK * 2 // 1024 // NW
+    out_r, out_k = [], []
+    b0 = wave * lpt
+    if clamp:
+        assert not ks
+        for i in range(lpt):
+            b = b0 + i
+            row = 8 * b + LANES // 8
+            c = kc_slot(row, LANES % 8)
+            gr = np.minimum(row0 + row, rows_valid - 1)
+            out_r.append(gr)
+            out_k.append(c * 8 + BK * kt)
+        return np.concatenate(out_r), np.concatenate(out_k)
+    if not ks:
+        period, nv = 2, 2
+        assert lpt % period == 0 and b0 % period == 0  # the phase of load i is i % 2 for every wavefront
+        for i in range(lpt):
+            v = i % nv
+            lr = LANES // 8
+            c = kc_slot(8 * v + lr, LANES % 8)
+            out_r.append(row0 + 8 * (b0 + i) + lr)
+            out_k.append(c * 8 + BK * kt)
+    else:
+        chunks, rows_per_kb = rows_tile // 8, 512 // rows_tile
+        period = max(chunks // rows_per_kb, 1)
+        periodic = lpt % period == 0
+        for i in range(lpt):
+            v = (i % min(period, lpt)) if periodic else b0 + i
+            kr = LANES // chunks
+            c = ((LANES % chunks) - ks_rot(rows_per_kb * v + kr)) & (chunks - 1)
+            if periodic:  # the offset registers are shared by all wavefronts: the phase must not depend on b0
+                c_true = ((LANES % chunks) - ks_rot(rows_per_kb * (b0 + i) + kr)) & (chunks - 1)
+                assert (c == c_true).all()
+            out_k.append(rows_per_kb * (b0 + i) + kr + BK * kt)
+            out_r.append(row0 + c * 8)
+    return np.concatenate(out_r), np.concatenate(out_k)
+
+
+_COVERED = set()
+
+
+def check_operand(mat_rows, K, ks, rows_tile, clamp, row0, kts, what, k_off=0, k_total=None):
+    """All loads of one operand tile.  The operand is (mat_rows x k_total) K-contiguous or (k_total x mat_rows)
+    K-strided in memory; the product covers k in [k_off, k_off + K)."""
+    k_total = K if k_total is None else k_total
+    mem = Matrix(what, k_total, mat_rows) if ks else Matrix(what, mat_rows, k_total)
+    for kt in kts:
+        for wave in range(NW):
+            r, k = loader_accesses(rows_tile, ks, clamp, row0, mat_rows, kt, wave)
+            if ks:
+                mem.check(k + k_off, r, 8, what)     # 8 consecutive rows of the operand at one k
+            else:
+                mem.check(r, k + k_off, 8, what)     # 8 consecutive k of one row
+            if not clamp:
+                assert (r >= row0).all() and (r < row0 + rows_tile).all()
+    # the tile is covered: every (row, k-chunk) of a K tile is fetched by exactly one lane (the lane arithmetic does
+    # not depend on the tile's position: checked once per layout)
+    if not clamp and (rows_tile, ks) not in _COVERED:
+        _COVERED.add((rows_tile, ks))
+        hits = np.zeros((rows_tile, BK), dtype=np.int32)
+        for wave in range(NW):
+            r, k = loader_accesses(rows_tile, ks, clamp, row0, mat_rows, 0, wave)
+            if ks:   # 8 consecutive rows at one k
+                for e in range(8):
+                    np.add.at(hits, (r - row0 + e, k), 1)
+            else:    # 8 consecutive k of one row
+                for e in range(8):
+                    np.add.at(hits, (r - row0, k + e), 1)
+        assert (hits == 1).all()
+
+
+# ------------------------------------------------------------------ epilogues
+def syrk_epilogue_accesses(cfg, M, m0, n0, diag, guard, skip_upper, addends, out, cmat):
+    tile, _, wgm, wgn, ns = CFGS[cfg]
+    tm = tile // wgm
+    fm = tm // MI
+    ring = ns * (2 * tile * BK * 2)
+    ldt = tile + 8
+    rp = tile if tile * ldt * 2 <= ring else tile // 2
+    npass = tile // rp
+    assert rp * ldt * 2 <= ring and rp % tm == 0
+    cprw = tile // 8
+    nt = NW * 64
+    assert rp * cprw % nt == 0
+    # addends, accumulator layout
+    for wave in range(NW):
+        wm, wn = wave % wgm, wave // wgm
+        for i in range(fm):
+            for j in range(fm):
+                m = m0 + wm * tm + i * MI + (LANES & 15)
+                n = n0 + wn * tm + j * MI + 4 * (LANES >> 4)
+                on = (m < M) & (n < M) if guard else np.ones(64, bool)
+                if addends:
+                    cmat.check(m[on], n[on], 4, "addend fetch")
+    # store counts in the tile's own window (rows from m0, columns from n0) and in the mirrored window
+    direct = np.zeros((tile, tile), dtype=np.int32)
+    mirror = direct if diag else np.zeros((tile, tile), dtype=np.int32)
+
+    def store(gr, gc, on):
+        gr, gc = gr[on], gc[on]
+        out.check(gr, gc, 8, "store")
+        in_direct = (gr >= m0) & (gr < m0 + tile) & (gc >= n0) & (gc + 8 <= n0 + tile)
+        in_mirror = (gr >= n0) & (gr < n0 + tile) & (gc >= m0) & (gc + 8 <= m0 + tile)
+        if diag:
+            assert in_direct.all(), "store outside the tile"
+        else:
+            assert (in_direct ^ in_mirror).all(), "store outside the tile and its mirror image"
+        for e in range(8):
+            np.add.at(direct, (gr[in_direct] - m0, gc[in_direct] - n0 + e), 1)
+            if not diag:
+                np.add.at(mirror, (gr[in_mirror] - n0, gc[in_mirror] - m0 + e), 1)
+
+    tids = np.arange(nt)
+    sym = diag and not skip_upper
+    for h in range(npass):
+        for it in range(rp * cprw // nt):
+            c = tids + it * nt
+            row, c8 = c // cprw, c % cprw
+            gr, gc = m0 + h * rp + row, n0 + c8 * 8
+            held = (c8 * 8 < ((h * rp + row) // tm + 1) * tm) if diag else np.ones(nt, bool)
+            on = held & ((gr < M) & (gc < M) if guard else True)
+            store(gr, gc, on)
+        if skip_upper:
+            continue
+
+        def mirror_out(rows, ccols, r_lo, grow0, gcol0):
+            nb = rows // 32
+            units = ccols // 4 * nb
+            for it in range((units + 15) // 16):
+                for wave in range(NW):
+                    unit = it * 16 + wave * 4 + (LANES >> 4)
+                    on = unit < units
+                    u = np.minimum(unit, units - 1)
+                    cq, rb = u // nb, u % nb
+                    l16 = LANES & 15
+                    gr, gc = grow0 + 4 * cq + (l16 & 3), gcol0 + 32 * rb + 8 * (l16 >> 2)
+                    if guard:
+                        on = on & (gr < M) & (gc < M)
+                    store(gr, gc, on)
+
+        if not diag:
+            mirror_out(rp, tile, 0, n0, m0 + h * rp)
+        elif (h + 1) * rp > tm:
+            lo = tm if npass == 1 else 0
+            mirror_out(tm, tm, lo, n0, m0 + h * rp + lo)
+    return direct, mirror
+
+
+def gemm_epilogue_accesses(cfg, M, N, m0, n0, xmat, out):
+    tile_m, tile_n, wgm, wgn, _ = CFGS[cfg]
+    tm, tn = tile_m // wgm, tile_n // wgn
+    assert tn in (32, 64, 128)
+    lpr = tn // 8
+    rpi = 64 // lpr
+    nit = MI // rpi
+    hits = np.zeros((tile_m, tile_n // 8), dtype=np.int32)
+    for wave in range(NW):
+        wm, wn = wave % wgm, wave // wgm
+        rr, cc = LANES // lpr, (LANES % lpr) * 8
+        for i in range(tm // MI):
+            for t in range(nit):
+                m = m0 + wm * tm + i * MI + t * rpi + rr
+                n = n0 + wn * tn + cc
+                xmat.check(m, n, 8, "Cin fetch")
+                out.check(m, n, 8, "store")
+                np.add.at(hits, (m - m0, (n - n0) // 8), 1)
+    assert (hits == 1).all()
+
+
+# ------------------------------------------------------------------ the launcher
+def launch_fast(cfg, p_ks, q_ks, mode, M, N, K):
+    """Mirrors launch_fast: ('refused', why) or ('ok', edge, tiles_m, tiles_n, grid)."""
+    tile_m, tile_n = CFGS[cfg][:2]
+    if K < BK or K % BK:
+        return ("refused", "K")
+    tiles_m, tiles_n = -(-M // tile_m), -(-N // tile_n)
+    grid = tiles_m * (tiles_m + 1) // 2 if mode == "syrk" else tiles_m * tiles_n
+    if mode == "syrk":
+        grid = (grid + 7) // 8 * 8
+    edge = M % tile_m != 0 or N % tile_n != 0
+    if edge and not (mode == "syrk" and not p_ks and not q_ks):
+        return ("refused", "edge")
+    return ("ok", edge, tiles_m, tiles_n, grid)
+
+
+def sample(seq, limit):
+    """First, last and an evenly spread selection of `seq` (the checks are per tile; the extremes matter most)."""
+    seq = list(seq)
+    if len(seq) <= limit:
+        return seq
+    idx = sorted(set([0, 1, len(seq) - 2, len(seq) - 1] + list(range(0, len(seq), max(len(seq) // limit, 1)))))
+    return [seq[i] for i in idx]
+
+
+SYRK_NS = [1024, 1032, 1096, 1152, 1280, 1536, 1792, 1800, 2048, 2304, 3072, 4096, 5120, 8192, 8184]
+SYRK_KS = [64, 128, 192, 1024, 14336]
+
+
+@pytest.mark.parametrize("cfg,p_ks,q_ks,mode", [i for i in INSTANCES if i[3] == "syrk"])
+def test_lower_triangle_launches_stay_inside_their_matrices(cfg, p_ks, q_ks, mode):
+    tile = CFGS[cfg][0]
+    launched = refused = 0
+    for n, k in itertools.product(SYRK_NS, SYRK_KS):
+        res = launch_fast(cfg, p_ks, q_ks, mode, n, n, k)
+        if res[0] == "refused":
+            assert n % tile != 0 and p_ks  # the only refusals: a K-strided operand whose last tile would overhang
+            refused += 1
+            continue
+        _, edge, tiles_m, _, grid = res
+        launched += 1
+        assert edge == (n % tile != 0)
+        tiles = syrk_grid_tiles(tiles_m)
+        assert len(tiles) == grid
+        nk = k // BK
+        out = Matrix("D", n, n)
+        cmat = Matrix("C", n, n)
+        real = [t for t in tiles if t is not None]
+        # corner tiles, the last block row (where the overhang is), diagonal and off-diagonal ones
+        last_row = [t for t in real if t[0] == tiles_m - 1]
+        picks = [(0, 0), (min(1, tiles_m - 1), 0), last_row[0], last_row[len(last_row) // 2], last_row[-1]] + sample(real, 4)
+        for tm_, tn_ in dict.fromkeys(picks):
+            m0, n0 = tm_ * tile, tn_ * tile
+            for ks, row0, what in ((p_ks, m0, "P"), (q_ks, n0, "Q")):
+                check_operand(n, k, ks, tile, edge, row0, sorted({0, nk - 1}), what)
+            if k != SYRK_KS[0]:
+                continue  # the epilogue does not depend on K
+            for skip_upper, addends in ((False, True), (True, False)):
+                diag = tm_ == tn_
+                direct, mirror = syrk_epilogue_accesses(cfg, n, m0, n0, diag, edge, skip_upper, addends, out, cmat)
+                # what ends up stored, each element once: the part of the tile inside the matrix (on a diagonal tile
+                # with the upper triangle skipped: without the block above the diagonal blocks) and, unless skipped,
+                # its mirror image
+                rr, cc = np.meshgrid(np.arange(tile), np.arange(tile), indexing="ij")
+                inside = (m0 + rr < n) & (n0 + cc < n)
+                if diag and skip_upper:
+                    inside &= cc < (rr // (tile // 2) + 1) * (tile // 2)
+                assert (direct == inside).all()
+                if not diag:
+                    want_mirror = ((n0 + rr < n) & (m0 + cc < n)) if not skip_upper else np.zeros_like(inside)
+                    assert (mirror == want_mirror).all()
+    assert launched > 0
+    assert (refused > 0) == p_ks
+
+
+GEMM_SHAPES = [(1024, 1024), (1024, 2304), (2048, 4096), (4096, 4096), (4096, 14336), (1792, 4096), (1280, 1536), (128, 512),
+               (384, 768), (896, 256), (128, 4096), (256, 1024), (1000, 2048), (1024, 1032), (1032, 2048)]
+
+
+@pytest.mark.parametrize("cfg,p_ks,q_ks,mode", [i for i in INSTANCES if i[3] == "gemm"])
+def test_gemm_launches_stay_inside_their_matrices(cfg, p_ks, q_ks, mode):
+    """GEMM+AXPY  OUT = beta X + alpha B X.  x_trans == 0: P = B (m x m, K-contiguous), Q[j][k] = X[k][j] (K-strided),
+    OUT and Cin are (m x n).  x_trans != 0: P = X^T (n x m), Q = B, OUT (n x m).  Shapes the tiles do not divide are
+    refused by the launcher (the callers never send them)."""
+    tile_m, tile_n = CFGS[cfg][:2]
+    launched = 0
+    for m, n in GEMM_SHAPES:
+        M, N, K = (m, n, m) if q_ks else (n, m, m)
+        res = launch_fast(cfg, p_ks, q_ks, mode, M, N, K)
+        if res[0] == "refused":
+            assert M % tile_m or N % tile_n or K % BK
+            continue
+        _, edge, tiles_m, tiles_n, grid = res
+        assert not edge and grid == tiles_m * tiles_n
+        launched += 1
+        nk = K // BK
+        out = Matrix("OUT", M, N)
+        pids = sample(range(grid), 10)
+        for pid in pids:
+            tm_, tn_ = gemm_tile_of(pid, tiles_m, tiles_n)
+            assert 0 <= tm_ < tiles_m and 0 <= tn_ < tiles_n
+            m0, n0 = tm_ * tile_m, tn_ * tile_n
+            check_operand(M, K, p_ks, tile_m, False, m0, sorted({0, nk - 1}), "P")
+            check_operand(N, K, q_ks, tile_n, False, n0, sorted({0, nk - 1}), "Q")
+            gemm_epilogue_accesses(cfg, M, N, m0, n0, Matrix("Cin", M, N), out)
+    assert launched > 0
+
+
+def test_tail_split_of_the_wide_gemm():
+    """batch 1, m = 4096, n = 14336 on 256 CUs: the last 2048 columns run as 256 x 128 tiles on pointers advanced by
+    `main_cols` elements; every access of both launches must stay inside the original matrices."""
+    m, n, cus = 4096, 14336, 256
+    tm, tn = m // 256, n // 256
+    rem = (tm * tn) % cus
+    assert rem > 0 and rem * 2 <= cus and rem % tm == 0 and tn > rem // tm
+    tail_cols = (rem // tm) * 256
+    main_cols = n - tail_cols
+    tiles_main, tiles_tail = tm * (main_cols // 256), tm * (tail_cols // 128)
+    assert (tiles_main, tiles_tail) == (768, 256)
+    nk = m // BK
+    for cfg, width, col_off in (("CfgBig", main_cols, 0), ("CfgHalfN", tail_cols, main_cols)):
+        tile_m, tile_n = CFGS[cfg][:2]
+        res = launch_fast(cfg, False, True, "gemm", m, width, m)
+        assert res[0] == "ok" and not res[1]
+        _, _, tiles_m, tiles_n, grid = res
+        xfull = Matrix("X", m, n)   # Q is X (k x columns) with ld = n; the tail launch starts `col_off` columns in
+        for pid in sample(range(grid), 12):
+            tm_, tn_ = gemm_tile_of(pid, tiles_m, tiles_n)
+            m0, n0 = tm_ * tile_m, tn_ * tile_n
+            check_operand(m, m, False, tile_m, False, m0, [0, nk - 1], "B")
+            for kt in (0, nk - 1):
+                for wave in range(NW):
+                    r, k = loader_accesses(tile_n, True, False, n0, width, kt, wave)
+                    xfull.check(k, r + col_off, 8, "X")
+        # partial-sum slots of both launches share one array of tiles_main + tiles_tail entries
+        base = 0 if cfg == "CfgBig" else tiles_main
+        assert base + grid <= tiles_main + tiles_tail
+
+
+@pytest.mark.parametrize("batch,m,n", [(32, 128, 4096), (2, 256, 1536), (4, 128, 1024), (1, 256, 1024)])
+def test_split_k_gram_partials(batch, m, n):
+    """Short, wide matrices: K slices of 512 columns run as extra batch entries of a 128 x 128-tile product whose
+    operand offset is outer * (m n) + inner * 512; every load must stay inside its matrix and inside its slice."""
+    splits = n // 512
+    assert m % 128 == 0 and n % 512 == 0
+    K = n // splits
+    res = launch_fast("CfgT128", False, False, "gemm", m, m, K)
+    assert res[0] == "ok" and not res[1]
+    _, _, tiles_m, tiles_n, grid = res
+    for y in sample(range(batch * splits), 8):
+        outer, inner = divmod(y, splits)
+        assert outer < batch
+        for pid in range(grid):
+            tm_, tn_ = gemm_tile_of(pid, tiles_m, tiles_n)
+            for row0, what in ((tm_ * 128, "P"), (tn_ * 128, "Q")):
+                check_operand(m, K, False, 128, False, row0, [0, K // BK - 1], what, k_off=inner * K, k_total=n)
+            gemm_epilogue_accesses("CfgT128", m, m, tm_ * 128, tn_ * 128, Matrix("none", m, m), Matrix("partial", m, m))
+
+
+def test_k_strided_edge_tiles_are_refused_not_clamped():
+    """A K-strided tile that overhangs the matrix would read past the end of each k-row (16-byte loads cannot be
+    clamped per element): the launcher must refuse it, and the loader has no such variant."""
+    for cfg, p_ks, q_ks, mode in INSTANCES:
+        tile_m, tile_n = CFGS[cfg][:2]
+        if p_ks or q_ks:
+            assert launch_fast(cfg, p_ks, q_ks, mode, 4096 + 8, 4096 + 8, 1024) == ("refused", "edge")
+        assert launch_fast(cfg, p_ks, q_ks, mode, 4096, 4096, 1000)[0] == "refused"   # K tail
+    with pytest.raises(AssertionError):
+        loader_accesses(256, True, True, 0, 1000, 0, 0)

@@ -5,7 +5,7 @@ neither sees an MFMA nor inserts the wait states an MFMA result needs before a V
 it.  That is safe only while the register allocator keeps every accumulator where it is for the whole K loop and
 the first read of an accumulator follows the drain (three ``s_nop 7``) after the loop.  A change elsewhere in a
 kernel (register pressure in the epilogue, for instance) can make the allocator swap or spill accumulator registers
-inside the loop; the result is then wrong in a few elements only.  This test compiles the library to assembly and
+inside the loop; the result is then wrong in a few elements only.  This test compiles every translation unit of the library to assembly and
 rejects, for every fast kernel,
   * any ``v_accvgpr_*`` move or AGPR spill inside an innermost loop that contains MFMAs,
   * any such instruction between an MFMA and the drain that follows it.
@@ -19,8 +19,6 @@ import subprocess
 import pytest
 
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "emerging-optimizers_amd", "csrc")
-FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-         "-Wno-unused-command-line-argument", "--cuda-device-only", "-S"]
 
 ACC_TRAFFIC = re.compile(r"^\s*(v_accvgpr_\w+|scratch_(store|load)\w*\s+(off,\s*)?a\[|scratch_load\w*\s+a\[)")
 
@@ -98,18 +96,19 @@ def test_detector_flags_swaps_and_spills():
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="hipcc not available")
 def test_no_accumulator_traffic_next_to_mfma(tmp_path):
-    asm = tmp_path / "mi_ns.s"
-    subprocess.run(["hipcc", *FLAGS, "mi_ns.hip", "-o", str(asm)], cwd=CSRC, check=True, capture_output=True, timeout=900)
+    # the Makefile's own flags, one assembly file per translation unit
+    subprocess.run(["make", "-j8", "-C", CSRC, "asm", f"ASMDIR={tmp_path}"], check=True, capture_output=True, timeout=900)
     kernels, name = {}, None
-    for line in asm.read_text().splitlines():
-        m = re.match(r"^(_ZN2mi\S+):\s", line)
-        if m:
-            name = m.group(1)
-            kernels[name] = []
-        elif name:
-            kernels[name].append(line)
-            if "s_endpgm" in line:
-                name = None
+    for asm in sorted(tmp_path.glob("*.s")):
+        for line in asm.read_text().splitlines():
+            m = re.match(r"^(_ZN2mi\S+):\s", line)
+            if m:
+                name = m.group(1)
+                kernels[name] = []
+            elif name:
+                kernels[name].append(line)
+                if "s_endpgm" in line:
+                    name = None
     fast = {n: ls for n, ls in kernels.items() if "gemm_fast_kernel" in n or "small_chain_kernel" in n}
     assert len(fast) >= 20 and all(any("v_mfma" in x for x in ls) for ls in fast.values())
     report = {n: accumulator_hazards(ls) for n, ls in fast.items()}
