@@ -1117,6 +1117,37 @@ static NsWorkspace ns_layout(int64_t batch, int64_t rows, int64_t cols) {
   return w;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Built-in scratch of mi_newton_schulz_bf16_noalloc: device memory that belongs to the loaded library itself (one
+// copy per GPU, held until the process ends), for callers that cannot allocate a workspace.
+// In host code `scratch` is only a handle for the symbol lookup below, never an address to hand to a kernel: each
+// device has its own copy at its own address, resolved once per device by hipGetSymbolAddress with that device current.
+// ---------------------------------------------------------------------------------------------
+static constexpr size_t SCRATCH_BYTES = MI_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
+
+static constexpr int SCRATCH_MAX_DEVICES = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[SCRATCH_MAX_DEVICES] = {};
+
+// Address of the current device's copy of `scratch` (looked up on the first call on that device).
+static int scratch_of_current_device(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= SCRATCH_MAX_DEVICES) return fail(MI_ERR_BAD_ARG, "device index %d is not supported", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr)
+      return fail(MI_ERR_LAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return MI_OK;
+}
+
 }  // namespace mi
 
 using namespace mi;
@@ -1398,6 +1429,20 @@ int mi_newton_schulz_bf16(const float* x, float* out, int64_t batch, int64_t row
                           int steps, float eps, int accumulate_fp64, float out_scale, void* workspace,
                           size_t workspace_bytes, void* stream) {
   return ns_impl(x, out, batch, rows, cols, abc, steps, eps, accumulate_fp64, out_scale, workspace, workspace_bytes,
+                 static_cast<hipStream_t>(stream), MomentumSrc{nullptr, 0.0f, 0}, 0.0f);
+}
+
+int mi_newton_schulz_bf16_noalloc(const float* x, float* out, int64_t batch, int64_t rows, int64_t cols, const float* abc,
+                                  int steps, float eps, int accumulate_fp64, float out_scale, void* stream) {
+  if (batch < 0 || rows < 0 || cols < 0) return fail(MI_ERR_BAD_ARG, "mi_newton_schulz_bf16_noalloc: negative argument");
+  if (batch == 0 || rows == 0 || cols == 0) return MI_OK;
+  const size_t need = ns_layout(batch, rows, cols).total;
+  if (need > SCRATCH_BYTES)
+    return fail(MI_ERR_WORKSPACE, "mi_newton_schulz_bf16_noalloc: this call needs %zu bytes of scratch, the built-in buffer has %zu", need,
+                SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (int rc = scratch_of_current_device(&ws)) return rc;
+  return ns_impl(x, out, batch, rows, cols, abc, steps, eps, accumulate_fp64, out_scale, ws, SCRATCH_BYTES,
                  static_cast<hipStream_t>(stream), MomentumSrc{nullptr, 0.0f, 0}, 0.0f);
 }
 

@@ -41,6 +41,7 @@ EXPORTS = (
     ("mi_frob_partials_len", _sz, (_i64, _i64)),
     ("mi_newton_schulz_bf16", _int, (_vp, _vp, _i64, _i64, _i64, _vp, _int, _f32, _int, _f32, _vp, _sz, _vp)),
     ("mi_newton_schulz_workspace_bytes", _sz, (_i64, _i64, _i64)),
+    ("mi_newton_schulz_bf16_noalloc", _int, (_vp, _vp, _i64, _i64, _i64, _vp, _int, _f32, _int, _f32, _vp)),
     ("mi_newton_schulz_schedule", _int, (_i64, _i64, _i64, _vp, _int, _vp, _int)),
     (
         "mi_muon_update_bf16",

@@ -136,6 +136,23 @@ int mi_newton_schulz_bf16(const float* x, float* out, int64_t batch, int64_t row
 size_t mi_newton_schulz_workspace_bytes(int64_t batch, int64_t rows, int64_t cols);
 
 /*
+ * mi_newton_schulz_bf16 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): the same computation with the workspace taken from a buffer of
+ * MI_NOALLOC_SCRATCH_BYTES that is part of the loaded library (each GPU the library runs on holds its own copy until
+ * the process ends).  No counterpart in the reference.  The call allocates and frees nothing and clears nothing with
+ * memset; calls whose mi_newton_schulz_workspace_bytes(batch, rows, cols) exceeds MI_NOALLOC_SCRATCH_BYTES return
+ * MI_ERR_WORKSPACE (128 MiB serve e.g. one 2048 x 8192 matrix, 4 x 1024 x 4096, or 32 x 128 x 4096).  All calls on
+ * one GPU share that GPU's buffer: calls that overlap in time on one GPU (different streams or host threads) race,
+ * and the buffer keeps the previous call's contents (every value the kernels read from it is written earlier in the
+ * same call).  The first call on a device looks up the buffer's address (hipGetSymbolAddress) and should be made
+ * outside stream capture.  Results are bit-identical to mi_newton_schulz_bf16.
+ */
+#define MI_NOALLOC_SCRATCH_BYTES ((size_t)128 << 20)
+int mi_newton_schulz_bf16_noalloc(const float* x, float* out, int64_t batch, int64_t rows, int64_t cols,
+                                  const float* abc, int steps, float eps, int accumulate_fp64, float out_scale,
+                                  void* stream);
+
+/*
  * How mi_newton_schulz_bf16 would group the steps of a call with these arguments (pure host code, no GPU needed):
  * writes the group sizes (1 = an ordinary step, 2 or 3 = that many steps on one Gram matrix) to groups[0..] and
  * returns their number (which may exceed max_groups; only max_groups entries are written), or a negative error
