@@ -349,23 +349,25 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x4_t (
 // A diagonal tile is made symmetric in LDS first: the wavefronts on the diagonal stage the lower half of their
 // block and fill its upper half with transposed 4 x 4 blocks; the block below the diagonal is written like any
 // other and mirrored into the tile's upper right.  The stored result is therefore symmetric bit for bit.
-// Tiles too large for the ring go in passes of RP rows.
-// The addends (the beta terms) are read straight in accumulator layout (8 bytes per quad, whole 32-byte sectors
-// per row); a one-pass tile requests the first one before the K loop.
+// The staging area may be larger than the ring (a 256 x 256 tile: 132 KB against 128 KB); the kernel sizes its LDS
+// for the larger of the two.
+// The addends (the beta terms) reach the accumulators in one of two ways.  Tiles of up to 192 x 192 read them straight
+// in accumulator layout (8 bytes per quad, whole 32-byte sectors per row), the first one before the K loop, the second
+// at the start of the epilogue.  A 256 x 256 tile has no registers to spare for that (256 accumulators per lane): its
+// addend tiles are copied to the staging area by the whole workgroup with 16-byte row-wise loads and picked up from
+// there in accumulator layout, one after the other; the finished values then overwrite them in place.
 // Every wavefront of the workgroup must call this (it contains barriers).
 // Geometry of the staged SYRK epilogue.
 template <class C>
 struct SyrkStage {
   static constexpr int TILE = C::TILE_M, LDT = TILE + 8;  // LDS row pitch in elements
-  static constexpr int RING = C::NS * C::SLOT_BYTES;
-  static constexpr int RP = (TILE * LDT * 2 <= RING) ? TILE : TILE / 2;  // rows per pass
-  static constexpr int NPASS = TILE / RP;
-  static constexpr int CPRW = TILE / 8;            // 16-byte chunks per tile row
-  static constexpr int NCH = RP * CPRW / C::NT;    // chunks per thread and pass
-  // a one-pass tile fetches its Cin values into registers before the K loop, in accumulator layout
-  // (one 8-byte quad per accumulator quad: NQUAD x 2 registers per lane)
+  static constexpr int STAGE_BYTES = TILE * LDT * 2;
+  static constexpr int CPRW = TILE / 8;              // 16-byte chunks per tile row
+  static constexpr int NCH = TILE * CPRW / C::NT;    // chunks per thread
+  // one 8-byte quad of an addend per accumulator quad: NQUAD x 2 registers per lane when held in registers
   static constexpr int NQUAD = C::FM * C::FN;
-  static constexpr bool CIN_EARLY = NPASS == 1 && NQUAD * 2 <= 80;
+  static constexpr bool CIN_EARLY = NQUAD * 2 <= 80;
+  static_assert(STAGE_BYTES <= 160 * 1024 - 256, "staging area exceeds the LDS");
 };
 // This lane's addend values of a one-pass tile, in accumulator layout: quad (i, j) covers row
 // m0 + mw + 16 i + (lane % 16), columns n0 + nw + 16 j + 4 (lane / 16) .. + 3.  One load
@@ -395,95 +397,109 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, f32x4_t (
                                                   bool diag, float alpha, float beta, float beta2, float shift,
                                                   const uint2 (&cin_pre)[SyrkStage<C>::CIN_EARLY ? SyrkStage<C>::NQUAD : 1]) {
   using S = SyrkStage<C>;
-  constexpr int LDT = S::LDT, MI = C::MI, FM = C::FM, FN = C::FN;
-  constexpr int RP = S::RP, NPASS = S::NPASS, CPRW = S::CPRW, NCH = S::NCH;
-  static_assert(RP * LDT * 2 <= S::RING, "staging pass exceeds the ring");
-  static_assert(RP % C::TM == 0 && RP % C::TN == 0, "a wavefront's block must fall into one pass");
+  constexpr int LDT = S::LDT, MI = C::MI, FM = C::FM, FN = C::FN, TILE = S::TILE;
+  constexpr int CPRW = S::CPRW, NCH = S::NCH;
   static_assert(C::TILE_M == C::TILE_N, "square tiles");
   static_assert(C::WGM == 2 && C::WGN == 2 && C::TM == C::TN, "2 x 2 wavefronts with square blocks: the diagonal blocks are (0,0) and (1,1)");
-  static_assert(RP * CPRW % C::NT == 0, "write-out must divide evenly");
+  static_assert(TILE * CPRW % C::NT == 0, "write-out must divide evenly");
   const int tid = threadIdx.x;
   const int frow = lane & (MI - 1), fk = lane / MI;
   const int mw = wm * C::TM, nw = wn * C::TN;           // this wavefront's block inside the tile
   uint16_t* __restrict__ ob = reinterpret_cast<uint16_t*>(p.Out) + batch * p.o_bs;
   const uint16_t* __restrict__ Cb = p.Cin ? p.Cin + batch * p.c_bs : nullptr;
   const bool use_c = beta != 0.0f && Cb != nullptr;
-
   const uint16_t* __restrict__ Cb2 = p.Cin2 ? p.Cin2 + batch * p.c_bs : nullptr;
   const bool use_c2 = beta2 != 0.0f && Cb2 != nullptr;
+  // whether this wavefront's block holds anything that is stored (see idle_wave in the kernel)
+  const bool active = (m0 + mw < p.M) && (n0 + nw < p.N) && !(diag && nw >= mw + C::TM);
 
-  // Finished bf16 quads of this lane.  A one-pass tile keeps them in registers; a tile staged in passes (a 256 x 256
-  // tile: 128 quads on top of 256 accumulators) finishes each quad on its way to LDS.
-  uint2 val[NPASS == 1 ? FM : 1][NPASS == 1 ? FN : 1];
+  auto add = [&](f32x4_t& v, const uint2& raw, float coef) {
+    v[0] = __builtin_fmaf(coef, __uint_as_float(raw.x << 16), v[0]);
+    v[1] = __builtin_fmaf(coef, __uint_as_float(raw.x & 0xffff0000u), v[1]);
+    v[2] = __builtin_fmaf(coef, __uint_as_float(raw.y << 16), v[2]);
+    v[3] = __builtin_fmaf(coef, __uint_as_float(raw.y & 0xffff0000u), v[3]);
+  };
+  auto finish = [&](f32x4_t v, int ml, int nl) -> uint2 {  // the shift on the diagonal, then one rounding to bf16
+    if (p.shift_mode == SHIFT_GRAM && diag) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (nl + r == ml) v[r] -= shift;
+    }
+    return __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));
+  };
+
+  // Finished bf16 quads of this lane, when they are few enough to be kept in registers.
+  uint2 val[S::CIN_EARLY ? FM : 1][S::CIN_EARLY ? FN : 1];
   // ---- values: alpha * acc (+ beta * Cin) (+ beta2 * Cin2) (- shift on the diagonal), rounded to bf16 ----
-  if constexpr (NPASS == 1) {
+  if constexpr (S::CIN_EARLY) {
     // Both addends arrive in accumulator layout: the first was requested before the K loop, the second is
     // requested now and consumed after the first.
-    constexpr int NQ = S::NQUAD;
-    uint2 c2[NQ];
+    uint2 c2[S::NQUAD];
     if (use_c2) syrk_addend_fetch<C, GUARD>(p, Cb2, lane, m0 + mw, n0 + nw, c2);
-    uint2 c1[S::CIN_EARLY ? 1 : NQ];
-    if constexpr (!S::CIN_EARLY) {
-      if (use_c) syrk_addend_fetch<C, GUARD>(p, Cb, lane, m0 + mw, n0 + nw, c1);
-    }
-    auto add = [&](f32x4_t& v, const uint2& raw, float coef) {
-      v[0] = __builtin_fmaf(coef, __uint_as_float(raw.x << 16), v[0]);
-      v[1] = __builtin_fmaf(coef, __uint_as_float(raw.x & 0xffff0000u), v[1]);
-      v[2] = __builtin_fmaf(coef, __uint_as_float(raw.y << 16), v[2]);
-      v[3] = __builtin_fmaf(coef, __uint_as_float(raw.y & 0xffff0000u), v[3]);
-    };
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+        const int ml = mw + i * MI + frow, nl = nw + j * MI + 4 * fk;
+        f32x4_t v;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][r];
+        if (use_c) add(v, cin_pre[i * FN + j], beta);
+        if (use_c2) add(v, c2[i * FN + j], beta2);
+        val[i][j] = finish(v, ml, nl);
+      }
+    __syncthreads();  // every wavefront has left the K loop: the ring can be reused as staging space
+  } else {
+    // Large tile: every addend tile goes through the staging area.  The workgroup copies it there row by row (16 bytes
+    // per lane, whole rows per 32 lanes), each lane adds its quads to its accumulators, and the next addend or the
+    // finished values overwrite it.
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
       for (int j = 0; j < FN; ++j)
-{
-          const int ml = mw + i * MI + frow, nl = nw + j * MI + 4 * fk;
-          const int q = i * FN + j;
-          f32x4_t v;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][r];
-          if (use_c) {
-            if constexpr (S::CIN_EARLY)
-              add(v, cin_pre[q], beta);
-            else
-              add(v, c1[q], beta);
-          }
-          if (use_c2) add(v, c2[q], beta2);
-          if (p.shift_mode == SHIFT_GRAM && diag) {
+        for (int r = 0; r < 4; ++r) acc[i][j][r] *= alpha;
+    auto stage_addend = [&](const uint16_t* __restrict__ src, float coef) {
+      __syncthreads();  // nobody reads the area any more (the ring, or the previous addend)
+      constexpr int BATCH = 8;
+      static_assert(NCH % BATCH == 0, "addend copy goes in batches");
+#pragma unroll 1
+      for (int it0 = 0; it0 < NCH; it0 += BATCH) {
+        uint4 buf[BATCH];
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-              if (nl + r == ml) v[r] -= shift;
-          }
-          val[i][j] = __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));
+        for (int u = 0; u < BATCH; ++u) {
+          const int c = tid + (it0 + u) * C::NT, row = c / CPRW, c8 = c % CPRW;
+          const int gr = m0 + row, gc = n0 + c8 * 8;
+          buf[u] = make_uint4(0u, 0u, 0u, 0u);
+          if (!GUARD || (gr < p.M && gc < p.N)) buf[u] = *reinterpret_cast<const uint4*>(src + (int64_t)gr * p.ldc + gc);
         }
+#pragma unroll
+        for (int u = 0; u < BATCH; ++u) {
+          const int c = tid + (it0 + u) * C::NT, row = c / CPRW, c8 = c % CPRW;
+          *reinterpret_cast<uint4*>(lds + (row * LDT + c8 * 8) * 2) = buf[u];
+        }
+      }
+      __syncthreads();
+      if (active) {
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+          for (int j = 0; j < FN; ++j) {
+            const int ml = mw + i * MI + frow, nl = nw + j * MI + 4 * fk;
+            add(acc[i][j], *reinterpret_cast<const uint2*>(lds + (ml * LDT + nl) * 2), coef);
+          }
+      }
+    };
+    if (use_c) stage_addend(Cb, beta);
+    if (use_c2) stage_addend(Cb2, beta2);
+    __syncthreads();  // the area is free for the finished values
   }
-  // finished bf16 quad (i, j) of this lane; a tile staged in passes reads its addends here, in accumulator layout
-  // (fetching them a fragment row ahead into registers was tried: it spills and is slower)
+  // finished bf16 quad (i, j) of this lane
   auto quad = [&](int i, int j) -> uint2 {
-    if constexpr (NPASS == 1) {
+    if constexpr (S::CIN_EARLY)
       return val[i][j];
-    } else {
-      const int ml = mw + i * MI + frow, nl = nw + j * MI + 4 * fk;
-      auto add = [&](f32x4_t& v, const uint2& raw, float coef) {
-        v[0] = __builtin_fmaf(coef, __uint_as_float(raw.x << 16), v[0]);
-        v[1] = __builtin_fmaf(coef, __uint_as_float(raw.x & 0xffff0000u), v[1]);
-        v[2] = __builtin_fmaf(coef, __uint_as_float(raw.y << 16), v[2]);
-        v[3] = __builtin_fmaf(coef, __uint_as_float(raw.y & 0xffff0000u), v[3]);
-      };
-      f32x4_t v;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][r];
-      if (!GUARD || (m0 + ml < p.M && n0 + nl < p.N)) {
-        if (use_c) add(v, *reinterpret_cast<const uint2*>(Cb + (int64_t)(m0 + ml) * p.ldc + n0 + nl), beta);
-        if (use_c2) add(v, *reinterpret_cast<const uint2*>(Cb2 + (int64_t)(m0 + ml) * p.ldc + n0 + nl), beta2);
-      }
-      if (p.shift_mode == SHIFT_GRAM && diag) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (nl + r == ml) v[r] -= shift;
-      }
-      return __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));
-    }
+    else
+      return finish(acc[i][j], mw + i * MI + frow, nw + j * MI + 4 * fk);
   };
   auto elem = [&](const uint2& q, int r) -> uint16_t {
     return (uint16_t)(r == 0 ? (q.x & 0xffffu) : r == 1 ? (q.x >> 16) : r == 2 ? (q.y & 0xffffu) : (q.y >> 16));
@@ -515,82 +531,73 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, f32x4_t (
         *reinterpret_cast<uint4*>(ob + (int64_t)gr * p.ldo + gc) = make_uint4(t0.x, t0.y, t1.x, t1.y);
     }
   };
-  for (int h = 0; h < NPASS; ++h) {
-    __syncthreads();  // previous readers of the staging area are done
-    // ---- this pass's rows, row-major ----
-    if (mw / RP == h) {
-      if (!sym || wm > wn) {
+  // ---- the tile, row-major ----
+  if (!sym || wm > wn) {
 #pragma unroll
-        for (int i = 0; i < FM; ++i) {
+    for (int i = 0; i < FM; ++i) {
 #pragma unroll
-          for (int j = 0; j < FN; ++j)
-{
-              const int ml = mw + i * MI + frow, nl = nw + j * MI + 4 * fk;
-              *reinterpret_cast<uint2*>(lds + ((ml - h * RP) * LDT + nl) * 2) = quad(i, j);
-            }
-        }
-      } else if (wm == wn) {
-        // block on the diagonal: quads below the diagonal's 4 x 4 blocks go in whole, a quad inside such a block
-        // puts its lower elements at both positions; the rest of the upper half is filled in below
+      for (int j = 0; j < FN; ++j) {
+        const int ml = mw + i * MI + frow, nl = nw + j * MI + 4 * fk;
+        *reinterpret_cast<uint2*>(lds + (ml * LDT + nl) * 2) = quad(i, j);
+      }
+    }
+  } else if (wm == wn) {
+    // block on the diagonal: quads below the diagonal's 4 x 4 blocks go in whole, a quad inside such a block
+    // puts its lower elements at both positions; the rest of the upper half is filled in below
 #pragma unroll
-        for (int i = 0; i < FM; ++i) {
+    for (int i = 0; i < FM; ++i) {
 #pragma unroll
-          for (int j = 0; j <= i; ++j)
-{
-              const int ml = mw + i * MI + frow, nl = nw + j * MI + 4 * fk;
-              if (j < i || nl < (ml & ~3)) {
-                *reinterpret_cast<uint2*>(lds + ((ml - h * RP) * LDT + nl) * 2) = quad(i, j);
-              } else if (nl == (ml & ~3)) {
-                const uint2 q4 = quad(i, j);
+      for (int j = 0; j <= i; ++j) {
+        const int ml = mw + i * MI + frow, nl = nw + j * MI + 4 * fk;
+        if (j < i || nl < (ml & ~3)) {
+          *reinterpret_cast<uint2*>(lds + (ml * LDT + nl) * 2) = quad(i, j);
+        } else if (nl == (ml & ~3)) {
+          const uint2 q4 = quad(i, j);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                  const uint16_t e = elem(q4, r);
-                  if (nl + r <= ml) *reinterpret_cast<uint16_t*>(lds + ((ml - h * RP) * LDT + nl + r) * 2) = e;
-                  if (nl + r < ml) *reinterpret_cast<uint16_t*>(lds + ((nl + r - h * RP) * LDT + ml) * 2) = e;
-                }
-              }
-            }
+          for (int r = 0; r < 4; ++r) {
+            const uint16_t e = elem(q4, r);
+            if (nl + r <= ml) *reinterpret_cast<uint16_t*>(lds + (ml * LDT + nl + r) * 2) = e;
+            if (nl + r < ml) *reinterpret_cast<uint16_t*>(lds + ((nl + r) * LDT + ml) * 2) = e;
+          }
         }
       }
     }
-    if (sym) {
-      __syncthreads();
-      if (wm == wn && mw / RP == h) {
-        // upper 4 x 4 blocks of the diagonal block <- transposed lower ones (16 blocks per transpose read)
-        constexpr int NB4 = C::TM / 4;
-        static_assert(NB4 * NB4 % 16 == 0, "blocks must fill whole transpose reads");
-        const int rowbase = mw - h * RP, colbase = nw;
-        for (int it = 0; it < NB4 * NB4 / 16; ++it) {
-          const int ids = it * 16 + 4 * (lane >> 4) + (lane & 3);  // block this lane fetches a row of
-          const uint2 t =
-              tr_read((uint32_t)(((rowbase + 4 * (ids / NB4) + (l16 >> 2)) * LDT + colbase + 4 * (ids % NB4)) * 2));
-          const int idr = it * 16 + (lane >> 2), br = idr / NB4, bc = idr % NB4;  // block this lane receives a column of
-          if (br > bc) *reinterpret_cast<uint2*>(lds + ((rowbase + 4 * bc + (lane & 3)) * LDT + colbase + 4 * br) * 2) = t;
-        }
-      }
-    }
+  }
+  if (sym) {
     __syncthreads();
-    // ---- row-wise write-out: LDS rows [0, RP) -> global rows m0 + h RP + row ----
-#pragma unroll
-    for (int it = 0; it < NCH; ++it) {
-      const int c = tid + it * C::NT, row = c / CPRW, c8 = c % CPRW;
-      const int gr = m0 + h * RP + row, gc = n0 + c8 * 8;
-      const uint4 v = *reinterpret_cast<const uint4*>(lds + (row * LDT + c8 * 8) * 2);
-      // a diagonal tile holds nothing right of the diagonal block of a row (the wavefront that owns that block sits
-      // the product out): that part comes from the mirror image, or stays unwritten when the upper triangle is skipped
-      const bool held = !diag || c8 * 8 < ((h * RP + row) / C::TM + 1) * C::TM;
-      if (held && (!GUARD || (gr < p.M && gc < p.N))) *reinterpret_cast<uint4*>(ob + (int64_t)gr * p.ldo + gc) = v;
-    }
-    // ---- the mirror image, straight from the staged rows ----
-    if (!p.skip_upper) {
-      if (!diag) {
-        mirror_out(std::integral_constant<int, RP>{}, std::integral_constant<int, C::TILE_M>{}, 0, n0, m0 + h * RP);
-      } else if ((h + 1) * RP > C::TM) {
-        // blocks below the diagonal blocks (rows from TM on, columns before TM) go to the upper right of the tile
-        constexpr int LO = NPASS == 1 ? C::TM : 0;  // first such row of the staged pass
-        static_assert(NPASS == 1 || RP == C::TM, "a pass is the tile or one block row");
-        mirror_out(std::integral_constant<int, C::TM>{}, std::integral_constant<int, C::TM>{}, LO, n0, m0 + h * RP + LO);
+    if (wm == wn) {
+      // upper 4 x 4 blocks of the diagonal block <- transposed lower ones (16 blocks per transpose read)
+      constexpr int NB4 = C::TM / 4;
+      static_assert(NB4 * NB4 % 16 == 0, "blocks must fill whole transpose reads");
+      const int rowbase = mw, colbase = nw;
+      for (int it = 0; it < NB4 * NB4 / 16; ++it) {
+        const int ids = it * 16 + 4 * (lane >> 4) + (lane & 3);  // block this lane fetches a row of
+        const uint2 t =
+            tr_read((uint32_t)(((rowbase + 4 * (ids / NB4) + (l16 >> 2)) * LDT + colbase + 4 * (ids % NB4)) * 2));
+        const int idr = it * 16 + (lane >> 2), br = idr / NB4, bc = idr % NB4;  // block this lane receives a column of
+        if (br > bc) *reinterpret_cast<uint2*>(lds + ((rowbase + 4 * bc + (lane & 3)) * LDT + colbase + 4 * br) * 2) = t;
       }
+    }
+  }
+  __syncthreads();
+  // ---- row-wise write-out: LDS row -> global row m0 + row ----
+#pragma unroll
+  for (int it = 0; it < NCH; ++it) {
+    const int c = tid + it * C::NT, row = c / CPRW, c8 = c % CPRW;
+    const int gr = m0 + row, gc = n0 + c8 * 8;
+    const uint4 v = *reinterpret_cast<const uint4*>(lds + (row * LDT + c8 * 8) * 2);
+    // a diagonal tile holds nothing right of the diagonal block of a row (the wavefront that owns that block sits
+    // the product out): that part comes from the mirror image, or stays unwritten when the upper triangle is skipped
+    const bool held = !diag || c8 * 8 < (row / C::TM + 1) * C::TM;
+    if (held && (!GUARD || (gr < p.M && gc < p.N))) *reinterpret_cast<uint4*>(ob + (int64_t)gr * p.ldo + gc) = v;
+  }
+  // ---- the mirror image, straight from the staged rows ----
+  if (!p.skip_upper) {
+    if (!diag) {
+      mirror_out(std::integral_constant<int, TILE>{}, std::integral_constant<int, TILE>{}, 0, n0, m0);
+    } else {
+      // the block below the diagonal blocks (rows from TM on, columns before TM) goes to the upper right of the tile
+      mirror_out(std::integral_constant<int, C::TM>{}, std::integral_constant<int, C::TM>{}, C::TM, n0, m0 + C::TM);
     }
   }
 }
@@ -603,8 +610,14 @@ constexpr int waitcnt_imm(int vmcnt, int lgkmcnt) {
 template <class C, bool P_KS, bool Q_KS, int MODE, bool OUT_F32, bool EDGE>
 __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   constexpr int NS = C::NS, FM = C::FM, FN = C::FN, P_BYTES = C::P_BYTES, NT = C::NT;
-  // One array per ring slot: every LDS access below names its slot statically.
-  __shared__ __align__(1024) char ring[NS][C::SLOT_BYTES];
+  // The ring of operand slots; every LDS access of the K loop names its slot statically (ring[u] is a constant
+  // offset into one LDS array).  The lower-triangle epilogue reuses the memory as its staging area, which may be
+  // larger than the ring, so the array is sized for the larger of the two.
+  constexpr bool SYRK_STAGED = MODE == MODE_SYRK && !OUT_F32 && C::NW == 4;
+  constexpr int RING_BYTES = NS * C::SLOT_BYTES;
+  constexpr int LDS_BYTES = (SYRK_STAGED && SyrkStage<C>::STAGE_BYTES > RING_BYTES) ? SyrkStage<C>::STAGE_BYTES : RING_BYTES;
+  __shared__ __align__(1024) char lds_mem[LDS_BYTES];
+  char(*const ring)[C::SLOT_BYTES] = reinterpret_cast<char(*)[C::SLOT_BYTES]>(lds_mem);
   __shared__ float red[NT / 64];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -782,7 +795,6 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   else
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
   __syncthreads();
-  constexpr bool SYRK_STAGED = MODE == MODE_SYRK && !OUT_F32 && C::NW == 4;
   constexpr bool CIN_EARLY = SYRK_STAGED && SyrkStage<C>::CIN_EARLY;
   uint2 cin_pre[CIN_EARLY ? SyrkStage<C>::NQUAD : 1];
   if constexpr (CIN_EARLY) {

@@ -90,21 +90,20 @@ static int num_cus() {
   return cached;
 }
 
-// Tile choice of the fast path by modelled time: rounds of workgroups over the CUs times the cost of one tile.
-// Measured on this part (SYRK n = 1024 .. 8192, batch 1 .. 16, K 1024 .. 14336; GEMM m = 1024 .. 4096).
+// Tile choice of the fast path by modelled time, fitted to measurements on this part (lower-triangle products with
+// n = 1024 .. 8192, batch 1 .. 16, K = 64 .. 8192; GEMM m = 1024 .. 4096).
 //  * GEMM: 256 x 128 tiles cost about 1.27x per FLOP of 256 x 256 tiles and win when the latter leave CUs idle
 //    (1024 x 4096: 64 tiles).
-// Tile of the lower-triangle kernel.  Modelled time of a launch = rounds x (start-up + epilogue + k-tiles x time per
-// 64-deep k-tile), in microseconds, fitted to measurements on this part (256 CUs, all busy):
-//   192 x 192 (one workgroup per CU)             12.6 + 0.80 kt
-//   256 x 256 (one per CU, two-pass epilogue)    29.7 + 1.30 kt   needs n % 256 == 0
-//   128 x 128, two-slot ring (two per CU)         9.2 + s kt per pair of tiles, s = 0.74 (kt <= 32) .. 0.85 (kt >= 128:
-//                                                 long runs of MFMA work from two workgroups lower the clock),
-//                                                 needs n % 128 == 0
-//   128 x 128, three-slot ring (one per CU)       9.0 + 0.44 kt (0.31 kt when the tiles do not fill the CUs: the
-//                                                 clock rises), needs n % 128 == 0
-// Short K or few tiles favour the small tiles (their epilogue is short and, two to a CU, hidden), long K the
-// 192 x 192 tile, and row counts that 192 divides badly (1792 = 7 x 256) the 256 x 256 tile.
+//  * Lower-triangle kernel: a launch runs in rounds of one workgroup per CU (two for the two-slot 128 x 128 tile); a
+//    round costs F + s kt microseconds (kt = 64-deep K tiles).  F is launch, prologue and the write-out of the tiles
+//    (bound by the write bandwidth of the fabric, about 13 us for the 33 MB of a 4096 x 4096 result).  s rises with
+//    the share f of the CUs that a round keeps busy, because the clock follows the power drawn:
+//      192 x 192                    F = 14.5   s = 0.55 (f <= 0.45) .. 0.78 (f = 1)
+//      256 x 256 (n % 256 == 0)     F = 16.5   s = 0.95 (f <= 0.55) .. 1.37 (f >= 0.9)
+//      128 x 128, two per CU        F =  9.2   s = 0.74 (kt <= 32) .. 0.85 (kt >= 128) per pair of tiles   (n % 128 == 0)
+//      128 x 128, one per CU        F =  9.0   s = 0.44 (0.31 when one round is not full)                  (n % 128 == 0)
+//    Short K or few tiles favour the small tiles, long K with many tiles the 192 x 192 tile, and shapes whose
+//    256 x 256 tiles fill one round (8 x 1792: 224 tiles) or that 192 divides badly the 256 x 256 tile.
 enum SyrkTile { SYRK_TILE_NONE, SYRK_TILE_128, SYRK_TILE_128X2, SYRK_TILE_192, SYRK_TILE_256 };
 // `k_strided`: the operand is stored transposed; its LDS layout exists for 128- and 256-row tiles only, and not for
 // tiles that overhang the matrix, so there may be no fast tile at all.
@@ -115,12 +114,19 @@ static SyrkTile pick_syrk_tile(int64_t n, int64_t batch, int64_t k, bool k_strid
     const int64_t t = ceil_div(n, tile);
     return t * (t + 1) / 2 * batch;
   };
+  // full rounds at the slope of a full chip, the last partial round at the slope of its own fill
+  auto by_rounds = [&](int64_t count, double fixed, auto slope) {
+    const int64_t full = count / cus, rem = count % cus;
+    return (double)full * (fixed + slope(1.0) * kt) + (rem ? fixed + slope((double)rem / (double)cus) * kt : 0.0);
+  };
+  auto slope192 = [](double f) { return f <= 0.45 ? 0.55 : 0.55 + (f - 0.45) * 0.42; };
+  auto slope256 = [](double f) { return f <= 0.55 ? 0.95 : std::min(1.37, 0.95 + (f - 0.55) * 1.2); };
   SyrkTile best = k_strided ? SYRK_TILE_NONE : SYRK_TILE_192;
-  double best_cost = k_strided ? 1e30 : (double)ceil_div(tiles(192), cus) * (12.6 + 0.80 * kt);
+  double best_cost = k_strided ? 1e30 : by_rounds(tiles(192), 14.5, slope192);
   auto offer = [&](SyrkTile t, double cost) {
     if (cost < best_cost) best = t, best_cost = cost;
   };
-  if (n % 256 == 0) offer(SYRK_TILE_256, (double)ceil_div(tiles(256), cus) * (29.7 + 1.30 * kt));
+  if (n % 256 == 0) offer(SYRK_TILE_256, by_rounds(tiles(256), 16.5, slope256));
   if (n % 128 == 0) {
     const int64_t t128 = tiles(128);
     const double s2 = 0.74 + 0.11 * std::min(std::max(kt - 32.0, 0.0) / 96.0, 1.0);

@@ -196,15 +196,24 @@ def syrk_epilogue_accesses(cfg, M, m0, n0, diag, guard, skip_upper, addends, out
     tile, _, wgm, wgn, ns = CFGS[cfg]
     tm = tile // wgm
     fm = tm // MI
-    ring = ns * (2 * tile * BK * 2)
     ldt = tile + 8
-    rp = tile if tile * ldt * 2 <= ring else tile // 2
-    npass = tile // rp
-    assert rp * ldt * 2 <= ring and rp % tm == 0
+    rp, npass = tile, 1          # the whole tile is staged at once (the kernel sizes its LDS for it)
+    assert rp * ldt * 2 <= 160 * 1024 - 256 and ns >= 2
     cprw = tile // 8
     nt = NW * 64
     assert rp * cprw % nt == 0
-    # addends, accumulator layout
+    # addends: a 256 x 256 tile copies them row-wise (16 bytes per lane) into the staging area ...
+    if fm * fm * 2 > 80 and addends:
+        nt_, cprw_ = NW * 64, tile // 8
+        assert tile * cprw_ % (nt_ * 8) == 0   # batches of 8 chunks per thread
+        for it in range(tile * cprw_ // nt_):
+            c = np.arange(nt_) + it * nt_
+            row, c8 = c // cprw_, c % cprw_
+            gr, gc = m0 + row, n0 + c8 * 8
+            on = (gr < M) & (gc < M) if guard else np.ones(nt_, bool)
+            cmat.check(gr[on], gc[on], 8, "addend copy")
+            assert ((row * ldt + c8 * 8) * 2 + 16 <= tile * ldt * 2).all()
+    # ... smaller tiles read them in accumulator layout
     for wave in range(NW):
         wm, wn = wave % wgm, wave // wgm
         for i in range(fm):

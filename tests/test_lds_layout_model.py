@@ -275,7 +275,7 @@ def syrk_epilogue_model(tile, mi, npass, diag, skip_upper=False):
     return out, (m0, n0)
 
 
-@pytest.mark.parametrize("tile,mi,npass", [(192, 16, 1), (256, 16, 2), (128, 16, 1)])
+@pytest.mark.parametrize("tile,mi,npass", [(192, 16, 1), (256, 16, 1), (128, 16, 1)])
 @pytest.mark.parametrize("diag", [False, True])
 def test_syrk_epilogue_writes_the_tile_and_its_mirror_image(tile, mi, npass, diag):
     out, (m0, n0) = syrk_epilogue_model(tile, mi, npass, diag)
@@ -290,13 +290,13 @@ def test_syrk_epilogue_writes_the_tile_and_its_mirror_image(tile, mi, npass, dia
     assert out == expect
 
 
-@pytest.mark.parametrize("tile,npass", [(192, 1), (256, 2)])
+@pytest.mark.parametrize("tile,npass", [(192, 1), (256, 1)])
 def test_syrk_epilogue_lower_only(tile, npass):
     out, (m0, n0) = syrk_epilogue_model(tile, 16, npass, diag=False, skip_upper=True)
     assert out == {(m0 + a, n0 + b): ("v", a, b) for a in range(tile) for b in range(tile)}
 
 
-@pytest.mark.parametrize("tile,npass", [(192, 1), (256, 2), (128, 1)])
+@pytest.mark.parametrize("tile,npass", [(192, 1), (256, 1), (128, 1)])
 def test_syrk_epilogue_lower_only_on_a_diagonal_tile(tile, npass):
     """With the upper triangle skipped, a diagonal tile stores its two diagonal blocks whole and the block below them;
     the block above the diagonal (whose wavefront computes nothing) must stay unwritten."""
