@@ -305,25 +305,43 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
     p.q_bs = x_bs;
     p.M = (int)m;
     p.N = (int)n;
-    // Tile-count quantisation: T full 256 x 256 tiles over C compute units leave a last round that is at
-    // most half full when 0 < T mod C <= C/2.  If that remainder is a whole number of tile columns, those
-    // columns are computed as 256 x 128 tiles instead (twice as many workgroups, one short round).
-    if (batch == 1 && m % 256 == 0 && n % 256 == 0 && m >= 1024 && n >= 1024 && m % 64 == 0) {
+    // Tile-count quantisation: T full 256 x 256 tiles over C compute units leave a last round that is at most half
+    // full when 0 < T mod C <= C/2.  If that remainder is a whole number of tile columns or of tile rows (of every
+    // matrix of the batch), those run as 256 x 128 tiles in a second launch: twice as many workgroups, one short round
+    // (4096 x 14336: 768 + 256 workgroups instead of 896; 8 x 1792 x 4096: the last tile row of every matrix).
+    if (m % 256 == 0 && n % 256 == 0 && m >= 1024 && n >= 1024 && !gemm_prefers_half_tiles(m, n, batch)) {
       const int64_t tm = m / 256, tn = n / 256, cus = num_cus();
-      const int64_t rem = (tm * tn) % cus;
-      if (rem > 0 && rem * 2 <= cus && rem % tm == 0 && tn > rem / tm) {
-        const int64_t tail_cols = (rem / tm) * 256, main_cols = n - tail_cols;
-        const int tiles_main = (int)(tm * (main_cols / 256)), tiles_tail = (int)(tm * (tail_cols / 128));
+      const int64_t rem = (tm * tn * batch) % cus;
+      int64_t tail_cols = 0, tail_rows = 0;
+      if (rem > 0 && rem * 2 <= cus) {
+        if (rem % (tm * batch) == 0 && rem / (tm * batch) < tn) tail_cols = rem / (tm * batch) * 256;
+        else if (rem % (tn * batch) == 0 && rem / (tn * batch) < tm) tail_rows = rem / (tn * batch) * 256;
+      }
+      if (tail_cols > 0 || tail_rows > 0) {
+        const int64_t main_cols = n - tail_cols, main_rows = m - tail_rows;
+        // per matrix: workgroups of the main launch, then those of the tail launch
+        const int tiles_main = (int)((main_rows / 256) * (main_cols / 256));
+        const int tiles_tail = (int)(tail_cols ? tm * (tail_cols / 128) : (tail_rows / 256) * (n / 128));
         GemmParams pm = p, pt = p;
-        pm.N = (int)main_cols;
         pm.slot_stride = pt.slot_stride = tiles_main + tiles_tail;
         pm.slot_base = 0;
         pt.slot_base = tiles_main;
-        pt.N = (int)tail_cols;
-        pt.Q = p.Q + main_cols;  // K-strided operand: column offset
-        if (pt.Cin) pt.Cin = p.Cin + main_cols;
-        pt.Out = out_fp32 ? static_cast<void*>(static_cast<float*>(p.Out) + main_cols)
-                          : static_cast<void*>(static_cast<uint16_t*>(p.Out) + main_cols);
+        int64_t out_off = 0;
+        if (tail_cols) {
+          pm.N = (int)main_cols;
+          pt.N = (int)tail_cols;
+          pt.Q = p.Q + main_cols;  // K-strided operand: column offset
+          if (pt.Cin) pt.Cin = p.Cin + main_cols;
+          out_off = main_cols;
+        } else {
+          pm.M = (int)main_rows;
+          pt.M = (int)tail_rows;
+          pt.P = p.P + main_rows * p.ldp;
+          if (pt.Cin) pt.Cin = p.Cin + main_rows * p.ldc;
+          out_off = main_rows * p.ldo;
+        }
+        pt.Out = out_fp32 ? static_cast<void*>(static_cast<float*>(p.Out) + out_off)
+                          : static_cast<void*>(static_cast<uint16_t*>(p.Out) + out_off);
         int rc = out_fp32 ? launch_fast<CfgBig, false, true, MODE_GEMM, true>(pm, batch, stream)
                           : launch_fast<CfgBig, false, true, MODE_GEMM, false>(pm, batch, stream);
         if (rc != MI_OK) return rc;

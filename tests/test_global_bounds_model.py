@@ -437,6 +437,41 @@ def test_tail_split_of_the_wide_gemm():
         assert base + grid <= tiles_main + tiles_tail
 
 
+def test_tail_split_by_rows_of_a_batched_gemm():
+    """8 x (1792 x 4096) on 256 CUs: 896 tiles of 256 x 256 leave half a round, which is the last tile row of every
+    matrix; it runs as 256 x 128 tiles on pointers advanced by `main_rows` rows.  Every access of both launches must stay
+    inside the matrices of its batch entry."""
+    m, n, batch, cus = 1792, 4096, 8, 256
+    tm, tn = m // 256, n // 256
+    rem = (tm * tn * batch) % cus
+    assert rem == 128 and rem % (tm * batch) != 0 and rem % (tn * batch) == 0
+    tail_rows = rem // (tn * batch) * 256
+    main_rows = m - tail_rows
+    tiles_main, tiles_tail = (main_rows // 256) * tn, (tail_rows // 256) * (n // 128)
+    assert (tiles_main * batch) % cus == 0 and (tiles_main, tiles_tail) == (96, 32)
+    nk = m // BK
+    for cfg, rows, row_off in (("CfgBig", main_rows, 0), ("CfgHalfN", tail_rows, main_rows)):
+        tile_m, tile_n = CFGS[cfg][:2]
+        res = launch_fast(cfg, False, True, "gemm", rows, n, m)
+        assert res[0] == "ok" and not res[1]
+        _, _, tiles_m, tiles_n, grid = res
+        assert grid == (tiles_main if cfg == "CfgBig" else tiles_tail)
+        bfull, xfull = Matrix("B", m, m), Matrix("X", m, n)
+        for pid in sample(range(grid), 12):
+            tm_, tn_ = gemm_tile_of(pid, tiles_m, tiles_n)
+            m0, n0 = tm_ * tile_m, tn_ * tile_n
+            for kt in (0, nk - 1):
+                for wave in range(NW):
+                    r, k = loader_accesses(tile_m, False, False, m0, rows, kt, wave)
+                    bfull.check(r + row_off, k, 8, "B")          # P starts `row_off` rows into B
+                    r, k = loader_accesses(tile_n, True, False, n0, n, kt, wave)
+                    xfull.check(k, r, 8, "X")
+            # Cin and Out are X and X' advanced by the same rows
+            gemm_epilogue_accesses(cfg, rows, n, m0, n0, Matrix("Cin", m - row_off, n), Matrix("OUT", m - row_off, n))
+        base = 0 if cfg == "CfgBig" else tiles_main
+        assert base + grid <= tiles_main + tiles_tail
+
+
 @pytest.mark.parametrize("batch,m,n", [(32, 128, 4096), (2, 256, 1536), (4, 128, 1024), (1, 256, 1024)])
 def test_split_k_gram_partials(batch, m, n):
     """Short, wide matrices: K slices of 512 columns run as extra batch entries of a 128 x 128-tile product whose

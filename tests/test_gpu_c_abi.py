@@ -143,6 +143,24 @@ def test_gemm_axpy_tail_split_integer_exact(gpu):
         assert torch.equal(got, ref.to(out_dtype))
 
 
+def test_gemm_axpy_batched_tail_split_integer_exact(gpu):
+    """8 x (1792 x 4096): 896 tiles of 256 x 256 are 3.5 rounds of 256 CUs; the last tile row of every matrix runs as
+    256 x 128 tiles in a second launch (96 + 32 workgroups per matrix)."""
+    b, m, n = 8, 1792, 4096
+    x = _int_bf16((b, m, n), -2, 3, gpu, seed=5)
+    bm = _int_bf16((b, m, m), -2, 3, gpu, seed=6)
+    ref = 0.5 * x.float() + 0.25 * torch.bmm(bm.float(), x.float())
+    for out_dtype in (BF, torch.float32):
+        got = hip_kernels.gemm_axpy(bm, x, alpha=0.25, beta=0.5, out_dtype=out_dtype)
+        info = _hip.last_launch()
+        if torch.cuda.get_device_properties(0).multi_processor_count == 256:
+            assert (info["tiles"], info["tile_m"], info["tile_n"]) == (96 + 32, 256, 128), info
+        assert torch.equal(got, ref.to(out_dtype))
+    want = O.gemm_axpy(bm[7].float().cpu().numpy(), x[7].float().cpu().numpy(), 0.25, 0.5)
+    got = hip_kernels.gemm_axpy(bm, x, alpha=0.25, beta=0.5)
+    assert np.array_equal(got[7].float().cpu().numpy(), want)
+
+
 # n, k, transposed operand, expected tile
 SYRK_VARIANTS = [
     (1024, 512, False, 128), (1024, 512, True, 128), (1280, 192, True, 128), (4096, 1024, False, 192),
