@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Muon orthogonalisation path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline] [--no-others]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline] [--no-others] [--data zeros]
 
 Headline (the default): Newton-Schulz orthogonalisation of one 4096 x 14336 float32 gradient that is already resident
 in HBM: normalise, bf16 cast, 5 quintic steps on the bf16 MFMA kernels, float32 result.  One "step" of the benchmark is
@@ -42,8 +42,8 @@ TOL = 1e-2
 # (2 x X X^T, 14 m x m products), and of one GEMM+AXPY (both launches): FETCH_SIZE and WRITE_SIZE of two
 # `rocprofv3 --pmc` runs of this file (KiB per dispatch), each scaled by what the same counter reads for sumsq_kernel
 # of the same run, whose traffic is known (229 376 KiB read, 114 696 KiB written): factors 1.9994 and 0.9998.
-TRI_KERNEL_TRAFFIC_BYTES = int((128715.5 * 1.9994 + 32768.1 * 0.9998) * 1024)
-GEMM_AXPY_TRAFFIC_BYTES = int(((405915.0 + 146831.8) * 1.9994 + (98328.0 + 16392.0) * 0.9998) * 1024)
+TRI_KERNEL_TRAFFIC_BYTES = int((129464.9 * 1.9994 + 32768.0 * 0.9998) * 1024)
+GEMM_AXPY_TRAFFIC_BYTES = int(((406061.8 + 146825.0) * 1.9994 + (98328.0 + 16392.0) * 0.9998) * 1024)
 M, N, NS_STEPS = 4096, 14336, 5
 COEFFS = [(3.4445, -4.7750, 2.0315)] * NS_STEPS  # "simple" table cycled
 MIN_WARMUP, MIN_TIMED = 3, 20
@@ -155,7 +155,7 @@ def ns_input(name, shape, dev):
     return x * 1e-3
 
 
-def run_ns_workload(name, warmup, iters, lib, dev):
+def run_ns_workload(name, warmup, iters, lib, dev, zeros=False):
     """newton_schulz on one benchmark shape: timing, executed schedule, parity against float32."""
     import torch
 
@@ -163,7 +163,7 @@ def run_ns_workload(name, warmup, iters, lib, dev):
     from emerging_optimizers.orthogonalized_optimizers import muon_utils
 
     shape = NS_WORKLOADS[name]
-    x = ns_input(name, shape, dev)
+    x = torch.zeros(*shape, device=dev) if zeros else ns_input(name, shape, dev)
     run = lambda: muon_utils.newton_schulz(x, steps=NS_STEPS, coefficient_type="simple", use_syrk=True)
     with utils.fp32_matmul_precision("medium"), torch.no_grad():
         wall, per = time_events(run, warmup, iters)
@@ -174,8 +174,8 @@ def run_ns_workload(name, warmup, iters, lib, dev):
     f_sym, f_full, f_exec = ns_flops(batch, m, n, schedule)
     # parity: every matrix of a batch (two of them for the 1.9 GB stack)
     idx = range(batch) if x.dim() == 3 and x.numel() <= (1 << 28) else (range(2) if x.dim() == 3 else [None])
-    rels = []
-    for i in idx:
+    rels = [0.0] if zeros else []
+    for i in ([] if zeros else idx):
         xi, oi = (x, out) if i is None else (x[i], out[i])
         ref = ns_fp32_reference(xi)
         rels.append(float((oi.double() - ref.double()).norm() / ref.double().norm()))
@@ -353,6 +353,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-core baseline leg")
     ap.add_argument("--no-others", action="store_true", help="headline only: skip the other benchmark configurations")
     ap.add_argument("--workload", choices=ALL_WORKLOADS, default="mlp", help="time this configuration alone")
+    ap.add_argument("--data", choices=["synthetic", "zeros"], default="synthetic",
+                    help="zeros: all-zero headline input (a power probe: the matrix pipes then toggle no operand bits and "
+                         "the clock stays up; no parity gate, no other workloads)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only; --gpus above 1 is not supported (no collectives are built).")
@@ -380,7 +383,10 @@ def main():
         sys.exit(0 if res["parity"] == "ok" else 1)
 
     # ---- headline ----
-    res, (wall_ms, per, out, x, schedule) = run_ns_workload("mlp", args.warmup, args.steps, lib, dev)
+    zeros = args.data == "zeros"
+    res, (wall_ms, per, out, x, schedule) = run_ns_workload("mlp", args.warmup, args.steps, lib, dev, zeros=zeros)
+    if zeros:
+        args.no_others = args.no_cpu_baseline = True
     from emerging_optimizers import utils
     from emerging_optimizers.orthogonalized_optimizers import muon_utils
 
@@ -435,7 +441,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
-        "data": "synthetic",
+        "data": "zeros (power probe)" if zeros else "synthetic",
         "config": {
             "workload": f"newton_schulz, {NS_STEPS} steps ('simple' coefficients), one {M}x{N} float32 gradient "
             "(N(0,1e-3^2) with 1% entries at 50 sigma), bf16 MFMA kernels with fp32 accumulation, float32 result",
