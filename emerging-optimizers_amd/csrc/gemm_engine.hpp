@@ -62,6 +62,15 @@ struct GemmParams {
   float* slots_out;          // GEMM mode: per-workgroup sum of squares of the output,
   int slot_stride, slot_base;  //   at slots_out[batch * slot_stride + slot_base + blockIdx.x]
   int slot_capacity;         // host side only: floats reserved per batch entry behind slots_out (0: not checked)
+  // Lower-triangle launches of the fast kernel number their tiles through the whole batch (tile = batch entry *
+  // tiles per matrix + position in the blocked triangular order) on a one-dimensional grid: tiles [0, lin_tiles) in
+  // rounds of lin_g workgroups (what the chip holds at once, a multiple of 8), the rest in a last, partial round
+  // shared evenly between the XCDs.  Filled in by the launcher.
+  int lin_tiles, lin_g;
+  // Split-tail launches (see gemm_fast_kernel): the sk_rem tiles from lin_tiles on are split along K between
+  // sk_splits workgroups each, sk_tpx left-over tiles per XCD; one float32 accumulator image per (split, tile).
+  int sk_rem, sk_splits, sk_tpx;
+  float* sk_partials;
 };
 
 // Consecutive steps can share one Gram matrix, because every factor involved is a polynomial of it and they all
@@ -262,14 +271,14 @@ struct Scalars {
   float shift, alpha, beta, beta2;
 };
 template <int NT>
-__device__ __forceinline__ Scalars resolve_shift(const GemmParams& p, int64_t batch, float* red) {
+__device__ __forceinline__ Scalars resolve_shift(const GemmParams& p, int64_t batch, float* red, bool first_of_batch) {
   float s = 0.0f, alpha = p.alpha, beta = p.beta, beta2 = p.beta2;
   if (p.shift_mode == SHIFT_GRAM) {
     float part = 0.0f;
     const float* sl = p.slots_in + batch * p.nslots_in;
     for (int i = threadIdx.x; i < p.nslots_in; i += NT) part += sl[i];
     s = block_sum_f32<NT>(part, red) / (float)p.M;
-    if (blockIdx.x == 0 && threadIdx.x == 0) p.shift_io[batch] = s;
+    if (first_of_batch && threadIdx.x == 0) p.shift_io[batch] = s;
   } else if (p.shift_mode == SHIFT_POLY) {
     s = p.shift_io[batch];
     beta = beta + 2.0f * p.cc * s;  // B' = c A'^2 + (b + 2 c s) A'
@@ -506,7 +515,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_bf16_kernel(GemmParams p) 
     __syncthreads();
   }
 
-  const Scalars sc = resolve_shift<NT>(p, batch, red);
+  const Scalars sc = resolve_shift<NT>(p, batch, red, blockIdx.x == 0);
   const bool diag = (MODE == MODE_SYRK) && (tm == tn);
   tile_epilogue<MODE, OUT_F32, true, FM, FN, NT>(p, acc, m0 + wm * TM, n0 + wn * TN, lane, batch, diag, sc.alpha, sc.beta,
                                                  sc.shift, red, sc.beta2);

@@ -218,7 +218,13 @@ __device__ __forceinline__ bf16x8_t fast_frag16_ks(uint32_t tile_lds, uint32_t S
 __device__ __forceinline__ void mfma16_inplace(f32x4_t& c, const bf16x8_t& a, const bf16x8_t& b) {
   asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
-__device__ __forceinline__ void mfma_drain() { asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory"); }
+// (The scheduling barriers keep the compiler from moving a register copy of an accumulator, which is no memory
+// access and so not ordered by the clobber, from behind the wait states to in front of them.)
+__device__ __forceinline__ void mfma_drain() {
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
 
 // Workgroup id -> GEMM tile.  Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its
 // own L2, so id % 8 names the XCD and id / 8 the position in that XCD's queue.  Each XCD gets a contiguous
@@ -607,7 +613,29 @@ constexpr int waitcnt_imm(int vmcnt, int lgkmcnt) {
   return (vmcnt & 15) | ((vmcnt >> 4) << 14) | 0x70 | ((lgkmcnt & 15) << 8);
 }
 
-template <class C, bool P_KS, bool Q_KS, int MODE, bool OUT_F32, bool EDGE>
+// Lower-triangle launches number their tiles through the whole batch on a one-dimensional grid (GemmParams::lin_*):
+// consecutive workgroup ids go round-robin to the 8 XCDs, so within a round of lin_g workgroups XCD x takes the
+// lin_g / 8 consecutive tiles from x lin_g / 8 on, and of the `rest` tiles of the last, partial round the tiles
+// [rest x / 8, rest (x + 1) / 8): the workgroups that share an L2 work on neighbouring tiles of (mostly) one
+// matrix, and every XCD gets the same number of tiles, give or take one, whatever the tile count of one matrix is.
+//
+// STREAMK != 0: the two extra launches of a split-tail product (lower-triangle products of K-contiguous operands
+// whose tiles do not fill whole rounds of the chip; 256 x 256 tiles).  The whole rounds, tiles [0, lin_tiles), go out
+// as an ordinary launch.  Then
+//   SK_PARTS   the sk_rem tiles left over, fewer than half a round, are split along K between sk_splits >= 2
+//              workgroups each (XCD x takes the left-over tiles [x sk_tpx, (x + 1) sk_tpx)); a workgroup multiplies
+//              its part of the K range and parks its float32 accumulators in global memory (accumulator layout of
+//              the 256 x 256 tile, lane-linear), nothing else.
+//   SK_FINISH  a kernel of 128 x 128 tiles without a K loop: four workgroups per left-over tile, one per 128 x 128
+//              quarter (what one wavefront of SK_PARTS accumulated), add the parked accumulators in split order
+//              and run the ordinary epilogue of a 128 x 128 tile.
+// The launches follow each other on one stream; no workgroup ever waits for another one.  (Separate kernels and not
+// one with several roles: a 256 x 256 tile leaves no register to spare, and a kernel that spills to scratch memory
+// was measured 40 % slower on whole tiles.)
+constexpr int SK_TILE = 256, SK_NT = 256, SK_FN = 8;                       // the tile, threads and fragment columns of SK_PARTS
+constexpr int64_t SK_IMAGE_FLOATS = (int64_t)SK_TILE * SK_TILE;            // one accumulator image
+enum { SK_NONE = 0, SK_FINISH = 2, SK_PARTS = 3 };
+template <class C, bool P_KS, bool Q_KS, int MODE, bool OUT_F32, bool EDGE, int STREAMK = 0>
 __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   constexpr int NS = C::NS, FM = C::FM, FN = C::FN, P_BYTES = C::P_BYTES, NT = C::NT;
   // The ring of operand slots; every LDS access of the K loop names its slot statically (ring[u] is a constant
@@ -623,16 +651,48 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: everything derived from it stays in SGPRs
   const int wm = wave % C::WGM, wn = wave / C::WGM;
-  const int64_t batch = blockIdx.y;
+  static_assert(!STREAMK || (MODE == MODE_SYRK && !P_KS && !Q_KS && !EDGE && !OUT_F32 && C::NW == 4), "stream-K variant");
+  static_assert(!STREAMK || (STREAMK == SK_FINISH ? (C::TILE_M == 128 && C::WGM == 2) : (C::TILE_M == SK_TILE && C::NT == SK_NT && C::FN == SK_FN)),
+                "SK_PARTS on 256 x 256 tiles, SK_FINISH on their 128 x 128 quarters");
+  int64_t batch = blockIdx.y;
   int tm, tn;
-  if (MODE == MODE_SYRK) {
-    // The grid is padded to a multiple of 8 workgroups: id % 8 names the XCD (round-robin dispatch), and
-    // each XCD takes one contiguous chunk of the blocked triangular enumeration.
-    const int total = p.tiles_m * (p.tiles_m + 1) / 2;
-    const int per_xcd = (int)gridDim.x / 8;
-    const int s = ((int)blockIdx.x % 8) * per_xcd + (int)blockIdx.x / 8;
-    if (s >= total) return;  // padding workgroup (whole workgroup leaves before any barrier)
-    tri_block_decode(s, p.tiles_m, tm, tn);
+  int k_first = 0, nk = p.K / C::BK;  // K tiles of this pass: [k_first, k_first + nk)
+  int sk_tile = 0, sk_split = 0;  // left-over tile and K split of this workgroup (SK_PARTS); tile and quarter (SK_FINISH)
+  if constexpr (MODE == MODE_SYRK) {
+    const int tri = p.tiles_m * (p.tiles_m + 1) / 2, bid = (int)blockIdx.x;
+    int tile;
+    if constexpr (STREAMK == SK_NONE) {
+      const int g = p.lin_g, full = p.lin_tiles / g * g;
+      if (bid < full) {
+        tile = bid / g * g + (bid % 8) * (g / 8) + (bid % g) / 8;
+      } else {
+        const int j = bid - full, rest = p.lin_tiles - full, lo = rest * (j % 8) / 8, hi = rest * (j % 8 + 1) / 8;
+        if (j / 8 >= hi - lo) return;  // padding workgroup (leaves before any barrier)
+        tile = full + lo + j / 8;
+      }
+    } else {
+      if constexpr (STREAMK == SK_PARTS) {
+        const int nk_full = p.K / C::BK;
+        sk_tile = (bid % 8) * p.sk_tpx + (bid / 8) % p.sk_tpx;
+        sk_split = (bid / 8) / p.sk_tpx;
+        if (sk_tile >= p.sk_rem || sk_split >= p.sk_splits) return;  // padding workgroup
+        k_first = nk_full * sk_split / p.sk_splits;
+        nk = nk_full * (sk_split + 1) / p.sk_splits - k_first;
+      } else {
+        sk_tile = bid / 4;
+        sk_split = bid % 4;  // (the quarter: row half + 2 * column half = the wavefront of SK_PARTS that computed it)
+        if (sk_tile >= p.sk_rem) return;
+      }
+      tile = p.lin_tiles + sk_tile;
+    }
+    batch = tile / tri;
+    tri_block_decode(tile % tri, p.tiles_m, tm, tn);  // (for SK_FINISH, p.tiles_m counts 256 x 256 tiles)
+    if constexpr (STREAMK == SK_FINISH) {
+      const int qm = sk_split % 2, qn = sk_split / 2;
+      if (tm == tn && qn > qm) return;  // the quarter above the diagonal of a diagonal tile: written as a mirror image
+      tm = 2 * tm + qm;
+      tn = 2 * tn + qn;
+    }
   } else {
     gemm_tile_of((int)blockIdx.x, p.tiles_m, p.tiles_n, tm, tn);
   }
@@ -646,8 +706,12 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
     p_off = outer * p.p_bs + inner * p.p_bs2;
     q_off = outer * p.q_bs + inner * p.q_bs2;
   }
-  lp.init(p.P + p_off, p.ldp, m0, p.M, wave, lane);
-  lq.init(p.Q + q_off, p.ldq, n0, p.N, wave, lane);
+  // A wavefront none of whose outputs is ever stored (its rows or columns lie beyond the matrix, or its block is
+  // strictly above the diagonal of a diagonal SYRK tile) keeps loading its share of the operand tiles and keeps
+  // every barrier, but issues no fragment reads and no MFMAs: on this part the clock follows the power drawn,
+  // so work that is thrown away slows down the work that is kept.
+  const bool idle_wave = (m0 + wm * C::TM >= p.M) || (n0 + wn * C::TN >= p.N) ||
+                         (MODE == MODE_SYRK && tm == tn && wn * C::TN >= (wm + 1) * C::TM);
 
   constexpr int MI = C::MI, ACC_N = 4;
   f32x4_t acc[FM][FN];
@@ -658,7 +722,6 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
 #pragma unroll
       for (int e = 0; e < ACC_N; ++e) acc[i][j][e] = 0.0f;
 
-  const int nk = p.K / C::BK;
   constexpr int NQ = C::BK / C::KI;  // k-steps of one tile
   constexpr int LOADS_PER_TILE = C::LPT_P + C::LPT_Q;  // per thread, both operands
   static_assert(NQ % 2 == 0, "fragment buffer parity assumes an even number of k-steps per tile");
@@ -785,66 +848,102 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   };
   static_assert(NQ <= 4, "k_tile spells out at most three k-steps before the barrier");
 
-  // prologue: tiles 0 .. NS-2 and part 0 of tile NS-1 in flight, wait for tile 0
-#pragma unroll
-  for (int t = 0; t < NS - 1; ++t)
-    if (t < nk) issue_parts(t, 0, PARTS);
-  if (NS - 1 < nk) issue_parts(NS - 1, 0, 1);
-  if (nk >= NS)
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm((NS - 2) * LOADS_PER_TILE + PL, 15));
-  else
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
-  __syncthreads();
   constexpr bool CIN_EARLY = SYRK_STAGED && SyrkStage<C>::CIN_EARLY;
   uint2 cin_pre[CIN_EARLY ? SyrkStage<C>::NQUAD : 1];
-  if constexpr (CIN_EARLY) {
-    // these loads are older than every direct-to-LDS load issued from here on, so the vmcnt waits of the K
-    // loop cover them as well
-    if (p.Cin != nullptr)
-      syrk_addend_fetch<C, EDGE>(p, p.Cin + batch * p.c_bs, lane, m0 + wm * C::TM, n0 + wn * C::TN, cin_pre);
-  }
-  // A wavefront none of whose outputs is ever stored (its rows or columns lie beyond the matrix, or its block is
-  // strictly above the diagonal of a diagonal SYRK tile) keeps loading its share of the operand tiles and keeps
-  // every barrier, but issues no fragment reads and no MFMAs: on this part the clock follows the power drawn,
-  // so work that is thrown away slows down the work that is kept.
-  const bool idle_wave = (m0 + wm * C::TM >= p.M) || (n0 + wn * C::TN >= p.N) ||
-                         (MODE == MODE_SYRK && tm == tn && wn * C::TN >= (wm + 1) * C::TM);
-  if (idle_wave) {
-    for (int kt = 0; kt < nk; ++kt) {
-      const int cur_slot = kt % NS, prev_slot = (cur_slot + NS - 1) % NS;
-      if (PARTS > 1 && kt + NS - 1 < nk) issue_parts(prev_slot, 1, PARTS);
-      __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
-      __syncthreads();
-      if (kt + NS < nk) issue_parts(cur_slot, 0, 1);
-    }
-  } else {
-    fetch(ring[0], 0, 0);
-    int kt = 0;
-    for (; kt + 2 * NS - 1 < nk; kt += NS) {  // every tile of this round is a steady one
+  if constexpr (STREAMK != SK_FINISH) {
+    lp.init(p.P + p_off + (STREAMK ? (int64_t)k_first * C::BK : 0), p.ldp, m0, p.M, wave, lane);
+    lq.init(p.Q + q_off + (STREAMK ? (int64_t)k_first * C::BK : 0), p.ldq, n0, p.N, wave, lane);
+    // prologue: tiles 0 .. NS-2 and part 0 of tile NS-1 in flight, wait for tile 0
 #pragma unroll
-      for (int u = 0; u < NS; ++u) k_tile(std::true_type{}, kt + u, u, ring[u], ring[(u + 1) % NS]);
+    for (int t = 0; t < NS - 1; ++t)
+      if (t < nk) issue_parts(t, 0, PARTS);
+    if (NS - 1 < nk) issue_parts(NS - 1, 0, 1);
+    if (nk >= NS)
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm((NS - 2) * LOADS_PER_TILE + PL, 15));
+    else
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+    __syncthreads();
+    if constexpr (CIN_EARLY) {
+      // these loads are older than every direct-to-LDS load issued from here on, so the vmcnt waits of the K
+      // loop cover them as well
+      if (p.Cin != nullptr)
+        syrk_addend_fetch<C, EDGE>(p, p.Cin + batch * p.c_bs, lane, m0 + wm * C::TM, n0 + wn * C::TN, cin_pre);
     }
-    for (; kt < nk; kt += NS) {
+    if (idle_wave) {
+      for (int kt = 0; kt < nk; ++kt) {
+        const int cur_slot = kt % NS, prev_slot = (cur_slot + NS - 1) % NS;
+        if (PARTS > 1 && kt + NS - 1 < nk) issue_parts(prev_slot, 1, PARTS);
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+        __syncthreads();
+        if (kt + NS < nk) issue_parts(cur_slot, 0, 1);
+      }
+    } else {
+      fetch(ring[0], 0, 0);
+      int kt = 0;
+      for (; kt + 2 * NS - 1 < nk; kt += NS) {  // every tile of this round is a steady one
 #pragma unroll
-      for (int u = 0; u < NS; ++u)
-        if (kt + u < nk) k_tile(std::false_type{}, kt + u, u, ring[u], ring[(u + 1) % NS]);
+        for (int u = 0; u < NS; ++u) k_tile(std::true_type{}, kt + u, u, ring[u], ring[(u + 1) % NS]);
+      }
+      for (; kt < nk; kt += NS) {
+#pragma unroll
+        for (int u = 0; u < NS; ++u)
+          if (kt + u < nk) k_tile(std::false_type{}, kt + u, u, ring[u], ring[(u + 1) % NS]);
+      }
+    }
+    mfma_drain();
+  }
+  // Scalars, then the write-out of the finished accumulators.
+  auto finish = [&]() __attribute__((always_inline)) {
+    const Scalars sc = resolve_shift<NT>(p, batch, red, MODE == MODE_SYRK ? (tm == 0 && tn == 0) : blockIdx.x == 0);
+    const float alpha = sc.alpha, beta = sc.beta, beta2 = sc.beta2, shift = sc.shift;
+    const bool diag = (MODE == MODE_SYRK) && (tm == tn);
+    if constexpr (MODE == MODE_GEMM && (C::TN == 32 || C::TN == 64 || C::TN == 128)) {
+      __syncthreads();  // every wavefront has finished reading the ring: it can be reused as staging space
+      gemm_epilogue_lds<C, OUT_F32, EDGE>(p, acc, &ring[0][0], wave, lane, m0 + wm * C::TM, n0 + wn * C::TN, batch, alpha,
+                                          beta, red);
+    } else if constexpr (SYRK_STAGED) {
+      syrk_epilogue_lds<C, EDGE>(p, acc, &ring[0][0], lane, wm, wn, m0, n0, batch, diag, alpha, beta, beta2, shift, cin_pre);
+    } else {
+      tile_epilogue<MODE, OUT_F32, EDGE, FM, FN, NT, MI>(p, acc, m0 + wm * C::TM, n0 + wn * C::TN, lane, batch, diag, alpha, beta, shift,
+                                                         red, beta2);
+    }
+  };
+  if constexpr (STREAMK == SK_PARTS) {
+    // image of split s of left-over tile t: slot s sk_rem + t; quad (i, j) of thread t at ((i SK_FN + j) SK_NT + t) float4s
+    if (!idle_wave) {
+      f32x4_t* img = reinterpret_cast<f32x4_t*>(p.sk_partials + ((int64_t)sk_split * p.sk_rem + sk_tile) * SK_IMAGE_FLOATS) + tid;
+      static_for<FM>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+#pragma unroll
+        for (int j = 0; j < FN; ++j) img[(int64_t)(i * FN + j) * NT] = acc[i][j];
+        __builtin_amdgcn_sched_barrier(0);  // one fragment row at a time: the image must not pile up in registers
+      });
+    }
+    return;
+  }
+  if constexpr (STREAMK == SK_FINISH) {
+    if constexpr (CIN_EARLY) {
+      if (p.Cin != nullptr)
+        syrk_addend_fetch<C, EDGE>(p, p.Cin + batch * p.c_bs, lane, m0 + wm * C::TM, n0 + wn * C::TN, cin_pre);
+    }
+    if (!idle_wave) {
+      // this wavefront's 64 x 64 block inside the quarter = fragments (wm FM + i, wn FN + j) of wavefront sk_split of SK_PARTS
+      const f32x4_t* img = reinterpret_cast<const f32x4_t*>(p.sk_partials + (int64_t)sk_tile * SK_IMAGE_FLOATS) +
+                           ((wm * FM) * SK_FN + wn * FN) * SK_NT + sk_split * 64 + lane;
+      for (int s = 0; s < p.sk_splits; ++s) {
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+          for (int j = 0; j < FN; ++j) {
+            const f32x4_t v = img[(int64_t)(i * SK_FN + j) * SK_NT];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][j][e] += v[e];
+          }
+        img += (int64_t)p.sk_rem * (SK_IMAGE_FLOATS / 4);
+      }
     }
   }
-
-  mfma_drain();
-  const Scalars sc = resolve_shift<NT>(p, batch, red);
-  const float alpha = sc.alpha, beta = sc.beta, beta2 = sc.beta2, shift = sc.shift;
-  const bool diag = (MODE == MODE_SYRK) && (tm == tn);
-  if constexpr (MODE == MODE_GEMM && (C::TN == 32 || C::TN == 64 || C::TN == 128)) {
-    __syncthreads();  // every wavefront has finished reading the ring: it can be reused as staging space
-    gemm_epilogue_lds<C, OUT_F32, EDGE>(p, acc, &ring[0][0], wave, lane, m0 + wm * C::TM, n0 + wn * C::TN, batch, alpha,
-                                        beta, red);
-  } else if constexpr (SYRK_STAGED) {
-    syrk_epilogue_lds<C, EDGE>(p, acc, &ring[0][0], lane, wm, wn, m0, n0, batch, diag, alpha, beta, beta2, shift, cin_pre);
-  } else {
-    tile_epilogue<MODE, OUT_F32, EDGE, FM, FN, NT, MI>(p, acc, m0 + wm * C::TM, n0 + wn * C::TN, lane, batch, diag, alpha, beta, shift,
-                                                       red, beta2);
-  }
+  finish();
 }
 
 }  // namespace mi

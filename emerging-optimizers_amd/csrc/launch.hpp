@@ -25,7 +25,25 @@ int launch_one(const GemmParams& p, int64_t batch, hipStream_t stream);
 // Fast kernel (gemm_fast.hpp): K a multiple of the ring-slot depth; tiles that overhang the matrix only for the
 // lower-triangle product of K-contiguous operands; anything else is refused with MI_ERR_UNSUPPORTED_SHAPE before
 // a kernel is launched.
+// A lower-triangle launch computes the tiles [0, tile_limit) of the batch, in the order of the kernel's numbering
+// (tile_limit < 0: all of them).
 template <class C, bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
-int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream);
+int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream, int64_t tile_limit = -1);
+
+// CUs of the current device (cached).
+int device_cus();
+
+// Split-tail (stream-K) launch of the lower-triangle kernel (256 x 256 tiles, K-contiguous operands, bf16 output):
+// with `cus` CUs (a multiple of 8), the whole rounds of `cus` tiles run one tile per workgroup, and the K range of each
+// left-over tile is shared between `splits` workgroups (streamk_plan) that park their float32 accumulators in
+// `workspace` (streamk_workspace_bytes), all in one launch; a second launch, one workgroup per left-over tile, adds
+// the parked accumulators and writes the tile.
+constexpr int MAX_STREAMK_SPLITS = 8;
+struct StreamKPlan {
+  int rounds, rem, splits;  // whole rounds of `cus` tiles, tiles left over, workgroups per left-over tile (0 or >= 2)
+};
+StreamKPlan streamk_plan(int64_t tiles, int k_tiles, int cus);
+size_t streamk_workspace_bytes(const StreamKPlan& plan);
+int launch_streamk(const GemmParams& p, int64_t batch, int cus, void* workspace, size_t workspace_bytes, hipStream_t stream);
 
 }  // namespace mi

@@ -40,8 +40,17 @@ int launch_one(const GemmParams& p, int64_t batch, hipStream_t stream) {
   return MI_OK;
 }
 
+// Workgroups of configuration C that the chip holds at once, rounded down to a multiple of 8 (the XCDs): two per CU
+// when two rings fit the LDS of a CU, else one.
+template <class C>
+int fast_round_size() {
+  constexpr int per_cu = 2 * C::NS * C::SLOT_BYTES <= 160 * 1024 ? 2 : 1;
+  const int g = device_cus() * per_cu / 8 * 8;
+  return g >= 8 ? g : 8;
+}
+
 template <class C, bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
-int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream) {
+int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream, int64_t tile_limit) {
   // the K loop of the fast kernel has no tail, and its loaders trust these extents
   if (p.K < C::BK || p.K % C::BK != 0)
     return fail(MI_ERR_UNSUPPORTED_SHAPE, "internal: K = %d is not a multiple of %d", p.K, C::BK);
@@ -49,12 +58,26 @@ int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream) {
   GemmParams q = p;
   q.tiles_m = (p.M + C::TILE_M - 1) / C::TILE_M;
   q.tiles_n = (p.N + C::TILE_N - 1) / C::TILE_N;
-  int64_t tiles = (MODE == MODE_SYRK) ? (int64_t)q.tiles_m * (q.tiles_m + 1) / 2 : (int64_t)q.tiles_m * q.tiles_n;
-  if (MODE == MODE_SYRK) tiles = (tiles + 7) / 8 * 8;  // XCD-chunked enumeration: grid padded to a multiple of 8
-  if (batch > 65535) return fail(MI_ERR_UNSUPPORTED_SHAPE, "batch %lld exceeds the grid limit 65535", (long long)batch);
-  if (q.slot_stride == 0) q.slot_stride = (int)tiles;
-  if (int rc = check_slots(q, tiles)) return rc;
-  dim3 grid((unsigned)tiles, (unsigned)batch, 1), block(C::NT, 1, 1);
+  dim3 grid, block(C::NT, 1, 1);
+  int64_t tiles;
+  if constexpr (MODE == MODE_SYRK) {
+    // one-dimensional grid over the tiles of the whole batch: whole rounds, then a last round with the same number
+    // of tiles for every XCD
+    tiles = (int64_t)q.tiles_m * (q.tiles_m + 1) / 2 * batch;
+    if (tile_limit >= 0 && tile_limit < tiles) tiles = tile_limit;
+    if (tiles > (int64_t)1 << 30) return fail(MI_ERR_UNSUPPORTED_SHAPE, "%lld tiles exceed the grid limit", (long long)tiles);
+    if (tiles == 0) return MI_OK;
+    q.lin_tiles = (int)tiles;
+    q.lin_g = fast_round_size<C>();
+    const int full = q.lin_tiles / q.lin_g * q.lin_g;
+    grid = dim3((unsigned)(full + (q.lin_tiles - full + 7) / 8 * 8), 1, 1);
+  } else {
+    tiles = (int64_t)q.tiles_m * q.tiles_n;
+    if (batch > 65535) return fail(MI_ERR_UNSUPPORTED_SHAPE, "batch %lld exceeds the grid limit 65535", (long long)batch);
+    if (q.slot_stride == 0) q.slot_stride = (int)tiles;
+    if (int rc = check_slots(q, tiles)) return rc;
+    grid = dim3((unsigned)tiles, (unsigned)batch, 1);
+  }
   const bool edge = (p.M % C::TILE_M) != 0 || (p.N % C::TILE_N) != 0;
   // Only the lower-triangle product of K-contiguous operands has a variant for tiles that overhang the matrix
   // (rows clamped in the loaders, guarded epilogue).
@@ -67,7 +90,7 @@ int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream) {
   } else {
     hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, false>), grid, block, 0, stream, q);
   }
-  g_last_launch = LastLaunch{(int)tiles, C::TILE_M, C::TILE_N, 1};
+  g_last_launch = LastLaunch{(int)grid.x, C::TILE_M, C::TILE_N, 1};
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
   return MI_OK;

@@ -77,7 +77,7 @@ static TileClass pick_class(int64_t extent) {
 static int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Device-wide compute units (workgroups that run concurrently at one fast-kernel workgroup per CU).
-static int num_cus() {
+int device_cus() {
   static int cached = 0;
   if (!cached) {
     int dev = 0, n = 0;
@@ -107,8 +107,8 @@ static int num_cus() {
 enum SyrkTile { SYRK_TILE_NONE, SYRK_TILE_128, SYRK_TILE_128X2, SYRK_TILE_192, SYRK_TILE_256 };
 // `k_strided`: the operand is stored transposed; its LDS layout exists for 128- and 256-row tiles only, and not for
 // tiles that overhang the matrix, so there may be no fast tile at all.
-static SyrkTile pick_syrk_tile(int64_t n, int64_t batch, int64_t k, bool k_strided) {
-  const int64_t cus = num_cus();
+static SyrkTile pick_syrk_tile(int64_t n, int64_t batch, int64_t k, bool k_strided, double* cost_us = nullptr) {
+  const int64_t cus = device_cus();
   const double kt = (double)ceil_div(k, 64);
   auto tiles = [&](int64_t tile) {
     const int64_t t = ceil_div(n, tile);
@@ -133,11 +133,36 @@ static SyrkTile pick_syrk_tile(int64_t n, int64_t batch, int64_t k, bool k_strid
     offer(SYRK_TILE_128X2, (double)ceil_div(t128, 2 * cus) * (9.2 + s2 * kt));
     offer(SYRK_TILE_128, (double)ceil_div(t128, cus) * (9.0 + (t128 <= cus ? 0.31 : 0.44) * kt));
   }
+  if (cost_us) *cost_us = best_cost;
   return best;
+}
+
+// Split-tail (stream-K) launch of the lower-triangle kernel (256 x 256 tiles; whole rounds of tiles, then the
+// left-over tiles with their K range split between workgroups): true when the shape qualifies and the model
+// expects a gain over the best ordinary launch; `plan` is filled either way.  Modelled time: the whole rounds and the
+// split round at the cost of a 256 x 256 tile on a full chip, and the finishing launch (8 us, and 3 us per
+// accumulator image it adds; 20 us measured for 64 tiles of 4 images).
+static int streamk_cus() { return device_cus() / 8 * 8; }
+static bool streamk_wanted(int64_t n, int64_t batch, int64_t k, bool k_strided, StreamKPlan* plan) {
+  *plan = StreamKPlan{0, 0, 0};
+  const int cus = streamk_cus();
+  if (k_strided || n < 1024 || n % 256 != 0 || k % 64 != 0 || k < 64 || cus < 8) return false;
+  const char* env = getenv("MI_STREAMK");  // "0": never, "1": whenever the shape qualifies (tests), else by the model
+  if (env && env[0] == '0') return false;
+  const int64_t t = n / 256, tiles = t * (t + 1) / 2 * batch, kt = k / 64;
+  if (tiles / cus > 4096) return false;
+  *plan = streamk_plan(tiles, (int)kt, cus);
+  if (env && env[0] == '1') return true;
+  if (plan->splits < 2) return false;
+  double best = 0.0;
+  pick_syrk_tile(n, batch, k, false, &best);
+  const double sk = plan->rounds * (16.5 + 1.37 * kt) + 16.5 + 1.37 * (double)ceil_div(kt, plan->splits) + 8.0 +
+                    3.0 * plan->splits;
+  return sk < 0.97 * best;
 }
 // 256 x 128 instead of 256 x 256 GEMM tiles for the whole product?
 static bool gemm_prefers_half_tiles(int64_t m, int64_t n, int64_t batch) {
-  const int64_t cus = num_cus(), tiles = (m / 256) * (n / 256) * batch;
+  const int64_t cus = device_cus(), tiles = (m / 256) * (n / 256) * batch;
   return (double)ceil_div(2 * tiles, cus) * 0.5 * 1.27 < (double)ceil_div(tiles, cus);
 }
 
@@ -226,7 +251,8 @@ struct ShiftArgs {
 static int syrk_impl(const void* A, int64_t batch, int64_t n, int64_t k, int64_t a_bs, int64_t a_ld, int a_trans,
                      const void* C, int64_t c_bs, int64_t c_ld, float alpha, float beta, void* D, int64_t d_bs,
                      int64_t d_ld, int skip_upper, hipStream_t stream, const ShiftArgs* sh = nullptr,
-                     const void* other = nullptr, const void* C2 = nullptr) {
+                     const void* other = nullptr, const void* C2 = nullptr, void* workspace = nullptr,
+                     size_t workspace_bytes = 0) {
   if (!A || !D) return fail(MI_ERR_BAD_ARG, "mi_syrk_bf16: A and D must not be null");
   if (batch < 0 || n < 0 || k < 0) return fail(MI_ERR_BAD_ARG, "mi_syrk_bf16: negative extent");
   if (beta != 0.0f && !C) return fail(MI_ERR_BAD_ARG, "mi_syrk_bf16: C is null but beta != 0");
@@ -259,6 +285,15 @@ static int syrk_impl(const void* A, int64_t batch, int64_t n, int64_t k, int64_t
   p.out_scale = 1.0f;
   p.skip_upper = skip_upper ? 1 : 0;
   if (sh) sh->apply(p);
+  // With a workspace, shapes whose tiles fill the chip's rounds badly go out as a split-tail launch.
+  if (!skip_upper && sh == nullptr && C2 == nullptr) {
+    StreamKPlan plan;
+    if (streamk_wanted(n, batch, k, a_trans != 0, &plan)) {
+      const size_t need = streamk_workspace_bytes(plan);
+      if (need == 0 || (workspace != nullptr && workspace_bytes >= need && !(reinterpret_cast<uintptr_t>(workspace) & 255u)))
+        return launch_streamk(p, batch, streamk_cus(), workspace, workspace_bytes, stream);
+    }
+  }
   TileClass tc = pick_class(n);
   return a_trans ? launch_class<true, true, MODE_SYRK, false>(tc, p, batch, stream)
                  : launch_class<false, false, MODE_SYRK, false>(tc, p, batch, stream);
@@ -310,7 +345,7 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
     // matrix of the batch), those run as 256 x 128 tiles in a second launch: twice as many workgroups, one short round
     // (4096 x 14336: 768 + 256 workgroups instead of 896; 8 x 1792 x 4096: the last tile row of every matrix).
     if (m % 256 == 0 && n % 256 == 0 && m >= 1024 && n >= 1024 && !gemm_prefers_half_tiles(m, n, batch)) {
-      const int64_t tm = m / 256, tn = n / 256, cus = num_cus();
+      const int64_t tm = m / 256, tn = n / 256, cus = device_cus();
       const int64_t rem = (tm * tn * batch) % cus;
       int64_t tail_cols = 0, tail_rows = 0;
       if (rem > 0 && rem * 2 <= cus) {
@@ -1383,6 +1418,21 @@ int mi_syrk_bf16(const void* A, int64_t batch, int64_t n, int64_t k, int64_t a_b
                  int64_t d_batch_stride, int64_t d_ld, int skip_upper, void* stream) {
   return syrk_impl(A, batch, n, k, a_batch_stride, a_ld, a_trans, C, c_batch_stride, c_ld, alpha, beta, D,
                    d_batch_stride, d_ld, skip_upper, static_cast<hipStream_t>(stream));
+}
+
+size_t mi_syrk_workspace_bytes(int64_t batch, int64_t n, int64_t k, int a_trans) {
+  if (batch <= 0 || n <= 0 || k <= 0) return 0;
+  StreamKPlan plan;
+  return streamk_wanted(n, batch, k, a_trans != 0, &plan) ? streamk_workspace_bytes(plan) : 0;
+}
+
+int mi_syrk_bf16_ws(const void* A, int64_t batch, int64_t n, int64_t k, int64_t a_batch_stride, int64_t a_ld, int a_trans,
+                    const void* C, int64_t c_batch_stride, int64_t c_ld, float alpha, float beta, void* D,
+                    int64_t d_batch_stride, int64_t d_ld, int skip_upper, void* workspace, size_t workspace_bytes,
+                    void* stream) {
+  return syrk_impl(A, batch, n, k, a_batch_stride, a_ld, a_trans, C, c_batch_stride, c_ld, alpha, beta, D,
+                   d_batch_stride, d_ld, skip_upper, static_cast<hipStream_t>(stream), nullptr, nullptr, nullptr, workspace,
+                   workspace_bytes);
 }
 
 int mi_gemm_axpy_bf16(const void* Bm, int64_t b_batch_stride, int64_t b_ld, const void* X,

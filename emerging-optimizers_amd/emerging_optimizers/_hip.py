@@ -32,6 +32,12 @@ EXPORTS = (
     ("mi_version", _int, ()),
     ("mi_last_error", ctypes.c_char_p, ()),
     ("mi_syrk_bf16", _int, (_vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _i64, _i64, _f32, _f32, _vp, _i64, _i64, _int, _vp)),
+    ("mi_syrk_workspace_bytes", _sz, (_i64, _i64, _i64, _int)),
+    (
+        "mi_syrk_bf16_ws",
+        _int,
+        (_vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _i64, _i64, _f32, _f32, _vp, _i64, _i64, _int, _vp, _sz, _vp),
+    ),
     (
         "mi_gemm_axpy_bf16",
         _int,

@@ -75,21 +75,6 @@ def fused_supported(x: torch.Tensor) -> bool:
     )
 
 
-# One cached workspace per (device, stream): Newton-Schulz calls on one stream are serialised by the
-# stream itself, so they can share scratch; different streams get different buffers.
-_workspaces: dict[tuple[int, int], torch.Tensor] = {}
-
-
-def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    key = (device.index if device.index is not None else torch.cuda.current_device(),
-           torch.cuda.current_stream(device).cuda_stream)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(nbytes, device=device, dtype=torch.uint8)
-        _workspaces[key] = ws
-    return ws
-
-
 def fused_newton_schulz(
     x: torch.Tensor,
     coefficients: Sequence[tuple[float, float, float]],
@@ -114,7 +99,7 @@ def fused_newton_schulz(
     abc = (ctypes.c_float * max(1, len(flat)))(*flat)
     with torch.cuda.device(x.device):
         nbytes = lib.mi_newton_schulz_workspace_bytes(batch, rows, cols)
-        ws = _workspace(x.device, nbytes)
+        ws = _launch.workspace(x.device, nbytes)
         rc = lib.mi_newton_schulz_bf16(
             _launch.ptr(xc), _launch.ptr(out), batch, rows, cols, abc, steps, float(eps),
             int(bool(normalize_in_double)), float(out_scale), _launch.ptr(ws), ws.numel(),
@@ -158,7 +143,7 @@ def fused_muon_update(
     abc = (ctypes.c_float * len(flat))(*flat)
     with torch.cuda.device(param.device):
         nbytes = lib.mi_newton_schulz_workspace_bytes(batch, rows, cols)
-        ws = _workspace(param.device, nbytes)
+        ws = _launch.workspace(param.device, nbytes)
         rc = lib.mi_muon_update_bf16(
             _launch.ptr(param), _launch.ptr(grad), _launch.ptr(momentum_buffer), batch, rows, cols,
             float(beta), int(bool(nesterov)), float(param_decay), float(update_scale), abc, len(coefficients),

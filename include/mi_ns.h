@@ -64,6 +64,29 @@ int mi_syrk_bf16(const void* A, int64_t batch, int64_t n, int64_t k,
                  int skip_upper, void* stream);
 
 /*
+ * mi_syrk_bf16 with a caller-provided scratch buffer.  Same arguments, same result up to the order of the float32
+ * additions along K.  The reference's kernels need no scratch (syrk.py:149-224, batched_syrk.py:158-234): they accept
+ * that a tile count which is not a multiple of what the GPU holds leaves it partly idle in the last round; this
+ * entry does not.  When the 256 x 256 tiles of the call would fill the rounds of the chip badly (batch 16 of
+ * 2048 x 8192: 576 tiles on 256 CUs), the whole rounds run as usual, the K range of each left-over tile is shared
+ * between several workgroups that park their float32 accumulators in `workspace`, and a last launch adds them, in a
+ * fixed order, and writes those tiles (three launches on `stream`; no workgroup waits for another).
+ * mi_syrk_workspace_bytes() gives the size needed (0: the call would not use one; any smaller buffer, or NULL,
+ * selects the ordinary launch); the buffer must be 256-byte aligned and must not be shared by calls that overlap in
+ * time.  The result is deterministic for a given (batch, n, k) and device, but which tiles are split depends on the
+ * batch size, so a matrix computed inside a batch and alone may differ in the last bit of float32 accumulation.
+ * Environment: MI_STREAMK=0 never splits, MI_STREAMK=1 splits whenever the shape qualifies (n a multiple of 256,
+ * n >= 1024, k a multiple of 64, A not transposed, skip_upper == 0) and tiles are left over after the whole rounds.
+ */
+size_t mi_syrk_workspace_bytes(int64_t batch, int64_t n, int64_t k, int a_trans);
+int mi_syrk_bf16_ws(const void* A, int64_t batch, int64_t n, int64_t k,
+                    int64_t a_batch_stride, int64_t a_ld, int a_trans,
+                    const void* C, int64_t c_batch_stride, int64_t c_ld,
+                    float alpha, float beta,
+                    void* D, int64_t d_batch_stride, int64_t d_ld,
+                    int skip_upper, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Xout[b] = beta * X[b] + alpha * (Bm[b] * X[b])      (bf16 in, fp32 accumulate)
  *
  * Replaces the third product of a Newton-Schulz step:
@@ -198,7 +221,7 @@ int mi_profile_end(float* ms_by_kind, int* launches_by_kind);
  * What the last product launched from this host thread used (for tests that must know which kernel variant served
  * a shape; the reference's tests check its autotuner's config pruning instead,
  * tests/test_triton_kernels.py:90-125): workgroups per batch entry, tile rows and columns, and whether it was the
- * direct-to-LDS kernel (1) or the general one (0).  Any pointer may be NULL.
+ * direct-to-LDS kernel (1; 2 for its stream-K launch) or the general one (0).  Any pointer may be NULL.
  */
 int mi_debug_last_launch(int* tiles, int* tile_m, int* tile_n, int* fast);
 

@@ -10,6 +10,8 @@ model replays, for every tile configuration x operand layout x product the libra
   * every 16-byte operand load of every wavefront for the first and the last K tile (``FastLoader``),
   * the addend loads and every store of both epilogues (row-wise and mirrored write-out, GEMM staging),
   * the per-workgroup partial-sum slot,
+  * the stream-K schedule of the 256 x 256 lower-triangle kernel (ranges of K tiles per workgroup, who parks an
+    accumulator image where, whom an owner waits for),
 over a grid of shapes (multiples of 8 on both sides of every tile size, batches, split-K slices, the tail split of
 the wide GEMM) and asserts that each access lies inside the matrix it belongs to.  It also checks that the tile
 enumerations visit every tile exactly once.  No GPU is involved.
@@ -79,22 +81,49 @@ def gemm_tile_of(pid, tiles_m, tiles_n, xcds=8, block_m=8):
     return rb * block_m + r % block_m, xcd * cols_per_xcd + r // block_m
 
 
-def syrk_grid_tiles(tiles_m):
-    """Workgroup id -> tile of the padded lower-triangle grid (None: padding workgroup that exits at once)."""
-    total = tiles_m * (tiles_m + 1) // 2
-    grid = (total + 7) // 8 * 8
-    per_xcd = grid // 8
+def round_size(cfg, cus=256):
+    """Workgroups of a configuration that the chip holds at once (two per CU when two rings fit its 160 KB of LDS)."""
+    tile_m, tile_n, _, _, slots = CFGS[cfg]
+    per_cu = 2 if 2 * slots * (tile_m + tile_n) * BK * 2 <= 160 * 1024 else 1
+    return max(cus * per_cu // 8 * 8, 8)
+
+
+def syrk_grid_tiles(tiles_m, batch=1, g=256, limit=None):
+    """Workgroup id -> (batch entry, tile) of the one-dimensional lower-triangle grid over a whole batch (None: padding
+    workgroup that exits at once): whole rounds of g workgroups, then a last round shared evenly between the XCDs."""
+    tri = tiles_m * (tiles_m + 1) // 2
+    total = tri * batch if limit is None else min(limit, tri * batch)
+    full = total // g * g
+    last = (total - full + 7) // 8
     out = []
-    for bid in range(grid):
-        s = (bid % 8) * per_xcd + bid // 8
-        out.append(tri_block_decode(s, tiles_m) if s < total else None)
+    for bid in range(full + 8 * last):
+        if bid < full:
+            tile = bid // g * g + (bid % 8) * (g // 8) + (bid % g) // 8
+        else:
+            j, rest = bid - full, total - full
+            lo, hi = rest * (j % 8) // 8, rest * (j % 8 + 1) // 8
+            if j // 8 >= hi - lo:
+                out.append(None)
+                continue
+            tile = full + lo + j // 8
+        out.append((tile // tri, tri_block_decode(tile % tri, tiles_m)))
     return out
 
 
 @pytest.mark.parametrize("tiles_m", list(range(1, 70)))
 def test_lower_triangle_grid_visits_every_tile_once(tiles_m):
-    seen = [t for t in syrk_grid_tiles(tiles_m) if t is not None]
-    assert sorted(seen) == [(i, j) for i in range(tiles_m) for j in range(i + 1)]
+    for batch, g in ((1, 256), (3, 256), (5, 512), (2, 8), (7, 304)):
+        grid = syrk_grid_tiles(tiles_m, batch, g)
+        seen = [t for t in grid if t is not None]
+        assert sorted(seen) == [(b, (i, j)) for b in range(batch) for i in range(tiles_m) for j in range(i + 1)]
+        # every XCD (workgroup id % 8) gets the same number of tiles, give or take one
+        per_xcd = [sum(1 for t in grid[x::8] if t is not None) for x in range(8)]
+        assert max(per_xcd) - min(per_xcd) <= 1
+    # a limited launch (the whole rounds of a split-tail product) computes exactly the first tiles of that order
+    tri = tiles_m * (tiles_m + 1) // 2
+    lim = 3 * tri // 2
+    seen = sorted(t for t in syrk_grid_tiles(tiles_m, 3, 256, limit=lim) if t is not None)
+    assert seen == sorted((b, tri_block_decode(s, tiles_m)) for b in range(3) for s in range(tri) if b * tri + s < lim)
 
 
 @pytest.mark.parametrize("tiles_m,tiles_n", [(4, 9), (8, 16), (16, 48), (16, 56), (8, 32), (1, 2), (3, 3), (16, 8), (24, 40), (7, 16)])
@@ -307,7 +336,8 @@ def launch_fast(cfg, p_ks, q_ks, mode, M, N, K):
     tiles_m, tiles_n = -(-M // tile_m), -(-N // tile_n)
     grid = tiles_m * (tiles_m + 1) // 2 if mode == "syrk" else tiles_m * tiles_n
     if mode == "syrk":
-        grid = (grid + 7) // 8 * 8
+        g = round_size(cfg)
+        grid = grid // g * g + 8 * ((grid % g + 7) // 8)
     edge = M % tile_m != 0 or N % tile_n != 0
     if edge and not (mode == "syrk" and not p_ks and not q_ks):
         return ("refused", "edge")
@@ -340,7 +370,7 @@ def test_lower_triangle_launches_stay_inside_their_matrices(cfg, p_ks, q_ks, mod
         _, edge, tiles_m, _, grid = res
         launched += 1
         assert edge == (n % tile != 0)
-        tiles = syrk_grid_tiles(tiles_m)
+        tiles = [t if t is None else t[1] for t in syrk_grid_tiles(tiles_m, 1, round_size(cfg))]
         assert len(tiles) == grid
         nk = k // BK
         out = Matrix("D", n, n)
@@ -502,3 +532,99 @@ def test_k_strided_edge_tiles_are_refused_not_clamped():
         assert launch_fast(cfg, p_ks, q_ks, mode, 4096, 4096, 1000)[0] == "refused"   # K tail
     with pytest.raises(AssertionError):
         loader_accesses(256, True, True, 0, 1000, 0, 0)
+
+
+# ------------------------------------------------------------------ split-tail (stream-K) launch of the 256 x 256 lower-triangle kernel
+MAX_STREAMK_SPLITS = 8
+
+
+def streamk_plan(tiles, k_tiles, cus):
+    rounds, rem = divmod(tiles, cus)
+    splits = min(cus // rem, MAX_STREAMK_SPLITS, k_tiles) if rem else 0
+    return rounds, rem, (splits if splits >= 2 else 0)
+
+
+def streamk_launches(tiles, nk_full, cus):
+    """Replays launch_streamk's geometry and the workgroup decoding of gemm_fast_kernel<..., SK_WHOLE / SK_PARTS /
+    SK_FINISH>: (whole, parts, finish) with whole = [(workgroup, tile)], parts = [(workgroup, tile, k_first, nk, image
+    slot)], finish = [(workgroup, tile, [image slots in the order they are added])]; padding workgroups left out."""
+    rounds, rem, splits = streamk_plan(tiles, nk_full, cus)
+    split = splits > 1
+    sk_whole = rounds * cus if split else tiles  # (computed whole by an ordinary launch limited to these tiles)
+    tpx = (rem + 7) // 8 if split else 1
+    whole, parts, finish = [(bid, bid) for bid in range(sk_whole)], [], []
+    if split:
+        for bid in range(8 * tpx * splits):
+            t, sp = (bid % 8) * tpx + (bid // 8) % tpx, (bid // 8) // tpx
+            if t >= rem or sp >= splits:
+                continue
+            k_first = nk_full * sp // splits
+            parts.append((bid, sk_whole + t, k_first, nk_full * (sp + 1) // splits - k_first, sp * rem + t))
+        for bid in range(4 * rem):  # four workgroups per left-over tile, one per 128 x 128 quarter
+            if bid % 4 == 0:
+                finish.append((bid, sk_whole + bid // 4, [sp * rem + bid // 4 for sp in range(splits)]))
+    return whole, parts, finish, (rounds, rem, splits)
+
+
+def test_split_tail_image_layout():
+    """SK_PARTS (256 x 256 tile, 2 x 2 wavefronts of 128 x 128, 8 x 8 fragments each) stores fragment (I, J) of thread t
+    at float4 ((I 8 + J) 256 + t) of the image; SK_FINISH (128 x 128 tile = one quarter, 2 x 2 wavefronts of 64 x 64,
+    4 x 4 fragments each) reads fragment (i, j) of its wavefront (wm, wn) from ((wm 4 + i) 8 + wn 4 + j) 256 + quarter
+    64 + lane.  Both must name the same element of the tile, every element once, inside the image."""
+    lane = np.arange(64)
+    where = {}
+    for wave in range(4):  # SK_PARTS: wavefront = row half + 2 * column half
+        WM, WN = wave % 2, wave // 2
+        for I in range(8):
+            for J in range(8):
+                idx = (I * 8 + J) * 256 + wave * 64 + lane
+                rows = WM * 128 + 16 * I + (lane & 15)
+                cols = WN * 128 + 16 * J + 4 * (lane >> 4)
+                for a, r, c in zip(idx, rows, cols):
+                    where[int(a)] = (int(r), int(c))
+    assert sorted(where) == list(range(256 * 64))  # 65536 float4 = one image
+    seen = set()
+    for quarter in range(4):
+        qm, qn = quarter % 2, quarter // 2
+        for wave in range(4):
+            wm, wn = wave % 2, wave // 2
+            for i in range(4):
+                for j in range(4):
+                    idx = ((wm * 4 + i) * 8 + wn * 4 + j) * 256 + quarter * 64 + lane
+                    rows = qm * 128 + wm * 64 + 16 * i + (lane & 15)
+                    cols = qn * 128 + wn * 64 + 16 * j + 4 * (lane >> 4)
+                    for a, r, c in zip(idx, rows, cols):
+                        assert where[int(a)] == (int(r), int(c))
+                        seen.add(int(a))
+    assert len(seen) == 256 * 64
+
+
+@pytest.mark.parametrize("batch,n,k", [(16, 2048, 8192), (1, 1024, 8192), (3, 1280, 1024), (2, 1536, 4096), (1, 4096, 14336),
+                                       (7, 1024, 64), (1, 2048, 128), (5, 1792, 448), (5, 1024, 448), (64, 1024, 256)])
+@pytest.mark.parametrize("cus", [256, 248, 8, 304])
+def test_split_tail_schedule(batch, n, k, cus):
+    t, nk_full = n // 256, k // 64
+    tiles = t * (t + 1) // 2 * batch
+    whole, parts, finish, (rounds, rem, splits) = streamk_launches(tiles, nk_full, cus)
+    assert splits == 0 or (2 <= splits and rem * splits <= cus)  # the split round is a single round
+    # every K tile of every tile is multiplied exactly once, inside the K range of the operands
+    cover = np.zeros((tiles, nk_full), dtype=np.int32)
+    for _, tile in whole:
+        assert 0 <= tile < tiles
+        cover[tile] += 1
+    for _, tile, k0, cnt, _ in parts:
+        assert 0 <= tile < tiles and 0 <= k0 and cnt > 0 and (k0 + cnt) * 64 <= k
+        cover[tile, k0:k0 + cnt] += 1
+    assert (cover == 1).all()
+    # every part has an image slot of its own inside the workspace the launcher asks for, and the finishing
+    # workgroup of a tile adds exactly the images of that tile's parts, every left-over tile once
+    n_images = rem * splits
+    assert sorted(slot for *_, slot in parts) == list(range(n_images))
+    assert sorted(tile for _, tile, _ in finish) == sorted({tile for _, tile, *_ in parts})
+    for _, tile, slots in finish:
+        assert sorted(slots) == sorted(slot for _, tl, _, _, slot in parts if tl == tile)
+    # the workgroups of one XCD (workgroup id % 8) that run at the same time work on neighbouring tiles
+    if splits:
+        for x in range(8):
+            mine = [tile for bid, tile, k0, *_ in parts if bid % 8 == x and k0 == 0]
+            assert mine == list(range(mine[0], mine[0] + len(mine))) if mine else True

@@ -93,6 +93,10 @@ def test_frob_normalize_clamp_and_underflow(gpu):
 
 
 # ---------------------------------------------------------------- which kernel variant served a shape
+def rel_fro_t(a, b):
+    return float((a - b).norm() / b.norm())
+
+
 def _int_bf16(shape, lo, hi, dev, seed=0):
     return torch.randint(lo, hi, shape, generator=torch.Generator().manual_seed(seed)).to(BF).to(dev)
 
@@ -213,3 +217,55 @@ def test_syrk_lower_triangle_only(gpu, n, k, batch, trans):
     assert torch.equal(out2[:, low], ref2[:, low])
     up2 = out2[:, ~low]
     assert bool((torch.isnan(up2) | (up2 == ref2[:, ~low])).all())
+
+
+# ---------------------------------------------------------------- split-tail (stream-K) launch of the lower-triangle kernel
+@pytest.mark.parametrize("batch,n,k", [(16, 2048, 8192), (1, 1024, 8192), (3, 1280, 1024), (2, 1536, 4096), (5, 1024, 448),
+                                       (30, 1024, 128), (26, 1024, 256)])
+def test_syrk_stream_k_integer_exact(gpu, monkeypatch, batch, n, k):
+    """Whole rounds of 256 x 256 tiles, then the left-over tiles with their K range split between workgroups that
+    park float32 accumulators in the workspace, then a launch that adds them and writes those tiles.  Small integers
+    make every float32 sum exact, so the result must equal the ordinary launch bit for bit.  30 x 1024 x 128: 300
+    tiles, 44 left over, 2 K tiles each (the split is capped by K); 26 x 1024 x 256: 260 tiles, 4 left over, 4 K tiles."""
+    monkeypatch.setenv("MI_STREAMK", "1")
+    a = _int_bf16((batch, n, k), -2, 3, gpu, seed=n + k)
+    print(f"stream-K {batch}x{n}x{k}", flush=True)
+    d = triton_kernels.batched_tsyrk_ex(a)
+    info = _hip.last_launch()
+    assert info["fast"] == 2 and info["tile_m"] == 256, info
+    ref = torch.bmm(a.float(), a.float().mT)
+    assert torch.equal(d, ref.to(BF)) and torch.equal(d, d.mT)
+    s = _int_bf16((batch, n, n), -3, 3, gpu, seed=n)
+    s = s + s.mT
+    d2 = triton_kernels.batched_tsyrk_ex(a, s, alpha=0.25, beta=0.5)
+    assert _hip.last_launch()["fast"] == 2
+    assert torch.equal(d2, torch.baddbmm(s.float(), a.float(), a.float().mT, alpha=0.25, beta=0.5).to(BF))
+    monkeypatch.setenv("MI_STREAMK", "0")
+    d3 = triton_kernels.batched_tsyrk_ex(a)
+    assert _hip.last_launch()["fast"] == 1 and torch.equal(d3, d)
+    if batch * n <= 1280:
+        assert np.array_equal(d[0].float().cpu().numpy(), O.syrk(a[0].float().cpu().numpy()))
+
+
+def test_syrk_stream_k_random_inputs_and_model_choice(gpu, monkeypatch):
+    """Gaussian operands: the stream-K launch adds the same products in another order (float32), so it agrees with the
+    ordinary launch to bf16 rounding of near-ties; which launch the cost model picks for the benchmark shapes."""
+    monkeypatch.delenv("MI_STREAMK", raising=False)
+    a = torch.randn(16, 2048, 8192, device=gpu, generator=torch.Generator(device=gpu).manual_seed(5)).to(BF)
+    d = triton_kernels.batched_tsyrk_ex(a)
+    chosen = _hip.last_launch()
+    if torch.cuda.get_device_properties(0).multi_processor_count == 256:
+        assert chosen["fast"] == 2, chosen  # 576 tiles of 256 x 256 = 2.25 rounds of 256 CUs
+    monkeypatch.setenv("MI_STREAMK", "0")
+    d0 = triton_kernels.batched_tsyrk_ex(a)
+    assert _hip.last_launch()["fast"] == 1
+    diff = (d.float() - d0.float()).abs()
+    # one bf16 ulp at most, and only where the float32 sums straddle a rounding boundary
+    assert float((diff / d0.float().abs().clamp_min(1.0)).max()) <= 2.0 ** -7
+    assert float((diff > 0).float().mean()) < 0.02
+    ref = a[3].float() @ a[3].float().T
+    assert rel_fro_t(d[3].float(), ref) < 3e-3
+    monkeypatch.delenv("MI_STREAMK", raising=False)
+    x = torch.randn(4096, 14336, device=gpu).to(BF)
+    triton_kernels.tsyrk_ex(x)
+    assert _hip.last_launch()["fast"] == 1  # 253 tiles of 192 x 192: one round already

@@ -34,9 +34,27 @@ def instructions(lines):
     return out
 
 
+def agprs_of(text):
+    """AGPR numbers an instruction names (a12, a[8:11])."""
+    out = set()
+    for m in re.finditer(r"\ba\[(\d+):(\d+)\]|\ba(\d+)\b", text):
+        if m.group(3) is not None:
+            out.add(int(m.group(3)))
+        else:
+            out.update(range(int(m.group(1)), int(m.group(2)) + 1))
+    return out
+
+
 def accumulator_hazards(lines):
     ins = instructions(lines)
     text = [t for _, t in ins]
+    # the accumulators are the AGPRs some MFMA writes; the compiler also parks ordinary values in free AGPRs, and
+    # moving those around next to an MFMA is harmless
+    accumulators = set()
+    for t in text:
+        if t.startswith("v_mfma"):
+            accumulators |= agprs_of(t.split(",")[0])
+    touches = lambda x: ACC_TRAFFIC.match(x) and (agprs_of(x) & accumulators)
     label_at = {t[:-1]: k for k, t in enumerate(text) if t.endswith(":")}
     bad = []
     # innermost loops (a branch back to an earlier label with no other loop inside)
@@ -52,7 +70,7 @@ def accumulator_hazards(lines):
             continue
         body = text[lo:hi]
         if any(x.startswith("v_mfma") for x in body):
-            bad += [f"in MFMA loop: {x}" for x in body if ACC_TRAFFIC.match(x)]
+            bad += [f"in MFMA loop: {x}" for x in body if touches(x)]
     # between an MFMA and the drain (or the next MFMA)
     for k, t in enumerate(text):
         if not t.startswith("v_mfma"):
@@ -60,7 +78,7 @@ def accumulator_hazards(lines):
         for x in text[k + 1:k + 13]:
             if x.startswith("v_mfma") or x.startswith("s_nop 7"):
                 break
-            if ACC_TRAFFIC.match(x):
+            if touches(x):
                 bad.append(f"after MFMA, before the drain: {x}")
     return bad
 
@@ -73,11 +91,14 @@ def test_detector_flags_swaps_and_spills():
 	;;#ASMSTART
 	v_mfma_f32_16x16x32_bf16 a[0:3], v[14:17], v[46:49], a[0:3]
 	;;#ASMEND
+	;;#ASMSTART
+	v_mfma_f32_16x16x32_bf16 a[220:223], v[14:17], v[50:53], a[220:223]
+	;;#ASMEND
 	s_cbranch_scc1 .LBB0_1
 """.splitlines()
     assert len(accumulator_hazards(swap)) == 2
     spill = """
-	v_mfma_f32_16x16x32_bf16 a[0:3], v[14:17], v[46:49], a[0:3]
+	v_mfma_f32_16x16x32_bf16 a[232:235], v[14:17], v[46:49], a[232:235]
 	scratch_store_dwordx4 off, a[232:235], off offset:100 ; 16-byte Folded Spill
 	s_nop 7
 	v_accvgpr_read_b32 v1, a0
@@ -88,10 +109,11 @@ def test_detector_flags_swaps_and_spills():
 	v_mfma_f32_16x16x32_bf16 a[0:3], v[14:17], v[46:49], a[0:3]
 	ds_read_b64_tr_b16 v[118:119], v66
 	s_cbranch_scc1 .LBB0_1
+	v_accvgpr_read_b32 v191, a151
 	s_nop 7
 	v_accvgpr_read_b32 v1, a0
 """.splitlines()
-    assert accumulator_hazards(clean) == []
+    assert accumulator_hazards(clean) == []  # a151 is no accumulator here: a value the compiler parked in a free AGPR
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="hipcc not available")
@@ -107,10 +129,12 @@ def test_no_accumulator_traffic_next_to_mfma(tmp_path):
                 kernels[name] = []
             elif name:
                 kernels[name].append(line)
-                if "s_endpgm" in line:
+                if line.startswith(".Lfunc_end"):  # (not the first s_endpgm: a kernel may return early)
                     name = None
     fast = {n: ls for n, ls in kernels.items() if "gemm_fast_kernel" in n or "small_chain_kernel" in n}
-    assert len(fast) >= 20 and all(any("v_mfma" in x for x in ls) for ls in fast.values())
+    # (the finishing kernel of a split-tail launch, last template argument 2, has an epilogue and no K loop)
+    no_mfma = [n for n, ls in fast.items() if not any("v_mfma" in x for x in ls)]
+    assert len(fast) >= 20 and all(n.endswith("ELi2EEEvNS_10GemmParamsE") for n in no_mfma) and len(no_mfma) <= 1, no_mfma
     report = {n: accumulator_hazards(ls) for n, ls in fast.items()}
     report = {n: b for n, b in report.items() if b}
     assert not report, "\n".join(f"{n}: {len(b)} hazards, e.g. {b[0]}" for n, b in report.items())
