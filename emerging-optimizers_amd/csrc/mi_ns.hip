@@ -101,6 +101,7 @@ int device_cus() {
 //      192 x 192                    F = 14.5   s = 0.55 (f <= 0.45) .. 0.78 (f = 1)
 //      256 x 256 (n % 256 == 0)     F = 16.5   s = 0.95 (f <= 0.55) .. 1.37 (f >= 0.9)
 //      128 x 128, two per CU        F =  9.2   s = 0.74 (kt <= 32) .. 0.85 (kt >= 128) per pair of tiles   (n % 128 == 0)
+//                                              (last, partial round: 0.5 + 0.35 f)
 //      128 x 128, one per CU        F =  9.0   s = 0.44 (0.31 when one round is not full)                  (n % 128 == 0)
 //    Short K or few tiles favour the small tiles, long K with many tiles the 192 x 192 tile, and shapes whose
 //    256 x 256 tiles fill one round (8 x 1792: 224 tiles) or that 192 divides badly the 256 x 256 tile.
@@ -126,11 +127,29 @@ static SyrkTile pick_syrk_tile(int64_t n, int64_t batch, int64_t k, bool k_strid
   auto offer = [&](SyrkTile t, double cost) {
     if (cost < best_cost) best = t, best_cost = cost;
   };
+  if (k_strided) {
+    // The transpose reads of a K-strided tile cost two LDS instructions per fragment: the K loop is 10 - 40 % slower
+    // than on K-contiguous operands and hardly follows the fill (measured, n = 1024 .. 8192, K = 1024 .. 14336):
+    //   256 x 256   s = 1.35 (f <= 0.55) .. 1.47      128 x 128, two per CU   0.90 per pair in a full round,
+    //   128 x 128, one per CU   0.6 in a single round, 0.8 else             0.65 + 0.25 f in the last, partial one
+    if (n % 256 == 0)
+      offer(SYRK_TILE_256, by_rounds(tiles(256), 16.5, [](double f) { return f <= 0.55 ? 1.35 : 1.35 + (f - 0.55) * 0.27; }));
+    if (n % 128 == 0) {
+      const int64_t t128 = tiles(128), full = t128 / (2 * cus), rem = t128 % (2 * cus);
+      offer(SYRK_TILE_128X2, (double)full * (9.2 + 0.90 * kt) +
+                                 (rem ? 9.2 + (0.65 + 0.25 * (double)rem / (double)(2 * cus)) * kt : 0.0));
+      offer(SYRK_TILE_128, t128 <= cus ? 9.0 + 0.6 * kt : (double)ceil_div(t128, cus) * (9.0 + 0.8 * kt));
+    }
+    if (cost_us) *cost_us = best_cost;
+    return best;
+  }
   if (n % 256 == 0) offer(SYRK_TILE_256, by_rounds(tiles(256), 16.5, slope256));
   if (n % 128 == 0) {
     const int64_t t128 = tiles(128);
     const double s2 = 0.74 + 0.11 * std::min(std::max(kt - 32.0, 0.0) / 96.0, 1.0);
-    offer(SYRK_TILE_128X2, (double)ceil_div(t128, 2 * cus) * (9.2 + s2 * kt));
+    const int64_t full2 = t128 / (2 * cus), rem2 = t128 % (2 * cus);
+    offer(SYRK_TILE_128X2, (double)full2 * (9.2 + s2 * kt) +
+                               (rem2 ? 9.2 + std::min(s2, 0.5 + 0.35 * (double)rem2 / (double)(2 * cus)) * kt : 0.0));
     offer(SYRK_TILE_128, (double)ceil_div(t128, cus) * (9.0 + (t128 <= cus ? 0.31 : 0.44) * kt));
   }
   if (cost_us) *cost_us = best_cost;
