@@ -265,6 +265,58 @@ struct ShiftArgs {
 
 // D = alpha * A A^T + beta * C, bf16 out.
 // Inside the fused driver the same lower-triangle kernel also forms products of two commuting symmetric matrices:
+// dst[b][r][c] = src[b][c][r] for bf16 matrices: src has `cols_out` rows of `rows_out` elements.  64 x 64 tiles through LDS,
+// 16-byte global accesses on both sides (all extents are multiples of 8).
+__global__ void __launch_bounds__(256) transpose_bf16_kernel(const uint16_t* __restrict__ src, int64_t src_bs, int64_t src_ld,
+                                                             uint16_t* __restrict__ dst, int64_t dst_bs, int64_t dst_ld,
+                                                             int rows_out, int cols_out) {
+  __shared__ uint16_t tile[64][64 + 2];  // [row of dst][column of dst]; 33 words per row: conflict-free column writes
+  const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64, tid = threadIdx.x;
+  const uint16_t* s = src + blockIdx.z * src_bs;
+  uint16_t* d = dst + blockIdx.z * dst_bs;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int ch = tid + 256 * i, c = ch / 8, r = (ch % 8) * 8;  // source row c0 + c, elements r0 + r .. + 7
+    if (c0 + c < cols_out && r0 + r < rows_out) {
+      const uint4 v = *reinterpret_cast<const uint4*>(s + (int64_t)(c0 + c) * src_ld + r0 + r);
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        tile[r + 2 * e][c] = (uint16_t)(w[e] & 0xffffu);
+        tile[r + 2 * e + 1][c] = (uint16_t)(w[e] >> 16);
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int ch = tid + 256 * i, r = ch / 8, c = (ch % 8) * 8;
+    if (r0 + r < rows_out && c0 + c < cols_out) {
+      uint32_t w[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) w[e] = (uint32_t)tile[r][c + 2 * e] | ((uint32_t)tile[r][c + 2 * e + 1] << 16);
+      *reinterpret_cast<uint4*>(d + (int64_t)(r0 + r) * dst_ld + c0 + c) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+  }
+}
+
+// A K-strided operand of a lower-triangle product (stored as K rows of N): copy it transposed into scratch memory
+// first?  The K loop of the K-strided kernels is slower and they have no 192 x 192 tile; the copy runs at about
+// 4 TB/s (read + write).  Bytes of scratch the copy needs, or 0 when the model expects no gain.
+static size_t transposed_copy_bytes(int64_t n, int64_t batch, int64_t k) {
+  if (n < 1024 || k % 64 != 0) return 0;  // (below, both layouts go to the general kernel)
+  const char* env = getenv("MI_SYRK_TRANSPOSE");  // "0": never, "1": always (tests), else by the model
+  if (env && env[0] == '0') return 0;
+  const size_t bytes = ((size_t)batch * n * k * 2 + 255) / 256 * 256;
+  if (env && env[0] == '1') return bytes;
+  if (n < 2048) return 0;  // (launches of a few dozen small tiles: the model is too coarse there, measured no gain)
+  double strided = 0.0, contiguous = 0.0;
+  if (pick_syrk_tile(n, batch, k, true, &strided) == SYRK_TILE_NONE) return bytes;
+  pick_syrk_tile(n, batch, k, false, &contiguous);
+  const double copy = 6.0 + 2.0 * (double)bytes / 4.0e6;
+  return contiguous + copy < 0.95 * strided ? bytes : 0;
+}
+
 // `other` != null computes alpha * A other^T (symmetric in exact arithmetic; the lower triangle is computed and
 // mirrored), and `C2` is a second addend laid out like C whose coefficient a SHIFT_GROUP_* mode supplies.
 static int syrk_impl(const void* A, int64_t batch, int64_t n, int64_t k, int64_t a_bs, int64_t a_ld, int a_trans,
@@ -1440,18 +1492,35 @@ int mi_syrk_bf16(const void* A, int64_t batch, int64_t n, int64_t k, int64_t a_b
 }
 
 size_t mi_syrk_workspace_bytes(int64_t batch, int64_t n, int64_t k, int a_trans) {
-  if (batch <= 0 || n <= 0 || k <= 0) return 0;
+  if (batch <= 0 || n <= 0 || k <= 0 || n % 8 || k % 8) return 0;
   StreamKPlan plan;
-  return streamk_wanted(n, batch, k, a_trans != 0, &plan) ? streamk_workspace_bytes(plan) : 0;
+  const size_t copy = a_trans ? transposed_copy_bytes(n, batch, k) : 0;
+  const bool contiguous = !a_trans || copy > 0;
+  return copy + (streamk_wanted(n, batch, k, !contiguous, &plan) ? streamk_workspace_bytes(plan) : 0);
 }
 
 int mi_syrk_bf16_ws(const void* A, int64_t batch, int64_t n, int64_t k, int64_t a_batch_stride, int64_t a_ld, int a_trans,
                     const void* C, int64_t c_batch_stride, int64_t c_ld, float alpha, float beta, void* D,
                     int64_t d_batch_stride, int64_t d_ld, int skip_upper, void* workspace, size_t workspace_bytes,
                     void* stream) {
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (a_trans && A && workspace && batch > 0 && n > 0 && k > 0 && n % 8 == 0 && k % 8 == 0 && a_ld % 8 == 0 &&
+      a_batch_stride % 8 == 0 && a_ld >= n && aligned16(A) && !(reinterpret_cast<uintptr_t>(workspace) & 255u)) {
+    const size_t copy = transposed_copy_bytes(n, batch, k);
+    if (copy > 0 && workspace_bytes >= copy && n < (1 << 30) && k < (1 << 30) && batch <= 65535) {
+      // the operand, K-contiguous, in the first part of the workspace; the rest serves the product itself
+      uint16_t* At = static_cast<uint16_t*>(workspace);
+      dim3 grid((unsigned)((n + 63) / 64), (unsigned)((k + 63) / 64), (unsigned)batch);
+      hipLaunchKernelGGL(transpose_bf16_kernel, grid, dim3(256), 0, st, static_cast<const uint16_t*>(A), a_batch_stride, a_ld, At,
+                         n * k, k, (int)n, (int)k);
+      hipError_t e = hipGetLastError();
+      if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+      return syrk_impl(At, batch, n, k, n * k, k, 0, C, c_batch_stride, c_ld, alpha, beta, D, d_batch_stride, d_ld, skip_upper,
+                       st, nullptr, nullptr, nullptr, static_cast<char*>(workspace) + copy, workspace_bytes - copy);
+    }
+  }
   return syrk_impl(A, batch, n, k, a_batch_stride, a_ld, a_trans, C, c_batch_stride, c_ld, alpha, beta, D,
-                   d_batch_stride, d_ld, skip_upper, static_cast<hipStream_t>(stream), nullptr, nullptr, nullptr, workspace,
-                   workspace_bytes);
+                   d_batch_stride, d_ld, skip_upper, st, nullptr, nullptr, nullptr, workspace, workspace_bytes);
 }
 
 int mi_gemm_axpy_bf16(const void* Bm, int64_t b_batch_stride, int64_t b_ld, const void* X,

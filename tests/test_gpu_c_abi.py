@@ -173,9 +173,11 @@ SYRK_VARIANTS = [
 
 
 @pytest.mark.parametrize("n,k,trans,tile", SYRK_VARIANTS)
-def test_syrk_variants_integer_exact(gpu, n, k, trans, tile):
+def test_syrk_variants_integer_exact(gpu, monkeypatch, n, k, trans, tile):
     """Both operand layouts on the direct-to-LDS kernels (a transposed operand has 128- and 256-row tiles and no
     variant for tiles that overhang the matrix: 1096 rows go to the general kernel there)."""
+    monkeypatch.setenv("MI_SYRK_TRANSPOSE", "0")  # the K-strided kernels themselves, not the transposing copy
+    monkeypatch.setenv("MI_STREAMK", "0")
     a = _int_bf16((k, n) if trans else (n, k), -3, 3, gpu, seed=n + k)
     if trans:
         a = a.T
@@ -269,3 +271,36 @@ def test_syrk_stream_k_random_inputs_and_model_choice(gpu, monkeypatch):
     x = torch.randn(4096, 14336, device=gpu).to(BF)
     triton_kernels.tsyrk_ex(x)
     assert _hip.last_launch()["fast"] == 1  # 253 tiles of 192 x 192: one round already
+
+
+# ---------------------------------------------------------------- K-strided operand through a transposed copy
+@pytest.mark.parametrize("batch,n,k", [(1, 1024, 512), (2, 1096, 192), (1, 4096, 14336), (3, 1280, 4096), (16, 2048, 8192)])
+def test_syrk_transposed_copy_integer_exact(gpu, monkeypatch, batch, n, k):
+    """A K-strided operand is first copied, transposed, into the workspace and then multiplied by the K-contiguous
+    kernels (which have a 192 x 192 tile and the faster K loop).  Bit-equal to the K-strided kernels on small integers.
+    4096 x 14336 is a shape where the model itself chooses the copy (elsewhere it is forced here); 16 x 2048 x 8192
+    adds the split-tail launch behind it, both parts of the workspace in use."""
+    forced = (n, k) != (4096, 14336)
+    if forced:
+        monkeypatch.setenv("MI_SYRK_TRANSPOSE", "1")
+    else:
+        monkeypatch.delenv("MI_SYRK_TRANSPOSE", raising=False)
+    a = _int_bf16((batch, k, n), -2, 3, gpu, seed=n + k + 1).mT  # stored as k rows of n
+    assert a.stride(-2) == 1
+    print(f"transposed copy {batch}x{n}x{k}", flush=True)
+    lib = _hip.lib()
+    need = lib.mi_syrk_workspace_bytes(batch, n, k, 1)
+    assert need >= batch * n * k * 2
+    d = triton_kernels.batched_tsyrk_ex(a)
+    info = _hip.last_launch()
+    if k % 64 == 0 and n >= 1024:
+        assert info["fast"] in (1, 2) and (info["tile_m"] == 192 if (n, k) == (4096, 14336) else True), info
+    ref = torch.bmm(a.float(), a.float().mT).to(BF)
+    assert torch.equal(d, ref)
+    s = _int_bf16((batch, n, n), -3, 3, gpu, seed=n)
+    s = s + s.mT
+    d2 = triton_kernels.batched_tsyrk_ex(a, s, alpha=0.25, beta=0.5)
+    assert torch.equal(d2, torch.baddbmm(s.float(), a.float(), a.float().mT, alpha=0.25, beta=0.5).to(BF))
+    monkeypatch.setenv("MI_SYRK_TRANSPOSE", "0")
+    assert torch.equal(triton_kernels.batched_tsyrk_ex(a), d)
+    assert lib.mi_syrk_workspace_bytes(batch, n, k, 1) < batch * n * k * 2
