@@ -90,21 +90,32 @@ int device_cus() {
   return cached;
 }
 
-// Tile choice of the fast path by modelled time, fitted to measurements on this part (lower-triangle products with
-// n = 1024 .. 8192, batch 1 .. 16, K = 64 .. 8192; GEMM m = 1024 .. 4096).
+// Tile choice of the fast path by modelled time, fitted to measurements on this part.
 //  * GEMM: 256 x 128 tiles cost about 1.27x per FLOP of 256 x 256 tiles and win when the latter leave CUs idle
 //    (1024 x 4096: 64 tiles).
-//  * Lower-triangle kernel: a launch runs in rounds of one workgroup per CU (two for the two-slot 128 x 128 tile); a
-//    round costs F + s kt microseconds (kt = 64-deep K tiles).  F is launch, prologue and the write-out of the tiles
-//    (bound by the write bandwidth of the fabric, about 13 us for the 33 MB of a 4096 x 4096 result).  s rises with
-//    the share f of the CUs that a round keeps busy, because the clock follows the power drawn:
-//      192 x 192                    F = 14.5   s = 0.55 (f <= 0.45) .. 0.78 (f = 1)
-//      256 x 256 (n % 256 == 0)     F = 16.5   s = 0.95 (f <= 0.55) .. 1.37 (f >= 0.9)
-//      128 x 128, two per CU        F =  9.2   s = 0.74 (kt <= 32) .. 0.85 (kt >= 128) per pair of tiles   (n % 128 == 0)
-//                                              (last, partial round: 0.5 + 0.35 f)
-//      128 x 128, one per CU        F =  9.0   s = 0.44 (0.31 when one round is not full)                  (n % 128 == 0)
+//  * Lower-triangle kernel (K-contiguous operands): a launch runs in rounds of g workgroups (one per CU; two for the
+//    two-slot 128 x 128 tile), the last round possibly part-filled (share f of g).  In microseconds, with kt = 64-deep
+//    K tiles:   L + full rounds x (F + s kt) + [last round] (F + min(s, s0 + s1 f) kt).
+//    L is the launch, F prologue and write-out of a tile; the slope of a part-filled round is lower because the clock
+//    follows the power drawn.  Least-squares fit over 437 shapes (n = 256 .. 8192, batch 1 .. 64, K = 256 .. 14336,
+//    every tile forced in turn): relative error 3 - 8 % rms; the tile chosen is within 2 % of the best forced tile on
+//    409 of them, 0.4 % slower on average, 18 % at worst (2 x 8192 x 256).
+//                               L      F      s      s0     s1
+//      128 x 128, one per CU   12.1    5.5   0.48   0.29   0.11     (n % 128 == 0)
+//      128 x 128, two per CU    8.9    7.4   0.84   0.43   0.45     (n % 128 == 0; per pair of tiles)
+//      192 x 192               14.6   10.8   0.81   0.50   0.26
+//      256 x 256               12.3   12.9   1.32   0.88   0.43     (n % 256 == 0)
 //    Short K or few tiles favour the small tiles, long K with many tiles the 192 x 192 tile, and shapes whose
-//    256 x 256 tiles fill one round (8 x 1792: 224 tiles) or that 192 divides badly the 256 x 256 tile.
+//    256 x 256 tiles fill whole rounds (8 x 1792: 224 tiles) or that 192 divides badly the 256 x 256 tile.
+struct TileCost {
+  double L, F, s, s0, s1;
+  double operator()(int64_t count, int64_t g, double kt) const {
+    const int64_t full = count / g, rem = count % g;
+    return L + (double)full * (F + s * kt) + (rem ? F + std::min(s, s0 + s1 * (double)rem / (double)g) * kt : 0.0);
+  }
+};
+static constexpr TileCost COST_128{12.1, 5.5, 0.48, 0.29, 0.11}, COST_128X2{8.9, 7.4, 0.84, 0.43, 0.45},
+    COST_192{14.6, 10.8, 0.81, 0.50, 0.26}, COST_256{12.3, 12.9, 1.32, 0.88, 0.43};
 enum SyrkTile { SYRK_TILE_NONE, SYRK_TILE_128, SYRK_TILE_128X2, SYRK_TILE_192, SYRK_TILE_256 };
 // `k_strided`: the operand is stored transposed; its LDS layout exists for 128- and 256-row tiles only, and not for
 // tiles that overhang the matrix, so there may be no fast tile at all.
@@ -115,15 +126,13 @@ static SyrkTile pick_syrk_tile(int64_t n, int64_t batch, int64_t k, bool k_strid
     const int64_t t = ceil_div(n, tile);
     return t * (t + 1) / 2 * batch;
   };
-  // full rounds at the slope of a full chip, the last partial round at the slope of its own fill
+  // (K-strided operands: full rounds at the slope of a full chip, the last partial round at the slope of its own fill)
   auto by_rounds = [&](int64_t count, double fixed, auto slope) {
     const int64_t full = count / cus, rem = count % cus;
     return (double)full * (fixed + slope(1.0) * kt) + (rem ? fixed + slope((double)rem / (double)cus) * kt : 0.0);
   };
-  auto slope192 = [](double f) { return f <= 0.45 ? 0.55 : 0.55 + (f - 0.45) * 0.42; };
-  auto slope256 = [](double f) { return f <= 0.55 ? 0.95 : std::min(1.37, 0.95 + (f - 0.55) * 1.2); };
   SyrkTile best = k_strided ? SYRK_TILE_NONE : SYRK_TILE_192;
-  double best_cost = k_strided ? 1e30 : by_rounds(tiles(192), 14.5, slope192);
+  double best_cost = k_strided ? 1e30 : COST_192(tiles(192), cus, kt);
   auto offer = [&](SyrkTile t, double cost) {
     if (cost < best_cost) best = t, best_cost = cost;
   };
@@ -143,14 +152,10 @@ static SyrkTile pick_syrk_tile(int64_t n, int64_t batch, int64_t k, bool k_strid
     if (cost_us) *cost_us = best_cost;
     return best;
   }
-  if (n % 256 == 0) offer(SYRK_TILE_256, by_rounds(tiles(256), 16.5, slope256));
+  if (n % 256 == 0) offer(SYRK_TILE_256, COST_256(tiles(256), cus, kt));
   if (n % 128 == 0) {
-    const int64_t t128 = tiles(128);
-    const double s2 = 0.74 + 0.11 * std::min(std::max(kt - 32.0, 0.0) / 96.0, 1.0);
-    const int64_t full2 = t128 / (2 * cus), rem2 = t128 % (2 * cus);
-    offer(SYRK_TILE_128X2, (double)full2 * (9.2 + s2 * kt) +
-                               (rem2 ? 9.2 + std::min(s2, 0.5 + 0.35 * (double)rem2 / (double)(2 * cus)) * kt : 0.0));
-    offer(SYRK_TILE_128, (double)ceil_div(t128, cus) * (9.0 + (t128 <= cus ? 0.31 : 0.44) * kt));
+    offer(SYRK_TILE_128X2, COST_128X2(tiles(128), 2 * cus, kt));
+    offer(SYRK_TILE_128, COST_128(tiles(128), cus, kt));
   }
   if (cost_us) *cost_us = best_cost;
   return best;
@@ -159,8 +164,8 @@ static SyrkTile pick_syrk_tile(int64_t n, int64_t batch, int64_t k, bool k_strid
 // Split-tail (stream-K) launch of the lower-triangle kernel (256 x 256 tiles; whole rounds of tiles, then the
 // left-over tiles with their K range split between workgroups): true when the shape qualifies and the model
 // expects a gain over the best ordinary launch; `plan` is filled either way.  Modelled time: the whole rounds and the
-// split round at the cost of a 256 x 256 tile on a full chip, and the finishing launch (8 us, and 3 us per
-// accumulator image it adds; 20 us measured for 64 tiles of 4 images).
+// split round as launches of 256 x 256 tiles, and the finishing launch (8 us, and 3 us per accumulator image it
+// adds; 20 us measured for 64 tiles of 4 images).
 static int streamk_cus() { return device_cus() / 8 * 8; }
 static bool streamk_wanted(int64_t n, int64_t batch, int64_t k, bool k_strided, StreamKPlan* plan) {
   *plan = StreamKPlan{0, 0, 0};
@@ -175,8 +180,8 @@ static bool streamk_wanted(int64_t n, int64_t batch, int64_t k, bool k_strided, 
   if (plan->splits < 2) return false;
   double best = 0.0;
   pick_syrk_tile(n, batch, k, false, &best);
-  const double sk = plan->rounds * (16.5 + 1.37 * kt) + 16.5 + 1.37 * (double)ceil_div(kt, plan->splits) + 8.0 +
-                    3.0 * plan->splits;
+  const double sk = (plan->rounds ? COST_256((int64_t)plan->rounds * cus, cus, (double)kt) : 0.0) +
+                    COST_256((int64_t)plan->rem * plan->splits, cus, (double)ceil_div(kt, plan->splits)) + 8.0 + 3.0 * plan->splits;
   return sk < 0.97 * best;
 }
 // 256 x 128 instead of 256 x 256 GEMM tiles for the whole product?
@@ -188,10 +193,10 @@ static bool gemm_prefers_half_tiles(int64_t m, int64_t n, int64_t batch) {
 template <bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
 static int launch_class(TileClass tc, const GemmParams& p, int64_t batch, hipStream_t stream) {
   const bool k_ok = p.K % 64 == 0 && p.K >= 64;
-  // (small matrices stay on the general kernel: measured on batches of 256- and 512-row lower-triangle products, the
-  // direct-to-LDS kernel with 128-row tiles is 10 - 50 % slower there, its prologue and staged epilogue outweigh the
-  // 16 - 32 K tiles of such a product)
-  const bool big = p.M >= 1024 && p.N >= 1024;
+  // Lower-triangle products of 256 rows and more whose rows are whole 128-row tiles also take the direct-to-LDS
+  // kernels (general kernel 1.25 - 2.45x slower over 129 shapes, n = 256 .. 768, batch 1 .. 64); other small
+  // matrices stay on the general kernel.
+  const bool big = (p.M >= 1024 && p.N >= 1024) || (MODE == MODE_SYRK && p.M >= 256 && p.M % 128 == 0);
   if (k_ok && big) {
     if constexpr (MODE == MODE_SYRK) {
       static_assert(P_KS == Q_KS, "the lower-triangle product reads one operand in one layout");

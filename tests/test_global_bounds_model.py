@@ -353,7 +353,7 @@ def sample(seq, limit):
     return [seq[i] for i in idx]
 
 
-SYRK_NS = [1024, 1032, 1096, 1152, 1280, 1536, 1792, 1800, 2048, 2304, 3072, 4096, 5120, 8192, 8184]
+SYRK_NS = [256, 384, 512, 768, 1024, 1032, 1096, 1152, 1280, 1536, 1792, 1800, 2048, 2304, 3072, 4096, 5120, 8192, 8184]
 SYRK_KS = [64, 128, 192, 1024, 14336]
 
 

@@ -169,6 +169,7 @@ def test_gemm_axpy_batched_tail_split_integer_exact(gpu):
 SYRK_VARIANTS = [
     (1024, 512, False, 128), (1024, 512, True, 128), (1280, 192, True, 128), (4096, 1024, False, 192),
     (2048, 2048, True, 128), (1792, 256, False, 128), (1096, 128, False, 192), (1096, 128, True, 256),
+    (512, 256, False, 128), (768, 1024, True, 128), (384, 128, False, 128), (256, 2048, False, 128),  # small matrices of whole 128-row tiles
 ]
 
 
