@@ -2,7 +2,7 @@
 
 from .. import _hip
 from .batched_syrk import batched_tsyrk_ex, can_use_batched_tsyrk
-from .newton_schulz import fused_muon_update, fused_newton_schulz, fused_supported, gemm_axpy
+from .newton_schulz import frob_normalize, fused_muon_update, fused_newton_schulz, fused_supported, gemm_axpy
 from .syrk import tsyrk_ex, tsyrk_ex_small_matrix
 
 
@@ -25,6 +25,7 @@ __all__ = [
     "HAS_TRITON_340",
     "batched_tsyrk_ex",
     "can_use_batched_tsyrk",
+    "frob_normalize",
     "fused_muon_update",
     "fused_newton_schulz",
     "fused_supported",

@@ -75,6 +75,42 @@ def fused_supported(x: torch.Tensor) -> bool:
     )
 
 
+def frob_normalize(
+    x: torch.Tensor,
+    eps: float = 1e-7,
+    *,
+    normalize_in_double: bool = False,
+    out_dtype: torch.dtype = torch.float32,
+    return_norm: bool = False,
+):
+    """``x / max(||x||_F, eps)`` per matrix of a float32 tensor whose last two dimensions are the matrix (the
+    pre-normalisation of ``newton_schulz``, muon_utils.py:212-222): squares summed in float32 like
+    ``torch.nn.functional.normalize`` or, with ``normalize_in_double``, in float64 (the reference's hook for
+    ill-scaled inputs); result in float32 or bfloat16.  One ``mi_frob_normalize`` call.  With ``return_norm`` also the
+    divisor used per matrix (float32, on the device)."""
+    if not x.is_cuda or x.dtype != torch.float32:
+        raise RuntimeError("frob_normalize needs a float32 tensor on the GPU")
+    if x.dim() < 2 or not x.is_contiguous():
+        raise ValueError("frob_normalize needs a contiguous tensor of at least two dimensions")
+    if out_dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("out_dtype must be float32 or bfloat16")
+    numel = x.shape[-2] * x.shape[-1]
+    batch = x.numel() // numel if numel else 0
+    out = torch.empty_like(x, dtype=out_dtype)
+    norm = torch.empty(max(batch, 1), device=x.device, dtype=torch.float32)
+    if batch == 0:
+        return (out, norm[:0]) if return_norm else out
+    lib = _hip.lib()
+    with torch.cuda.device(x.device):
+        partials = torch.empty(lib.mi_frob_partials_len(batch, numel), device=x.device, dtype=torch.float64)
+        rc = lib.mi_frob_normalize(
+            _launch.ptr(x), batch, numel, float(eps), int(bool(normalize_in_double)), _launch.ptr(out),
+            int(out_dtype == torch.bfloat16), _launch.ptr(partials), _launch.ptr(norm), _hip.current_stream_ptr(x.device),
+        )  # fmt: skip
+    _hip.check(rc)
+    return (out, norm[:batch]) if return_norm else out
+
+
 def fused_newton_schulz(
     x: torch.Tensor,
     coefficients: Sequence[tuple[float, float, float]],

@@ -73,6 +73,28 @@ def test_frob_normalize_random_inputs(gpu, f64):
     np.testing.assert_allclose(got16.float().cpu().numpy(), want16, rtol=2**-7, atol=0)
 
 
+def test_frob_normalize_python_wrapper(gpu):
+    """hip_kernels.frob_normalize against torch.nn.functional.normalize over the flattened matrix (what the
+    reference's driver calls, muon_utils.py:219-222) and against the numpy oracle; batch of 3, both output types,
+    float64 accumulation, the divisor handed back."""
+    g = torch.Generator(device=gpu).manual_seed(11)
+    x = torch.randn(3, 256, 520, device=gpu, generator=g) * torch.tensor([1e-3, 1.0, 40.0], device=gpu)[:, None, None]
+    want = torch.nn.functional.normalize(x.flatten(1), p=2, dim=-1, eps=1e-7).view_as(x)
+    got, norm = hip_kernels.frob_normalize(x, return_norm=True)
+    torch.testing.assert_close(got, want, rtol=1e-6, atol=0)
+    torch.testing.assert_close(norm, x.flatten(1).norm(dim=-1), rtol=1e-6, atol=0)
+    got64 = hip_kernels.frob_normalize(x, normalize_in_double=True)
+    want64 = (x.double() / x.double().flatten(1).norm(dim=-1)[:, None, None]).float()
+    torch.testing.assert_close(got64, want64, rtol=2e-7, atol=0)
+    assert np.allclose(got64[1].cpu().numpy(), O.frobenius_normalize(x[1].cpu().numpy(), eps=1e-7, in_double=True), rtol=3e-7, atol=0)
+    bf = hip_kernels.frob_normalize(x, out_dtype=BF)
+    assert bf.dtype == BF and torch.equal(bf, got.to(BF))
+    with pytest.raises(RuntimeError):
+        hip_kernels.frob_normalize(x.cpu())
+    with pytest.raises(ValueError):
+        hip_kernels.frob_normalize(x, out_dtype=torch.float16)
+
+
 def test_frob_normalize_clamp_and_underflow(gpu):
     # all-zero matrix: divisor is eps, result 0, no NaN; dev_norm reports the clamp
     z = torch.zeros(2, 64, 64, device=gpu)
