@@ -33,6 +33,13 @@ int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream, int64_t 
 // CUs of the current device (cached).
 int device_cus();
 
+// 128-row matrices (inst_head_apply.hip): X' = beta X + alpha S X with S = p.P (128 x 128), X = p.Q (128 x p.N,
+// row-major) and, when `gram_next` is given, the float32 partial Gram matrices of X' over slices of 512 columns
+// ([batch][splits][128][128], lower-left three quadrants written).  One workgroup per (matrix, slice); scalars as in
+// the GEMM mode of the tile engine, one partial sum of squares per workgroup at p.slots_out.
+bool head_apply_supported(const GemmParams& p, int64_t batch, int splits);
+int launch_head_apply(const GemmParams& p, int64_t batch, int splits, float* gram_next, bool out_f32, hipStream_t stream);
+
 // Split-tail (stream-K) launch of the lower-triangle kernel (256 x 256 tiles, K-contiguous operands, bf16 output):
 // with `cus` CUs (a multiple of 8), the whole rounds of `cus` tiles run one tile per workgroup, and the K range of each
 // left-over tile is shared between `splits` workgroups (streamk_plan) that park their float32 accumulators in

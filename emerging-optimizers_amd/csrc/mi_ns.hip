@@ -379,7 +379,8 @@ static int syrk_impl(const void* A, int64_t batch, int64_t n, int64_t k, int64_t
 static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void* X, int64_t x_bs,
                           int64_t x_ld, int x_trans, void* Xout, int64_t o_bs, int64_t o_ld, int64_t batch,
                           int64_t m, int64_t n, float alpha, float beta, int out_fp32, float out_scale,
-                          hipStream_t stream, const ShiftArgs* sh = nullptr, float out_accum = 0.0f) {
+                          hipStream_t stream, const ShiftArgs* sh = nullptr, float out_accum = 0.0f, int head_splits = 0,
+                          float* head_gram_next = nullptr, bool* head_used = nullptr) {
   if (!Bm || !X || !Xout) return fail(MI_ERR_BAD_ARG, "mi_gemm_axpy_bf16: null pointer");
   if (batch < 0 || m < 0 || n < 0) return fail(MI_ERR_BAD_ARG, "mi_gemm_axpy_bf16: negative extent");
   if (m % 8 || n % 8) return fail(MI_ERR_UNSUPPORTED_SHAPE, "M and N must be multiples of 8, got M=%lld, N=%lld", (long long)m, (long long)n);
@@ -416,6 +417,12 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
     p.q_bs = x_bs;
     p.M = (int)m;
     p.N = (int)n;
+    // 128-row matrices inside the driver: one workgroup per 512-column slice does product, addend and the next
+    // group's partial Gram matrices on slabs it keeps in LDS
+    if (head_splits > 0 && head_apply_supported(p, batch, head_splits)) {
+      if (head_used) *head_used = true;
+      return launch_head_apply(p, batch, head_splits, out_fp32 ? nullptr : head_gram_next, out_fp32 != 0, stream);
+    }
     // Tile-count quantisation: T full 256 x 256 tiles over C compute units leave a last round that is at most half
     // full when 0 < T mod C <= C/2.  If that remainder is a whole number of tile columns or of tile rows (of every
     // matrix of the batch), those run as 256 x 128 tiles in a second launch: twice as many workgroups, one short round
@@ -1170,9 +1177,12 @@ static int small_gram(const uint16_t* X, int64_t batch, int64_t m, int64_t n, in
 // Partials, then everything up to the multiplier of the B X product in one launch (128-row matrices only).
 static int small_chain(const uint16_t* X, int64_t batch, int64_t n, int splits, float* partials, const float* slots_in,
                        int nslots_in, float* shift_io, const float* xscale, const float* abc, int group, uint16_t* out,
-                       hipStream_t stream) {
-  int rc = small_gram_partials(X, batch, CH_M, n, splits, partials, stream);
-  if (rc != MI_OK) return rc;
+                       hipStream_t stream, bool have_partials) {
+  // (the product that ended the previous group may have left the partials of its result already)
+  if (!have_partials) {
+    int rc = small_gram_partials(X, batch, CH_M, n, splits, partials, stream);
+    if (rc != MI_OK) return rc;
+  }
   ChainArgs a{};
   a.partials = partials;
   a.splits = splits;
@@ -1359,6 +1369,7 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
   int cur = 0;
   int nslots = 1;  // the normalisation kernel left one value per matrix
   bool want_group = true;
+  bool have_partials = false;  // the partial Gram matrices of xbuf[cur] are in the workspace already
   for (int s = 0; s < steps;) {
     const float a = abc[3 * s], b = abc[3 * s + 1], c = abc[3 * s + 2];
     const int taken = ns_group_size(w.pairs, abc, steps, s, want_group);
@@ -1374,7 +1385,7 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
       {
         ProfScope prof(PROF_GRAM, stream);
         rc = small_chain(xbuf[cur], batch, n, w.gram_splits, reinterpret_cast<float*>(ws + w.gpart), slots, nslots, shift, xs,
-                         abc + 3 * s, taken, poly, stream);
+                         abc + 3 * s, taken, poly, stream, have_partials);
       }
       if (rc != MI_OK) return rc;
       mult = poly;
@@ -1463,8 +1474,11 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
     sh_apply.slot_capacity = (int)w.max_slots;
     {
       ProfScope prof(PROF_APPLY, stream);
+      bool head_used = false;
       rc = gemm_axpy_impl(mult, g_bs, m, xbuf[cur], x_bs, ld, trans, dst, x_bs, ld, batch, m, n, alpha, taken > 1 ? 1.0f : a,
-                          last ? 1 : 0, last ? out_scale : 1.0f, stream, &sh_apply, (last && !tall) ? out_accum : 0.0f);
+                          last ? 1 : 0, last ? out_scale : 1.0f, stream, &sh_apply, (last && !tall) ? out_accum : 0.0f,
+                          chain ? w.gram_splits : 0, reinterpret_cast<float*>(ws + w.gpart), &head_used);
+      have_partials = head_used && !last;
     }
     if (rc != MI_OK) return rc;
     nslots = g_last_launch.tiles;

@@ -303,3 +303,86 @@ def test_syrk_epilogue_lower_only_on_a_diagonal_tile(tile, npass):
     out, (m0, n0) = syrk_epilogue_model(tile, 16, npass, diag=True, skip_upper=True)
     tm = tile // 2
     assert out == {(m0 + a, n0 + b): ("v", a, b) for a in range(tile) for b in range(tile) if b < (a // tm + 1) * tm}
+
+
+# ---- per-head product kernel (inst_head_apply.hip): a 128 x 128 slab of X in the K-strided tile layout ----
+#
+# The slab is parked by `park_slab` (row k = thread / 16 + 16 u, chunk = thread % 16, rotated by ks_rot), read as the
+# Q operand of S X with `fast_frag16_ks<128>` for four k-steps (128 k-rows instead of the 64 of a ring slot), read and
+# overwritten in place by the epilogue (row m, four columns), written out row-wise, and read as both operands of
+# X' X'^T with plain 16-byte reads.  This restates each of them and checks them against each other.
+HA_M, HA_W = 128, 128
+HA_ROWB, HA_CH = HA_W * 2, HA_W // 8
+
+
+def ha_chunk(k, c8):
+    return k * HA_ROWB + ((c8 + ks_rot(16, k)) & (HA_CH - 1)) * 16
+
+
+def test_head_apply_slab_layout():
+    # park: every 16-byte chunk of the slab once, at an address of its own (512 threads, four chunks each)
+    lds = {}
+    for tid in range(512):
+        for u in range(4):
+            k, c8 = (tid >> 4) + 32 * u, tid & 15
+            at = ha_chunk(k, c8)
+            assert 0 <= at < HA_M * HA_ROWB and at % 16 == 0 and at // 16 not in lds
+            lds[at // 16] = (k, c8)
+    assert len(lds) == HA_M * HA_CH
+    elem = {}  # byte address of a bf16 -> (k, column)
+    for pos, (k, c8) in lds.items():
+        for e in range(8):
+            elem[pos * 16 + 2 * e] = (k, 8 * c8 + e)
+    # Q fragments of S X: fragment (j, q), lane l must end up with X[32 q + 8 (l / 16) + 0 .. 7][16 j + l % 16]
+    for j in range(HA_W // 16):
+        for q in range(HA_M // 32):
+            a_lo, a_hi = [], []
+            for lane in range(64):
+                g, i16 = lane >> 4, lane & 15
+                kk, cq = i16 >> 2, i16 & 3
+                s = ((cq >> 1) + 2 * kk + 8 * g) * 16 + (cq & 1) * 8  # ks16_consts with wave_row_base = 0
+                r0 = (8 * g + kk) * HA_ROWB
+                a_lo.append((((s + 2 * j * 16) & (HA_ROWB - 1)) | r0) + 32 * q * HA_ROWB)
+                a_hi.append((((s + (2 * j + 8) * 16) & (HA_ROWB - 1)) | r0) + (32 * q + 4) * HA_ROWB)
+            lo, hi = tr_read(elem, a_lo), tr_read(elem, a_hi)
+            for lane in range(64):
+                want = [(32 * q + 8 * (lane >> 4) + e, 16 * j + (lane & 15)) for e in range(8)]
+                assert lo[lane] + hi[lane] == want
+            for addrs in (a_lo, a_hi):  # one pass = 32 lanes of an 8-byte read: every bank at most once
+                for p0 in (0, 32):
+                    banks = [((addrs[lane] + 4 * w) // 4) % 64 for lane in range(p0, p0 + 32) for w in range(2)]
+                    assert max(banks.count(x) for x in set(banks)) == 1
+    # epilogue (8 wavefronts of 16 rows): a lane's four columns of row m are 8 contiguous bytes inside one chunk, each
+    # element owned by one lane; the slab of X' uses the same addresses
+    owners = {}
+    for wave in range(8):
+        for lane in range(64):
+            for j in range(8):
+                m, n = 16 * wave + (lane & 15), 16 * j + 4 * (lane >> 4)
+                at = ha_chunk(m, n >> 3) + (n & 7) * 2
+                assert at % 8 == 0
+                for r in range(4):
+                    assert elem[at + 2 * r] == (m, n + r)
+                    assert (m, n + r) not in owners
+                    owners[(m, n + r)] = (wave, lane)
+    assert len(owners) == HA_M * HA_W
+    # operands of X' X'^T: fragment rows 16 w + l % 16, k-step q: columns 32 q + 8 (l / 16) .. + 7 in one chunk
+    for w in range(8):
+        for q in range(4):
+            for lane in range(64):
+                row = 16 * w + (lane & 15)
+                at = ha_chunk(row, 4 * q + (lane >> 4))
+                assert [elem[at + 2 * e] for e in range(8)] == [(row, 32 * q + 8 * (lane >> 4) + e) for e in range(8)]
+    # the partial Gram matrix: wavefront w writes rows 16 w .. + 15, column blocks 0 .. w: the lower triangle, each
+    # element once
+    seen = set()
+    for wave in range(8):
+        for lane in range(64):
+            for j in range(wave + 1):
+                m, n = 16 * wave + (lane & 15), 16 * j + 4 * (lane >> 4)
+                for r in range(4):
+                    assert (m, n + r) not in seen and m * HA_M + n + r < HA_M * HA_M
+                    seen.add((m, n + r))
+    assert all((m, n) in seen for m in range(HA_M) for n in range(m + 1))
+    # and every float4 the chain kernel adds (groups of four columns starting at j <= i) lies inside what is written
+    assert all((i, j + e) in seen for i in range(HA_M) for j in range(0, HA_M, 4) if j <= i for e in range(4))
