@@ -66,6 +66,10 @@ SYRK_WORKLOADS = {
     "syrk_4x4096x4096": (4, 4096, 4096),
     "syrk_32x512x2048": (32, 512, 2048),
     "syrk_64x256x1024": (64, 256, 1024),
+    # the Gram product of the headline shape alone, operand stored row-major (K-contiguous) and transposed (K-strided:
+    # the reference's TRANS layout, triton_kernels/syrk.py:200-207 there)
+    "syrk_4096x14336": (1, 4096, 14336),
+    "syrk_4096x14336_trans": (1, 4096, 14336),
 }
 STEP_WORKLOADS = {
     "muon_step": (4096, 14336),      # whole Muon.step() (momentum 0.95, Nesterov, weight decay) on the headline gradient
@@ -73,7 +77,8 @@ STEP_WORKLOADS = {
     "muon_heads": (32, 128, 4096),   # Muon.step() over 32 separate 128 x 4096 parameters, one batched orthogonalisation
 }
 DEFAULT_OTHERS = ["attn", "batched_syrk", "per_head", "moe_shard", "moe", "muon_step", "muon_step_attn", "mlp_tall",
-                  "syrk_8x2048x2048", "syrk_4x4096x4096", "syrk_32x512x2048", "syrk_64x256x1024", "muon_heads"]
+                  "syrk_8x2048x2048", "syrk_4x4096x4096", "syrk_32x512x2048", "syrk_64x256x1024", "syrk_4096x14336",
+                  "syrk_4096x14336_trans", "muon_heads"]
 ALL_WORKLOADS = list(NS_WORKLOADS) + list(SYRK_WORKLOADS) + list(STEP_WORKLOADS)
 
 
@@ -207,6 +212,9 @@ def run_syrk_workload(name, warmup, iters, dev):
 
     b, n, k = SYRK_WORKLOADS[name]
     a = (torch.randn(b, n, k, device=dev, generator=torch.Generator(device=dev).manual_seed(0)) * 0.02).to(torch.bfloat16)
+    trans = name.endswith("_trans")
+    if trans:
+        a = a.mT.contiguous().mT  # same values, stored as k rows of n
     out = torch.empty(b, n, n, dtype=torch.bfloat16, device=dev)
     wall, per = time_events(lambda: batched_tsyrk_ex(a, out=out), warmup, iters)
     nref = min(b, 2)
@@ -216,7 +224,7 @@ def run_syrk_workload(name, warmup, iters, dev):
     med, mn = statistics.median(per), min(per)
     flop = b * n * n * k
     return {
-        "workload": f"batched_tsyrk_ex on {b}x{n}x{k} bf16 ({name})",
+        "workload": f"batched_tsyrk_ex on {b}x{n}x{k} bf16{', operand stored transposed' if trans else ''} ({name})",
         "ms_median": round(med, 4), "ms_min": round(mn, 4), "ms_wall": round(wall, 4), "iters": iters,
         "tflops_sym": round(flop / med / 1e9, 1), "pct_peak": round(100 * flop / med / 1e9 / PEAK_BF16_TFLOPS, 2),
         "rel_fro": round(rel, 6), "bitwise_symmetric": sym, "parity": "ok" if (rel <= TOL and sym) else "FAILED",

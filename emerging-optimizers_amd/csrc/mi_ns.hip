@@ -419,7 +419,8 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
     p.N = (int)n;
     // 128-row matrices inside the driver: one workgroup per 512-column slice does product, addend and the next
     // group's partial Gram matrices on slabs it keeps in LDS
-    if (head_splits > 0 && head_apply_supported(p, batch, head_splits)) {
+    const char* head_env = getenv("MI_HEAD_APPLY");  // "0": the general GEMM+AXPY kernels also for 128-row matrices (A/B runs, tests)
+    if (head_splits > 0 && !(head_env && head_env[0] == '0') && head_apply_supported(p, batch, head_splits)) {
       if (head_used) *head_used = true;
       return launch_head_apply(p, batch, head_splits, out_fp32 ? nullptr : head_gram_next, out_fp32 != 0, stream);
     }

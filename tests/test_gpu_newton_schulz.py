@@ -464,3 +464,27 @@ def test_muon_step_keeps_the_statement_path_when_something_watches_the_update(gp
         p.grad = torch.randn_like(p)
         cls([p], use_syrk=True, **kw).step()
     assert calls == []
+
+
+@pytest.mark.parametrize("shape", [(32, 128, 4096), (3, 128, 1024), (1, 128, 2048), (5, 4096, 128)])
+@pytest.mark.parametrize("coefficient_type", ["simple", "quintic", "polar_express"])
+def test_per_head_slab_kernel_against_the_general_kernels(gpu, monkeypatch, shape, coefficient_type):
+    """128-row matrices: the product that ends a group of steps, and the partial Gram matrices of its result, come from
+    the slab kernel (inst_head_apply.hip).  MI_HEAD_APPLY=0 sends the same call through the general GEMM+AXPY kernel
+    and a separate Gram kernel.  The two differ in how the sum of squares behind the diagonal shift is split into
+    partial sums (one per 512-column slice against one per 256-column tile), i.e. in the last bits of the shift, which
+    moves a few bf16 roundings: measured 0 to 6e-5 apart for the "simple" and "quintic" coefficients and up to 2.7e-3
+    for "polar_express", whose first step (a = 8.2) amplifies rounding noise most -- inside the distance of either from
+    float32, not bit for bit.  A batch entry equals the matrix computed alone, bit for bit."""
+    x = torch.randn(*shape, device=gpu, generator=torch.Generator(device=gpu).manual_seed(21)) * 3e-3
+    with utils.fp32_matmul_precision("medium"):
+        monkeypatch.delenv("MI_HEAD_APPLY", raising=False)
+        new = muon_utils.newton_schulz(x, steps=5, coefficient_type=coefficient_type, use_syrk=True)
+        alone = muon_utils.newton_schulz(x[-1], steps=5, coefficient_type=coefficient_type, use_syrk=True)
+        monkeypatch.setenv("MI_HEAD_APPLY", "0")
+        old = muon_utils.newton_schulz(x, steps=5, coefficient_type=coefficient_type, use_syrk=True)
+    assert torch.isfinite(new).all()
+    diff = rel_fro(new, old)
+    print(f"\n  {shape} {coefficient_type}: slab kernel vs general kernels rel_fro = {diff:.2e}")
+    assert diff <= (5e-3 if coefficient_type == "polar_express" else 2e-4)
+    assert torch.equal(new[-1], alone)
