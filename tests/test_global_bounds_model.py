@@ -628,3 +628,46 @@ def test_split_tail_schedule(batch, n, k, cus):
         for x in range(8):
             mine = [tile for bid, tile, k0, *_ in parts if bid % 8 == x and k0 == 0]
             assert mine == list(range(mine[0], mine[0] + len(mine))) if mine else True
+
+
+# ------------------------------------------------------------------ per-head slab kernel (inst_head_apply.hip)
+@pytest.mark.parametrize("batch,n", [(32, 4096), (3, 1024), (1, 2048), (5, 512)])
+def test_head_apply_global_accesses(batch, n):
+    """One workgroup of 512 threads per (matrix, 512-column slice): every global access of S (128 x 128), of X and X'
+    (128 x n), of the partial Gram matrices ([batch][slices][128][128] float32) and of the partial sums of squares
+    ([batch][slices]) lies inside its array, every element of X' is written once, and the partial Gram matrix of
+    every slice has its lower triangle written once."""
+    m, split, w = 128, 512, 128
+    splits = n // split
+    assert n % split == 0
+    tid = np.arange(512)
+    lane, wave = tid & 63, tid >> 6
+    # S fragments: 16 bytes at row 16 wave + lane % 16, k = 32 q + 8 (lane / 16)
+    for q in range(4):
+        row, k = 16 * wave + (lane & 15), 32 * q + 8 * (lane >> 4)
+        assert (row < m).all() and (k + 8 <= m).all()
+    written = np.zeros((batch, m, n), dtype=np.int32)
+    for wg in sample(range(batch * splits), 6):
+        b, s = divmod(wg, splits)
+        assert b < batch
+        for t in range(split // w):
+            for u in range(4):  # slab <-> threads, loads of X and stores of the bf16 X'
+                row, col = (tid >> 4) + 32 * u, s * split + t * w + 8 * (tid & 15)
+                assert (row < m).all() and (col + 8 <= n).all()
+                for r, c in zip(row, col):
+                    written[b, r, c:c + 8] += 1
+            for j in range(8):  # float32 stores of the last group: row 16 wave + lane % 16, four columns
+                row, col = 16 * wave + (lane & 15), s * split + t * w + 16 * j + 4 * (lane >> 4)
+                assert (row < m).all() and (col + 4 <= n).all()
+        assert (written[b, :, s * split:(s + 1) * split] == 1).all()
+        # partial Gram matrix of slice (b, s): wavefront w, column blocks 0 .. w
+        g = np.zeros((m, m), dtype=np.int32)
+        for wv in range(8):
+            for j in range(wv + 1):
+                for ln in range(64):
+                    r, c = 16 * wv + (ln & 15), 16 * j + 4 * (ln >> 4)
+                    off = (b * splits + s) * m * m + r * m + c
+                    assert 0 <= off and off + 4 <= batch * splits * m * m
+                    g[r, c:c + 4] += 1
+        assert (np.tril(g) == np.tril(np.ones_like(g))).all() and g.max() == 1
+        assert b * splits + s < batch * splits  # slot of the partial sum of squares
