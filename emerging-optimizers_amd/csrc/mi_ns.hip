@@ -982,8 +982,51 @@ __global__ void __launch_bounds__(256) gram_reduce_kernel(const float* __restric
 // ---------------------------------------------------------------------------------------------
 static constexpr int CH_M = 128;                       // matrix size served
 static constexpr int CH_BYTES = CH_M * CH_M * 2;       // one matrix in LDS
+static constexpr int CH_THREADS = 1024;                // 16 wavefronts per workgroup
 __device__ __forceinline__ int ch_off(int row, int chunk) { return row * (CH_M * 2) + (((chunk ^ row) & 15) << 4); }
 __device__ __forceinline__ int ch_elem(int row, int col) { return ch_off(row, col >> 3) + (col & 7) * 2; }
+
+// Mirror image of an LDS matrix whose lower triangle (diagonal included) is complete: the 16 x 16 blocks on and
+// below the diagonal are dealt out to the 16 wavefronts; a wavefront reads a block with the LDS transpose read (16
+// lanes fetch 4 rows x 16 columns, 8 bytes each, and lane i receives column i of those four rows) and stores it
+// transposed, 8 bytes per lane.  In a diagonal block only what lies right of the diagonal is stored.
+__device__ __forceinline__ void chain_mirror(char* mat, int wave, int lane) {
+  typedef s16x4_t __attribute__((address_space(3))) * lds_tr_ptr;
+  const uint32_t base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)mat;
+  const int patch = lane >> 4, i16 = lane & 15;  // rows 4 patch .. + 3 of the block; source lane / destination row
+  constexpr int BLOCKS = (CH_M / 16) * (CH_M / 16 + 1) / 2;  // 36
+  constexpr int PER_WAVE = (BLOCKS + CH_THREADS / 64 - 1) / (CH_THREADS / 64);  // 3
+  uint2 t[PER_WAVE];
+  int bi[PER_WAVE], bj[PER_WAVE];
+  // (`wave` is uniform: the block indices live in scalar registers; all reads are issued before the first store)
+#pragma unroll
+  for (int u = 0; u < PER_WAVE; ++u) {
+    const int sb = wave + u * (CH_THREADS / 64);
+    int r = 0;
+#pragma unroll
+    for (int c = 1; c < CH_M / 16; ++c) r += (c * (c + 1) / 2 <= sb) ? 1 : 0;  // largest r with r (r + 1) / 2 <= sb
+    bi[u] = r;
+    bj[u] = sb - r * (r + 1) / 2;
+    if (sb < BLOCKS) {
+      const int src_row = 16 * bi[u] + 4 * patch + (i16 >> 2), src_col = 16 * bj[u] + 4 * (i16 & 3);
+      t[u] = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(uintptr_t)(base + ch_elem(src_row, src_col))));
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < PER_WAVE; ++u) {
+    if (wave + u * (CH_THREADS / 64) >= BLOCKS) continue;
+    // lane i16 holds source rows 16 bi + 4 patch + 0 .. 3 at source column 16 bj + i16
+    const int dst_row = 16 * bj[u] + i16, dst_col = 16 * bi[u] + 4 * patch;
+    if (bi[u] != bj[u] || dst_col > dst_row) {
+      *reinterpret_cast<uint2*>(mat + ch_elem(dst_row, dst_col)) = t[u];
+    } else if (dst_col + 3 > dst_row) {
+      const uint16_t e[4] = {(uint16_t)(t[u].x & 0xffffu), (uint16_t)(t[u].x >> 16), (uint16_t)(t[u].y & 0xffffu), (uint16_t)(t[u].y >> 16)};
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (dst_col + r > dst_row) *reinterpret_cast<uint16_t*>(mat + ch_elem(dst_row, dst_col + r)) = e[r];
+    }
+  }
+}
 
 // dst = alpha * P Q^T + beta1 * C1 + beta2 * C2 on the lower triangle, mirrored; all operands are LDS matrices.
 // Wavefront w of the 16 owns the 32 x 32 block (w / 4, w % 4); the six blocks above the diagonal are only ever
@@ -996,6 +1039,14 @@ __device__ __forceinline__ void chain_product(const char* P, const char* Q, cons
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[e] = 0.0f;
     const int frow = lane & 31, fk = lane >> 5;
+    // the addends do not depend on the product: their reads go out first and arrive behind the MFMAs
+    uint2 c1[4], c2[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int m = ti * 32 + frow, n = tj * 32 + 8 * g + 4 * fk;
+      c1[g] = *reinterpret_cast<const uint2*>(C1 + ch_elem(m, n));
+      c2[g] = C2 != nullptr ? *reinterpret_cast<const uint2*>(C2 + ch_elem(m, n)) : make_uint2(0u, 0u);
+    }
 #pragma unroll
     for (int q = 0; q < CH_M / 16; ++q) {
       const bf16x8_t fp = *reinterpret_cast<const bf16x8_t*>(P + ch_off(ti * 32 + frow, 2 * q + fk));
@@ -1009,27 +1060,29 @@ __device__ __forceinline__ void chain_product(const char* P, const char* Q, cons
       f32x4_t v;
 #pragma unroll
       for (int r = 0; r < 4; ++r) v[r] = alpha * acc[4 * g + r];
-      const uint2 c1 = *reinterpret_cast<const uint2*>(C1 + ch_elem(m, n));
-      v[0] = __builtin_fmaf(beta1, __uint_as_float(c1.x << 16), v[0]);
-      v[1] = __builtin_fmaf(beta1, __uint_as_float(c1.x & 0xffff0000u), v[1]);
-      v[2] = __builtin_fmaf(beta1, __uint_as_float(c1.y << 16), v[2]);
-      v[3] = __builtin_fmaf(beta1, __uint_as_float(c1.y & 0xffff0000u), v[3]);
+      v[0] = __builtin_fmaf(beta1, __uint_as_float(c1[g].x << 16), v[0]);
+      v[1] = __builtin_fmaf(beta1, __uint_as_float(c1[g].x & 0xffff0000u), v[1]);
+      v[2] = __builtin_fmaf(beta1, __uint_as_float(c1[g].y << 16), v[2]);
+      v[3] = __builtin_fmaf(beta1, __uint_as_float(c1[g].y & 0xffff0000u), v[3]);
       if (C2 != nullptr) {
-        const uint2 c2 = *reinterpret_cast<const uint2*>(C2 + ch_elem(m, n));
-        v[0] = __builtin_fmaf(beta2, __uint_as_float(c2.x << 16), v[0]);
-        v[1] = __builtin_fmaf(beta2, __uint_as_float(c2.x & 0xffff0000u), v[1]);
-        v[2] = __builtin_fmaf(beta2, __uint_as_float(c2.y << 16), v[2]);
-        v[3] = __builtin_fmaf(beta2, __uint_as_float(c2.y & 0xffff0000u), v[3]);
+        v[0] = __builtin_fmaf(beta2, __uint_as_float(c2[g].x << 16), v[0]);
+        v[1] = __builtin_fmaf(beta2, __uint_as_float(c2[g].x & 0xffff0000u), v[1]);
+        v[2] = __builtin_fmaf(beta2, __uint_as_float(c2[g].y << 16), v[2]);
+        v[3] = __builtin_fmaf(beta2, __uint_as_float(c2[g].y & 0xffff0000u), v[3]);
       }
       const uint2 h = __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));
-      const uint16_t e[4] = {(uint16_t)(h.x & 0xffffu), (uint16_t)(h.x >> 16), (uint16_t)(h.y & 0xffffu), (uint16_t)(h.y >> 16)};
+      if (n + 3 <= m) {
+        *reinterpret_cast<uint2*>(dst + ch_elem(m, n)) = h;  // four columns on or below the diagonal
+      } else {
+        const uint16_t e[4] = {(uint16_t)(h.x & 0xffffu), (uint16_t)(h.x >> 16), (uint16_t)(h.y & 0xffffu), (uint16_t)(h.y >> 16)};
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        if (n + r <= m) *reinterpret_cast<uint16_t*>(dst + ch_elem(m, n + r)) = e[r];
-        if (n + r < m) *reinterpret_cast<uint16_t*>(dst + ch_elem(n + r, m)) = e[r];
+        for (int r = 0; r < 4; ++r)
+          if (n + r <= m) *reinterpret_cast<uint16_t*>(dst + ch_elem(m, n + r)) = e[r];
       }
     }
   }
+  __syncthreads();  // the lower triangle of dst is complete
+  chain_mirror(dst, wave, lane);
   __syncthreads();  // dst is complete, and nobody still reads what the next product overwrites
 }
 
@@ -1045,97 +1098,151 @@ struct ChainArgs {
   uint16_t* out;          // [batch][128][128] bf16: the multiplier S_g of X (R_1 for a single step)
 };
 
+// One product of the chain: operands, addends and destination as indices of the four LDS matrices (-1: none).
+struct ChainOp {
+  int p, q, c1, c2, dst;
+  float alpha, beta1, beta2;
+};
+static constexpr int CH_MAX_OPS = 12;  // a group of three steps has 9 products
+
 // 16 wavefronts per workgroup, one per 32 x 32 block of the products; together they stream the float32 partials in
 // (the only part that touches HBM; one workgroup per matrix leaves most of the chip idle, so each one needs many
-// loads in flight) and the result out.
-static constexpr int CH_THREADS = 1024;
+// loads in flight) and the result out.  The products of the chain run as a loop over a small table, so that the code
+// of a product exists once and stays in the instruction cache (spelled out nine times, every product was a cold walk
+// through new code: 2 us each instead of 1).
 __global__ void __launch_bounds__(CH_THREADS) small_chain_kernel(ChainArgs a) {
   __shared__ __align__(16) char chain_lds[4 * CH_BYTES];
   __shared__ float red[CH_THREADS / 64];
+  __shared__ ChainOp ops[CH_MAX_OPS];
+  __shared__ int nops_lds, result_lds;
   const int64_t b = blockIdx.x;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: what depends on it alone branches on the scalar unit
   char* B0 = chain_lds;
-  char* B1 = chain_lds + CH_BYTES;
-  char* B2 = chain_lds + 2 * CH_BYTES;
-  char* B3 = chain_lds + 3 * CH_BYTES;
-  // shift and input scale of this matrix, as gram_reduce_kernel resolves them
-  float part = 0.0f;
-  for (int i = tid; i < a.nslots_in; i += CH_THREADS) part += a.slots_in[b * a.nslots_in + i];
-  const float s = block_sum_f32<CH_THREADS>(part, red) / (float)CH_M;
-  if (tid == 0) a.shift_io[b] = s;
-  const float r = a.xscale ? a.xscale[b] : 1.0f;
-  // D -> B0: four consecutive columns per thread and step, the slices added in their fixed order
+  // D -> B0.  Only the groups of four columns that start on or left of the diagonal are needed: 33 per pair of rows
+  // (p, 127 - p), 2112 in all.  Every thread takes two of them, with all slices (up to 8 at a time) in flight at once;
+  // the 64 groups left over are fetched slice by slice by 512 threads, parked in LDS (in a matrix buffer that is
+  // still free) and added up, in slice order like the others, by 64 threads.  The shift is summed while the loads fly.
   const float* __restrict__ src = a.partials + b * a.splits * (int64_t)(CH_M * CH_M);
-  constexpr int GROUPS = CH_M * CH_M / 4, PER_THREAD = GROUPS / CH_THREADS, DEPTH = 4;
-  f32x4_t sum[PER_THREAD];
+  constexpr int PAIR_GROUPS = CH_M / 4 + 1, LOWER_GROUPS = (CH_M / 2) * PAIR_GROUPS, DEPTH = 8;
+  static_assert(LOWER_GROUPS > 2 * CH_THREADS && LOWER_GROUPS - 2 * CH_THREADS <= 64, "two groups per thread and at most 64 left over");
+  constexpr int EXTRA = LOWER_GROUPS - 2 * CH_THREADS;
+  auto group_of = [](int g, int& i, int& j) {  // g-th needed group -> row i, first column j
+    const int pair = g / PAIR_GROUPS, r = g % PAIR_GROUPS, n_lo = pair / 4 + 1;
+    i = r < n_lo ? pair : CH_M - 1 - pair;
+    j = 4 * (r < n_lo ? r : r - n_lo);
+  };
+  int gi[3], gj[3];
+  group_of(tid, gi[0], gj[0]);
+  group_of(tid + CH_THREADS, gi[1], gj[1]);
+  group_of(2 * CH_THREADS + (tid < EXTRA ? tid : 0), gi[2], gj[2]);
+  int xi, xj;  // the left-over group this thread fetches one slice of
+  group_of(2 * CH_THREADS + ((tid >> 3) < EXTRA ? (tid >> 3) : 0), xi, xj);
+  f32x4_t* parked = reinterpret_cast<f32x4_t*>(chain_lds + CH_BYTES);  // [EXTRA][DEPTH]
+  f32x4_t sum[3];
 #pragma unroll
-  for (int t = 0; t < PER_THREAD; ++t) sum[t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int t = 0; t < 3; ++t) sum[t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  float s = 0.0f;
   for (int sp0 = 0; sp0 < a.splits; sp0 += DEPTH) {
-    f32x4_t v[PER_THREAD][DEPTH];
+    f32x4_t v[2][DEPTH], x = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int t = 0; t < PER_THREAD; ++t) {
-      const int g = tid + t * CH_THREADS, i = g / (CH_M / 4), j = (g % (CH_M / 4)) * 4;
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int u = 0; u < DEPTH; ++u) {
         v[t][u] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-        if (j <= i && sp0 + u < a.splits)
-          v[t][u] = *reinterpret_cast<const f32x4_t*>(src + (int64_t)(sp0 + u) * (CH_M * CH_M) + (int64_t)g * 4);
+        if (sp0 + u < a.splits)
+          v[t][u] = *reinterpret_cast<const f32x4_t*>(src + (int64_t)(sp0 + u) * (CH_M * CH_M) + gi[t] * CH_M + gj[t]);
       }
+    if ((tid >> 3) < EXTRA && sp0 + (tid & 7) < a.splits)
+      x = *reinterpret_cast<const f32x4_t*>(src + (int64_t)(sp0 + (tid & 7)) * (CH_M * CH_M) + xi * CH_M + xj);
+    if (sp0 > 0) __syncthreads();  // the parked slices of the previous round have been added
+    if ((tid >> 3) < EXTRA) parked[tid] = x;
+    if (sp0 == 0) {
+      // shift and input scale of this matrix, as gram_reduce_kernel resolves them (its barriers also publish `parked`)
+      float part = 0.0f;
+      for (int i = tid; i < a.nslots_in; i += CH_THREADS) part += a.slots_in[b * a.nslots_in + i];
+      s = block_sum_f32<CH_THREADS>(part, red) / (float)CH_M;
+      if (tid == 0) a.shift_io[b] = s;
+    } else {
+      __syncthreads();
     }
 #pragma unroll
-    for (int t = 0; t < PER_THREAD; ++t)
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int u = 0; u < DEPTH; ++u)
         if (sp0 + u < a.splits) sum[t] += v[t][u];
-  }
+    if (tid < EXTRA) {
 #pragma unroll
-  for (int t = 0; t < PER_THREAD; ++t) {
-    const int g = tid + t * CH_THREADS, i = g / (CH_M / 4), j = (g % (CH_M / 4)) * 4;
-    if (j > i) continue;  // the whole group lies above the diagonal
+      for (int u = 0; u < DEPTH; ++u)
+        if (sp0 + u < a.splits) sum[2] += parked[tid * DEPTH + u];
+    }
+  }
+  const float r = a.xscale ? a.xscale[b] : 1.0f;
+  __syncthreads();  // (the buffer behind `parked` becomes a matrix again)
+#pragma unroll
+  for (int t = 0; t < 3; ++t) {
+    if (t == 2 && tid >= EXTRA) continue;
+    const int i = gi[t], j = gj[t];
+    f32x4_t d;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      if (j + e > i) continue;
-      float acc = sum[t][e] * (r * r);
-      if (i == j + e) acc -= s;
-      const uint16_t h = __builtin_bit_cast(uint16_t, (__bf16)acc);
-      *reinterpret_cast<uint16_t*>(B0 + ch_elem(i, j + e)) = h;
-      *reinterpret_cast<uint16_t*>(B0 + ch_elem(j + e, i)) = h;
+      d[e] = sum[t][e] * (r * r);
+      if (i == j + e) d[e] -= s;
     }
-  }
-  __syncthreads();
-  // The steps of the group (SHIFT_GROUP_* in gemm_engine.hpp spells out the recursion); D_k stays in B0, the other
-  // three matrices are handed out and returned as what they hold dies.
-  char* pool[3] = {B1, B2, B3};
-  int free_n = 3;
-  char* D = B0;
-  char* S = nullptr;
-  float sk = s, before = 1.0f;
-#pragma unroll
-  for (int k = 0; k < 3; ++k) {
-    if (k >= a.group) break;
-    const float ak = a.co[k][0], bk = a.co[k][1], ck = a.co[k][2];
-    const float e = ak + bk * sk + ck * sk * sk;
-    char* R = pool[--free_n];
-    chain_product(D, D, D, nullptr, R, ck, bk + 2.0f * ck * sk, 0.0f, wave, lane);  // R_k
-    if (k == 0) {
-      S = R;
+    const uint2 h = __builtin_bit_cast(uint2, __builtin_convertvector(d, bf16x4_t));
+    if (j + 3 <= i) {
+      *reinterpret_cast<uint2*>(B0 + ch_elem(i, j)) = h;
     } else {
-      char* Sk = pool[--free_n];
-      chain_product(R, S, S, R, Sk, 1.0f, e, before, wave, lane);                   // S_k
-      pool[free_n++] = S;
-      S = Sk;
+      const uint16_t e[4] = {(uint16_t)(h.x & 0xffffu), (uint16_t)(h.x >> 16), (uint16_t)(h.y & 0xffffu), (uint16_t)(h.y >> 16)};
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (j + q <= i) *reinterpret_cast<uint16_t*>(B0 + ch_elem(i, j + q)) = e[q];
     }
-    if (k + 1 < a.group) {
-      char* T = pool[--free_n];
-      chain_product(R, D, D, R, T, 1.0f, e, sk, wave, lane);                        // T'_k
-      chain_product(R, T, T, R, D, 1.0f, e, e * sk, wave, lane);                    // D_{k+1} over D_k
-      pool[free_n++] = T;
-      sk = e * e * sk;
-    }
-    if (k > 0) pool[free_n++] = R;
-    before *= e;
   }
-  const char* result = S;
+  // The steps of the group (SHIFT_GROUP_* in gemm_engine.hpp spells out the recursion) as a table of products; D_k
+  // stays in matrix 0, the other three are handed out and returned as what they hold dies.
+  if (tid == 0) {
+    int pool[3] = {1, 2, 3};
+    int free_n = 3, n = 0, D = 0, S = -1;
+    float sk = s, before = 1.0f;
+    for (int k = 0; k < 3 && k < a.group; ++k) {
+      const float ak = a.co[k][0], bk = a.co[k][1], ck = a.co[k][2];
+      const float e = ak + bk * sk + ck * sk * sk;
+      const int R = pool[--free_n];
+      ops[n++] = ChainOp{D, D, D, -1, R, ck, bk + 2.0f * ck * sk, 0.0f};  // R_k
+      if (k == 0) {
+        S = R;
+      } else {
+        const int Sk = pool[--free_n];
+        ops[n++] = ChainOp{R, S, S, R, Sk, 1.0f, e, before};  // S_k
+        pool[free_n++] = S;
+        S = Sk;
+      }
+      if (k + 1 < a.group) {
+        const int T = pool[--free_n];
+        ops[n++] = ChainOp{R, D, D, R, T, 1.0f, e, sk};         // T'_k
+        ops[n++] = ChainOp{R, T, T, R, D, 1.0f, e, e * sk};     // D_{k+1} over D_k
+        pool[free_n++] = T;
+        sk = e * e * sk;
+      }
+      if (k > 0) pool[free_n++] = R;
+      before *= e;
+    }
+    nops_lds = n;
+    result_lds = S;
+  }
+  __syncthreads();  // the lower triangle of D and the table are complete
+  chain_mirror(B0, wave, lane);
+  __syncthreads();
+  const int nops = nops_lds;
+#pragma unroll 1
+  for (int o = 0; o < nops; ++o) {
+    const ChainOp op = ops[o];
+    chain_product(chain_lds + op.p * CH_BYTES, chain_lds + op.q * CH_BYTES, chain_lds + op.c1 * CH_BYTES,
+                  op.c2 >= 0 ? chain_lds + op.c2 * CH_BYTES : nullptr, chain_lds + op.dst * CH_BYTES, op.alpha, op.beta1,
+                  op.beta2, wave, lane);
+  }
+  const char* result = chain_lds + result_lds * CH_BYTES;
   uint16_t* __restrict__ ob = a.out + b * (int64_t)(CH_M * CH_M);
   for (int c = tid; c < CH_M * (CH_M / 8); c += CH_THREADS) {
     const int row = c / (CH_M / 8), ch = c % (CH_M / 8);

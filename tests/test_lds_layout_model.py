@@ -386,3 +386,86 @@ def test_head_apply_slab_layout():
     assert all((m, n) in seen for m in range(HA_M) for n in range(m + 1))
     # and every float4 the chain kernel adds (groups of four columns starting at j <= i) lies inside what is written
     assert all((i, j + e) in seen for i in range(HA_M) for j in range(0, HA_M, 4) if j <= i for e in range(4))
+
+
+# ---- chain kernel of the 128-row matrices (small_chain_kernel in mi_ns.hip): lower triangle stored, then mirrored ----
+CH_M = 128
+
+
+def ch_elem(row, col):
+    return row * (CH_M * 2) + ((((col >> 3) ^ row) & 15) << 4) + (col & 7) * 2
+
+
+def chain_mirror_model(lds):
+    """`chain_mirror`: the 36 blocks of 16 x 16 on and below the diagonal, dealt out to 16 wavefronts; transpose read
+    of 4 rows x 16 columns per 16-lane group, 8-byte store of the transposed piece (element-wise right of the diagonal
+    inside a diagonal block).  Returns the set of (row, column) written."""
+    written = []
+    for wave in range(16):
+        for sb in range(wave, 36, 16):
+            bi = 0
+            while (bi + 1) * (bi + 2) // 2 <= sb:
+                bi += 1
+            bj = sb - bi * (bi + 1) // 2
+            assert 0 <= bj <= bi < 8
+            addr = []
+            for lane in range(64):
+                patch, i16 = lane >> 4, lane & 15
+                addr.append(ch_elem(16 * bi + 4 * patch + (i16 >> 2), 16 * bj + 4 * (i16 & 3)))
+            got = tr_read(lds, addr)
+            for lane in range(64):
+                patch, i16 = lane >> 4, lane & 15
+                dst_row, dst_col = 16 * bj + i16, 16 * bi + 4 * patch
+                for r in range(4):
+                    if bi != bj or dst_col + r > dst_row:
+                        # the lane must hold source row 16 bi + 4 patch + r at source column 16 bj + i16 (what a
+                        # diagonal block reads from above the diagonal is not there yet and is not used)
+                        assert got[lane][r] == (16 * bi + 4 * patch + r, 16 * bj + i16)
+                        written.append((dst_row, dst_col + r, got[lane][r]))
+    return written
+
+
+def test_chain_kernel_lower_triangle_then_mirror():
+    # direct phase of a product: wavefront (ti, tj), tj <= ti, lane: row m = 32 ti + lane % 32, four columns from
+    # n = 32 tj + 8 g + 4 (lane / 32); only what lies on or below the diagonal
+    lds, count = {}, {}
+    for wave in range(16):
+        ti, tj = wave >> 2, wave & 3
+        if tj > ti:
+            continue
+        for lane in range(64):
+            for g in range(4):
+                m, n = ti * 32 + (lane & 31), tj * 32 + 8 * g + 4 * (lane >> 5)
+                for r in range(4):
+                    if n + r <= m:
+                        lds[ch_elem(m, n + r)] = (m, n + r)
+                        count[(m, n + r)] = count.get((m, n + r), 0) + 1
+                assert ch_elem(m, n) % 8 == 0 and [ch_elem(m, n + r) for r in range(4)] == [ch_elem(m, n) + 2 * r for r in range(4)]
+    assert count == {(m, n): 1 for m in range(CH_M) for n in range(m + 1)}
+    # the same for the build of D from the partial sums: the groups of four columns that start on or left of the
+    # diagonal are numbered 33 per pair of rows (p, 127 - p); two per thread and 64 left over
+    groups = []
+    for g in range(64 * 33):
+        pair, r = divmod(g, 33)
+        n_lo = pair // 4 + 1
+        groups.append((pair, 4 * r) if r < n_lo else (CH_M - 1 - pair, 4 * (r - n_lo)))
+    assert len(groups) == 2 * 1024 + 64
+    assert sorted(groups) == sorted((i, j) for i in range(CH_M) for j in range(0, CH_M, 4) if j <= i)
+    built = set()
+    for i, j in groups:
+        built.update((i, j + e) for e in range(4) if j + e <= i)
+    assert built == set(count)
+    # mirror phase: everything right of the diagonal, once, and as the transpose of what is stored below it
+    written = chain_mirror_model(lds)
+    assert sorted((r, c) for r, c, _ in written) == [(r, c) for r in range(CH_M) for c in range(r + 1, CH_M)]
+    assert all(src == (c, r) for r, c, src in written)
+    # one pass of the transpose read (32 lanes x 8 bytes) touches every LDS bank at most once
+    for bi in range(8):
+        for bj in range(bi + 1):
+            for half in (0, 32):
+                banks = []
+                for lane in range(half, half + 32):
+                    patch, i16 = lane >> 4, lane & 15
+                    a = ch_elem(16 * bi + 4 * patch + (i16 >> 2), 16 * bj + 4 * (i16 & 3))
+                    banks += [(a // 4) % 64, (a // 4 + 1) % 64]
+                assert max(banks.count(x) for x in set(banks)) <= 2
