@@ -488,3 +488,30 @@ def test_per_head_slab_kernel_against_the_general_kernels(gpu, monkeypatch, shap
     print(f"\n  {shape} {coefficient_type}: slab kernel vs general kernels rel_fro = {diff:.2e}")
     assert diff <= (5e-3 if coefficient_type == "polar_express" else 2e-4)
     assert torch.equal(new[-1], alone)
+
+
+@pytest.mark.parametrize("shape", [(32, 128, 4096), (1024, 4096)])
+def test_fused_call_replays_from_a_hip_graph(gpu, shape):
+    """The single-call driver allocates nothing and records no memset: captured into a HIP graph (its workspace
+    allocated beforehand by a warm-up call), every replay -- with eager work of the same library in between -- gives
+    the bits of the eager call."""
+    x = torch.randn(*shape, device=gpu, generator=torch.Generator(device=gpu).manual_seed(5)) * 1e-3
+    other = torch.randn(2048, 2048, device=gpu).to(torch.bfloat16)
+    with utils.fp32_matmul_precision("medium"):
+        run = lambda: muon_utils.newton_schulz(x, steps=5, coefficient_type="quintic", use_syrk=True)
+        eager = run()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            run()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = run()
+        for _ in range(3):
+            out.fill_(float("nan"))
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager)
+            hip_kernels.tsyrk_ex(other)  # eager work between the replays
+            torch.cuda.synchronize()
