@@ -37,11 +37,8 @@ __global__ void __launch_bounds__(HA_NT) head_apply_kernel(GemmParams p, float* 
   const int s = blockIdx.x % splits;
   const int64_t c_begin = (int64_t)s * HA_SPLIT;
 
-  const Scalars sc = resolve_shift<HA_NT>(p, b, red, s == 0);
-  const float alpha = sc.alpha, beta = sc.beta;
   const uint16_t* __restrict__ X = p.Q + b * p.q_bs;
   const uint16_t* __restrict__ Sm = p.P + b * p.p_bs;
-  const bool use_c = beta != 0.0f && p.Cin != nullptr;  // (the addend is X itself: p.Cin == p.Q)
 
   // S as fragments of the P operand: rows 16 wave + lane % 16, k = 32 q + 8 (lane / 16) .. + 7
   bf16x8_t sfrag[4];
@@ -73,6 +70,10 @@ __global__ void __launch_bounds__(HA_NT) head_apply_kernel(GemmParams p, float* 
 
   float ssq = 0.0f;
   fetch_slab(0);
+  // (the scalars are resolved while the first loads are on their way)
+  const Scalars sc = resolve_shift<HA_NT>(p, b, red, s == 0);
+  const float alpha = sc.alpha, beta = sc.beta;
+  const bool use_c = beta != 0.0f && p.Cin != nullptr;  // (the addend is X itself: p.Cin == p.Q)
   park_slab(slab_in[0]);
   __syncthreads();
   constexpr int SLABS = HA_SPLIT / HA_W;
@@ -92,6 +93,10 @@ __global__ void __launch_bounds__(HA_NT) head_apply_kernel(GemmParams p, float* 
 #pragma unroll
       for (int j = 0; j < 8; ++j)
         acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fast_frag16_ks<HA_W>(cur_lds, ks_s, ks_r, j, q), sfrag[q], acc[j], 0, 0, 0);
+    // The next slab of X goes into the buffer whose readers (fragments and addends of the previous pass) finished
+    // before the barrier of the previous pass.  With float32 output this happens before the epilogue: the wait for
+    // the loads would otherwise also wait for the stores of the epilogue, which share their counter.
+    if constexpr (OUT_F32 && t + 1 < SLABS) park_slab(slab_in[(t + 1) & 1]);
     // ---- epilogue: a lane owns row m = 16 wave + lane % 16, columns n .. n + 3 with n = 16 j + 4 (lane / 16) ----
     const int m = 16 * wave + (lane & 15);
 #pragma unroll
@@ -125,9 +130,7 @@ __global__ void __launch_bounds__(HA_NT) head_apply_kernel(GemmParams p, float* 
         *reinterpret_cast<uint2*>(res + at) = __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));  // same layout as the slab of X
       }
     }
-    // the next slab of X goes into the buffer whose readers (fragments and addends of the previous pass) finished
-    // before the barrier of the previous pass
-    if constexpr (t + 1 < SLABS) park_slab(slab_in[(t + 1) & 1]);
+    if constexpr (!OUT_F32 && t + 1 < SLABS) park_slab(slab_in[(t + 1) & 1]);
     if constexpr (t + 1 < SLABS || !OUT_F32) __syncthreads();  // X' of this pass and X of the next one are complete
     if constexpr (!OUT_F32) {
       // (the buffer of X' is written again two passes on, behind the barrier of the next pass)
