@@ -191,4 +191,171 @@ int launch_head_apply(const GemmParams& p, int64_t batch, int splits, float* gra
   return MI_OK;
 }
 
+// ---------------------------------------------------------------------------------------------
+// The pass over the float32 input of 128-row matrices that starts a call: sum of squares, bf16 cast (unnormalised: the
+// divide by the norm is left to the consumers) and, because the slab that was just cast sits in LDS anyway, the
+// split-K partial Gram matrices of the cast -- the first group of steps then needs no Gram kernel that reads X again.
+// One workgroup per (matrix, slice of 512 columns), slabs of 128 columns as above.
+//
+// FINALIZE = false is that pass.  FINALIZE = true follows it: every workgroup adds the partial sums of its matrix, and
+// for a norm in the range where the divide may be deferred that is all (one thread per matrix leaves norm, scale and
+// the squared norm of the normalised matrix); for a norm outside it the workgroup does the work again on x / norm:
+// the cast and the partial Gram matrices are replaced by those of the normalised matrix, and the scale is 1.
+// ---------------------------------------------------------------------------------------------
+struct HeadFrontArgs {
+  const float* x;     // [batch][128][n] float32 (the gradient, with a momentum source)
+  int64_t n;
+  int splits;         // n / 512
+  float eps;
+  MomentumSrc mom;
+  uint16_t* xb;       // [batch][128][n] bf16
+  double* partials;   // [batch][splits]
+  float* gram;        // [batch][splits][128][128]
+  float* norm;        // [batch] or null
+  float* sumsq_out;   // [batch] or null
+  float* xscale;      // [batch]
+};
+
+template <bool FINALIZE>
+__global__ void __launch_bounds__(HA_NT) head_front_kernel(HeadFrontArgs a) {
+  __shared__ __align__(1024) char slab[2][HA_SLAB_BYTES];
+  __shared__ double red_d[HA_NT / 64];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int64_t b = blockIdx.x / a.splits;
+  const int s = blockIdx.x % a.splits;
+  float divisor = 1.0f;
+  if constexpr (FINALIZE) {
+    double tot = 0.0;
+    for (int i = 0; i < a.splits; ++i) tot += a.partials[b * a.splits + i];  // (same order in every thread and workgroup)
+    divisor = fmaxf(sqrtf((float)tot), a.eps);
+    const bool deferred = divisor >= NORM_DEFER_MIN && divisor <= NORM_DEFER_MAX;  // false for NaN
+    if (s == 0 && tid == 0) {
+      if (a.norm) a.norm[b] = divisor;
+      a.xscale[b] = deferred ? 1.0f / divisor : 1.0f;
+      if (a.sumsq_out) {
+        // squared Frobenius norm of the normalised matrix: 1 unless the divisor was clamped
+        const float ratio = sqrtf((float)tot) / divisor;
+        a.sumsq_out[b] = (divisor > 0.0f && ratio == ratio) ? ratio * ratio : 0.0f;
+      }
+    }
+    if (deferred) return;
+  }
+
+  // slab <-> threads as in head_apply_kernel: 8 columns of row (tid >> 4) + 32 u, chunk tid & 15
+  const int ck = tid >> 4, cc = tid & 15;
+  const int64_t base = b * (int64_t)HA_M * a.n + (int64_t)s * HA_SPLIT + 8 * cc;
+  const float* __restrict__ xs = a.x + base;
+  float* __restrict__ ms = a.mom.buf ? a.mom.buf + base : nullptr;
+  uint16_t* __restrict__ os = a.xb + base;
+  const float keep = 1.0f - a.mom.beta;
+  f32x4_t pre[HA_PRE][2], mpre[HA_PRE][2];
+  auto fetch = [&](int t) {
+#pragma unroll
+    for (int u = 0; u < HA_PRE; ++u) {
+      const int64_t at = (int64_t)(ck + 32 * u) * a.n + t * HA_W;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        pre[u][h] = FINALIZE ? *reinterpret_cast<const f32x4_t*>(xs + at + 4 * h) : stream_load4(xs + at + 4 * h);
+        if (ms) mpre[u][h] = *reinterpret_cast<const f32x4_t*>(ms + at + 4 * h);
+      }
+    }
+  };
+  f32x4_t gacc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) gacc[j] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  f32x4_t ssq = {0.0f, 0.0f, 0.0f, 0.0f};
+  constexpr int SLABS = HA_SPLIT / HA_W;
+  fetch(0);
+  static_for<SLABS>([&](auto tc) {
+    constexpr int t = decltype(tc)::value;
+    char* cur = slab[t & 1];
+#pragma unroll
+    for (int u = 0; u < HA_PRE; ++u) {
+      const int64_t at = (int64_t)(ck + 32 * u) * a.n + t * HA_W;
+      uint2 half[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        f32x4_t v = pre[u][h];
+        if (ms) {
+          f32x4_t m = mpre[u][h];
+          if constexpr (!FINALIZE) {  // (the second pass finds the buffer updated)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) m[e] = torch_lerp(m[e], v[e], keep);
+            *reinterpret_cast<f32x4_t*>(ms + at + 4 * h) = m;
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = momentum_direction(v[e], m[e], a.mom.beta, a.mom.nesterov);
+        }
+        if constexpr (FINALIZE) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = v[e] / divisor;
+        } else {
+          // squares are formed in float32: tiny inputs underflow exactly like a float32 reduction
+#pragma unroll
+          for (int e = 0; e < 4; ++e) ssq[e] = __builtin_fmaf(v[e], v[e], ssq[e]);
+        }
+        half[h] = __builtin_bit_cast(uint2, __builtin_convertvector(v, bf16x4_t));
+      }
+      const u32x4_t chunk = {half[0].x, half[0].y, half[1].x, half[1].y};
+      *reinterpret_cast<u32x4_t*>(os + at) = chunk;
+      *reinterpret_cast<u32x4_t*>(cur + ha_chunk(ck + 32 * u, cc)) = chunk;
+    }
+    if constexpr (t + 1 < SLABS) fetch(t + 1);  // in flight during the products below
+    // One barrier per slab: the buffer written above was last read by the products of two slabs ago, which every
+    // wavefront finished before it arrived at the barrier of the previous slab.
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const bf16x8_t fp = *reinterpret_cast<const bf16x8_t*>(cur + ha_chunk(16 * wave + (lane & 15), 4 * q + (lane >> 4)));
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if (j > wave) continue;  // (uniform)
+        const bf16x8_t fq = *reinterpret_cast<const bf16x8_t*>(cur + ha_chunk(16 * j + (lane & 15), 4 * q + (lane >> 4)));
+        gacc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fq, fp, gacc[j], 0, 0, 0);
+      }
+    }
+  });
+  if constexpr (!FINALIZE) {
+    // the cross-thread tree is carried in float64, so the result does not depend on its shape
+    double v = (double)((ssq[0] + ssq[1]) + (ssq[2] + ssq[3]));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+    if (lane == 0) red_d[wave] = v;
+    __syncthreads();
+    if (tid == 0) {
+      double tot = 0.0;
+      for (int w = 0; w < HA_NT / 64; ++w) tot += red_d[w];
+      a.partials[b * a.splits + s] = tot;
+    }
+  }
+  float* __restrict__ g = a.gram + (b * a.splits + s) * (int64_t)(HA_M * HA_M);
+  const int m = 16 * wave + (lane & 15);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    if (j > wave) continue;
+    *reinterpret_cast<f32x4_t*>(g + (int64_t)m * HA_M + 16 * j + 4 * (lane >> 4)) = gacc[j];
+  }
+}
+
+static inline bool ha_aligned16(const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15u) == 0; }
+
+bool head_front_supported(const float* x, int64_t batch, int64_t n, const MomentumSrc& mom) {
+  return x != nullptr && batch > 0 && n > 0 && n % HA_SPLIT == 0 && batch * (n / HA_SPLIT) <= (int64_t)1 << 30 && ha_aligned16(x) &&
+         ha_aligned16(mom.buf);
+}
+
+int launch_head_front(const float* x, int64_t batch, int64_t n, float eps, MomentumSrc mom, uint16_t* xb, double* partials,
+                      float* gram, float* norm, float* sumsq_out, float* xscale, hipStream_t stream) {
+  if (!head_front_supported(x, batch, n, mom) || !xb || !partials || !gram || !xscale || !ha_aligned16(xb) || !ha_aligned16(gram))
+    return fail(MI_ERR_UNSUPPORTED_SHAPE, "internal: per-head input pass on %lld matrices of 128 x %lld", (long long)batch, (long long)n);
+  HeadFrontArgs a{x, n, (int)(n / HA_SPLIT), eps, mom, xb, partials, gram, norm, sumsq_out, xscale};
+  dim3 grid((unsigned)(batch * a.splits)), block(HA_NT);
+  hipLaunchKernelGGL(head_front_kernel<false>, grid, block, 0, stream, a);
+  hipLaunchKernelGGL(head_front_kernel<true>, grid, block, 0, stream, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));
+  return MI_OK;
+}
+
 }  // namespace mi

@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include "gemm_fast.hpp"
+#include "norm_common.hpp"
 
 namespace mi {
 
@@ -39,6 +40,16 @@ int device_cus();
 // the GEMM mode of the tile engine, one partial sum of squares per workgroup at p.slots_out.
 bool head_apply_supported(const GemmParams& p, int64_t batch, int splits);
 int launch_head_apply(const GemmParams& p, int64_t batch, int splits, float* gram_next, bool out_f32, hipStream_t stream);
+
+// 128-row matrices, first pass over the float32 input x ([batch][128][n], n a multiple of 512; with a momentum
+// source, over the direction it defines, updating the buffer in place): the unnormalised bf16 copy to `xb`, one
+// float64 partial sum of squares per (matrix, slice of 512 columns) to `partials`, and the float32 partial Gram
+// matrices of the copy to `gram` (layout as above).  A second launch resolves the norm: norm[b], sumsq_out[b] (the
+// squared norm of the normalised matrix) and xscale[b] = 1 / norm when the norm is in the range where the divide may
+// be left to the consumers of X; outside it (xscale[b] = 1) that launch rewrites xb and `gram` from x / norm.
+bool head_front_supported(const float* x, int64_t batch, int64_t n, const MomentumSrc& mom);
+int launch_head_front(const float* x, int64_t batch, int64_t n, float eps, MomentumSrc mom, uint16_t* xb, double* partials,
+                      float* gram, float* norm, float* sumsq_out, float* xscale, hipStream_t stream);
 
 // Split-tail (stream-K) launch of the lower-triangle kernel (256 x 256 tiles, K-contiguous operands, bf16 output):
 // with `cus` CUs (a multiple of 8), the whole rounds of `cus` tiles run one tile per workgroup, and the K range of each

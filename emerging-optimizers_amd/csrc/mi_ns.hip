@@ -493,8 +493,6 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
 // ---------------------------------------------------------------------------------------------
 static constexpr int NORM_THREADS = 256;
 static constexpr int NORM_MAX_BLOCKS = 1024;  // partials per matrix
-// Frobenius norms in this range let the divide be deferred to the consumers of X (see scale_cast_kernel).
-static constexpr float NORM_DEFER_MIN = 1e-10f, NORM_DEFER_MAX = 1e10f;
 
 static int norm_blocks(int64_t numel) {
   int64_t vec = numel / 4;  // float4 units
@@ -528,28 +526,8 @@ __device__ __forceinline__ T block_sum(T v, T* scratch) {
   return total;
 }
 
-// Momentum source of the fused optimizer step (orthogonalized_optimizer.py:185-192 of the reference):
-//   buf <- buf + (1 - beta) (g - buf)           [buf.lerp_(grad, 1 - beta)]
-//   d    = nesterov ? buf - (buf - g) (1 - beta) [grad.lerp(buf, beta)] : buf
-// lerp follows torch's two-branch formula (weight < 0.5: start + w (end - start); else end - (end - start)(1 - w)).
-struct MomentumSrc {
-  float* buf;     // momentum buffer, updated in place by the sum-of-squares pass; null: plain input
-  float beta;
-  int nesterov;
-};
-__device__ __forceinline__ float torch_lerp(float start, float end, float w) {
-  const float diff = end - start;
-  return w < 0.5f ? start + w * diff : end - diff * (1.0f - w);
-}
-__device__ __forceinline__ float momentum_direction(float g, float buf_new, float beta, int nesterov) {
-  return nesterov ? torch_lerp(g, buf_new, beta) : buf_new;
-}
-
-// The float32 input is read exactly once on this path: a non-temporal load keeps it from displacing the bf16 copy
-// (which the first Gram product reads next) from the caches.  Measured at 4096 x 14336: 65 -> 60 us for this pass and
-// 200 -> 193 us for the Gram product that follows; a non-temporal store of the bf16 copy costs 7 us instead.
 __device__ __forceinline__ float4 stream_load(const float4* p) {
-  const f32x4_t t = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(p));
+  const f32x4_t t = stream_load4(reinterpret_cast<const float*>(p));
   return make_float4(t[0], t[1], t[2], t[3]);
 }
 
@@ -1467,17 +1445,27 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
   // norm is folded into the first Gram product and the first B X product: one pass over the float32 input, not two.
   float* xscale = reinterpret_cast<float*>(ws + w.xscale);
   int rc;
+  // 128-row matrices whose first group goes through the chain kernel: the input pass also leaves the partial Gram
+  // matrices of its bf16 copy (MI_HEAD_FRONT=0: the general passes and a Gram kernel of its own).
+  const char* front_env = getenv("MI_HEAD_FRONT");
+  const bool head_front = w.gram_splits > 0 && m == CH_M && !tall && !accumulate_fp64 && abc[2] != 0.0f &&
+                          w.gram_splits == n / 512 && w.gram_splits <= NORM_MAX_BLOCKS && !(front_env && front_env[0] == '0') &&
+                          head_front_supported(x, batch, n, mom);
   {
     ProfScope prof(PROF_NORMALIZE, stream);
-    rc = frob_impl(x, batch, numel, eps, accumulate_fp64, xbuf[0], /*out_bf16=*/1, 1.0f, partials, norm, stream, slots,
-                   tall ? rows : 0, tall ? cols : 0, mom, xscale);
+    if (head_front)
+      rc = launch_head_front(x, batch, n, eps, mom, xbuf[0], partials, reinterpret_cast<float*>(ws + w.gpart), norm, slots,
+                             xscale, stream);
+    else
+      rc = frob_impl(x, batch, numel, eps, accumulate_fp64, xbuf[0], /*out_bf16=*/1, 1.0f, partials, norm, stream, slots,
+                     tall ? rows : 0, tall ? cols : 0, mom, xscale);
   }
   if (rc != MI_OK) return rc;
 
   int cur = 0;
   int nslots = 1;  // the normalisation kernel left one value per matrix
   bool want_group = true;
-  bool have_partials = false;  // the partial Gram matrices of xbuf[cur] are in the workspace already
+  bool have_partials = head_front;  // the partial Gram matrices of xbuf[cur] are in the workspace already
   for (int s = 0; s < steps;) {
     const float a = abc[3 * s], b = abc[3 * s + 1], c = abc[3 * s + 2];
     const int taken = ns_group_size(w.pairs, abc, steps, s, want_group);

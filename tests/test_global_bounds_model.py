@@ -671,3 +671,33 @@ def test_head_apply_global_accesses(batch, n):
                     g[r, c:c + 4] += 1
         assert (np.tril(g) == np.tril(np.ones_like(g))).all() and g.max() == 1
         assert b * splits + s < batch * splits  # slot of the partial sum of squares
+
+
+@pytest.mark.parametrize("batch,n", [(32, 4096), (3, 1024), (1, 2048), (5, 512)])
+def test_head_front_global_accesses(batch, n):
+    """The input pass of 128-row matrices (head_front_kernel), one workgroup of 512 threads per (matrix, 512-column
+    slice): a thread reads two 16-byte groups of float32 (eight columns) per 32 rows and slab and writes the 16 bytes
+    of bf16 they become; every element of x is read once and every element of the copy written once, inside their
+    arrays; the partial sums ([batch][slices] float64) and the partial Gram matrices are indexed as the consumers
+    index them."""
+    m, split, w = 128, 512, 128
+    splits = n // split
+    tid = np.arange(512)
+    ck, cc = tid >> 4, tid & 15
+    for wg in sample(range(batch * splits), 6):
+        b, s = divmod(wg, splits)
+        seen = np.zeros((m, split), dtype=np.int32)
+        base = b * m * n + s * split + 8 * cc
+        for t in range(split // w):
+            for u in range(4):
+                at = base + (ck + 32 * u) * n + t * w
+                for h in range(2):
+                    lo = at + 4 * h
+                    assert (lo >= b * m * n).all() and (lo + 4 <= (b + 1) * m * n).all() and (lo % 4 == 0).all()
+                assert (at % 8 == 0).all()  # 16-byte alignment of the bf16 store
+                rows, cols = (at - b * m * n) // n, (at - b * m * n) % n - s * split
+                assert (cols >= 0).all() and (cols + 8 <= split).all()
+                for r, c in zip(rows, cols):
+                    seen[r, c:c + 8] += 1
+        assert (seen == 1).all()
+        assert 0 <= b * splits + s < batch * splits

@@ -490,6 +490,57 @@ def test_per_head_slab_kernel_against_the_general_kernels(gpu, monkeypatch, shap
     assert torch.equal(new[-1], alone)
 
 
+@pytest.mark.parametrize("shape", [(32, 128, 4096), (3, 128, 1024), (1, 128, 2048)])
+@pytest.mark.parametrize("magnitude", [3e-3, 1e-17, 1e15])
+def test_per_head_input_pass_against_the_general_passes(gpu, monkeypatch, shape, magnitude):
+    """128-row matrices: the pass over the float32 input also leaves the partial Gram matrices of its bf16 copy
+    (head_front_kernel in inst_head_apply.hip).  MI_HEAD_FRONT=0 sends the same call through the general sum-of-squares
+    pass and a Gram kernel of its own.  The two add the squares in a different order, so the norm may differ in its last
+    bit, which moves a few bf16 roundings: the results agree to 2e-4 and either is as far from float32 as the other.
+    The magnitudes 1e-17 and 1e15 put the norm outside the range where the divide by it may be left to the consumers:
+    the second launch of the input pass then rewrites the copy and its Gram matrices from x / norm.  A batch entry
+    equals the matrix computed alone, bit for bit."""
+    x = torch.randn(*shape, device=gpu, generator=torch.Generator(device=gpu).manual_seed(33)) * magnitude
+    with utils.fp32_matmul_precision("medium"):
+        monkeypatch.delenv("MI_HEAD_FRONT", raising=False)
+        new = muon_utils.newton_schulz(x, steps=5, coefficient_type="simple", use_syrk=True)
+        alone = muon_utils.newton_schulz(x[-1], steps=5, coefficient_type="simple", use_syrk=True)
+        monkeypatch.setenv("MI_HEAD_FRONT", "0")
+        old = muon_utils.newton_schulz(x, steps=5, coefficient_type="simple", use_syrk=True)
+    assert torch.isfinite(new).all()
+    diff = rel_fro(new, old)
+    ref = ns_fp32_torch((x.double() / magnitude).float(), SIMPLE5)  # (the iteration does not depend on the scale of x)
+    print(f"\n  {shape} x {magnitude:g}: input pass with Gram partials vs general passes rel_fro = {diff:.2e}; "
+          f"vs float32 {rel_fro(_np(new), _np(ref)):.2e} / {rel_fro(_np(old), _np(ref)):.2e}")
+    assert diff <= 2e-4
+    assert rel_fro(_np(new), _np(ref)) <= TOL_FP32
+    assert torch.equal(new[-1], alone)
+
+
+@pytest.mark.parametrize("nesterov", [True, False])
+def test_per_head_input_pass_with_a_momentum_source(gpu, monkeypatch, nesterov):
+    """The fused optimizer update on 128-row matrices: the input pass that leaves the Gram partials also updates the
+    momentum buffer and orthogonalises the direction it defines.  Against the same call through the general passes
+    (MI_HEAD_FRONT=0): the buffer bit for bit (the same elementwise formula), the parameter to rounding noise."""
+    shape, lr, beta, wd = (8, 128, 2048), 0.02, 0.95, 0.1
+    gen = torch.Generator().manual_seed(11)
+    p0 = (torch.randn(shape, generator=gen) * 0.02).to(gpu)
+    buf0 = (torch.randn(shape, generator=gen) * 1e-3).to(gpu)
+    g = (torch.randn(shape, generator=gen) * 1e-2).to(gpu)
+    res = {}
+    for front in ("1", "0"):
+        monkeypatch.setenv("MI_HEAD_FRONT", front)
+        p, buf = p0.clone(), buf0.clone()
+        hip_kernels.fused_muon_update(p, g, buf, SIMPLE5, beta=beta, nesterov=nesterov, param_decay=1 - wd * lr, update_scale=-lr)
+        res[front] = (p, buf)
+    buf_ref = buf0.clone().lerp_(g, 1 - beta)
+    torch.testing.assert_close(res["1"][1], buf_ref, rtol=2e-6, atol=5e-9)
+    assert torch.equal(res["1"][1], res["0"][1])
+    assert float((res["1"][0] - res["0"][0]).norm() / (res["0"][0] - p0).norm()) <= 2e-4
+    direction = g.lerp(buf_ref, beta) if nesterov else buf_ref
+    assert float(rel_fro(_np((res["1"][0] - (1 - wd * lr) * p0) / (-lr)), _np(ns_fp32_torch(direction, SIMPLE5)))) <= TOL_FP32
+
+
 @pytest.mark.parametrize("shape", [(32, 128, 4096), (1024, 4096)])
 def test_fused_call_replays_from_a_hip_graph(gpu, shape):
     """The single-call driver allocates nothing and records no memset: captured into a HIP graph (its workspace
