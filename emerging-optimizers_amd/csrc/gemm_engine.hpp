@@ -43,6 +43,9 @@ struct GemmParams {
   float alpha, beta, out_scale;
   float beta2;                   // coefficient of Cin2
   float out_accum;               // float32 output only: Out = out_accum * Out + out_scale * value (0: plain store)
+  // float32 output of a GEMM-mode product through the fast kernel's staged epilogue only: Out holds the transposed
+  // result, element (m, n) at Out[n * ldo + m] (ldo >= M).  Every other kernel is refused by its launcher.
+  int out_transposed;
   int tiles_m, tiles_n;
   int skip_upper;
   // Diagonal-shift bookkeeping of the fused Newton-Schulz driver (all null / 0 for plain calls).

@@ -253,6 +253,10 @@ __device__ __forceinline__ void gemm_tile_of(int pid, int tiles_m, int tiles_n, 
 // Cin loads and the stores become 16-byte-per-lane, 128-byte-per-row accesses.  (MI = rows of one MFMA tile.)
 // No workgroup barrier is needed between the passes: a wavefront only touches its own region and LDS operations of one wavefront
 // complete in order.
+// Transposed float32 output (p.out_transposed): the finished values go back to the staging rows and are read a
+// second time down the columns, a lane taking four consecutive rows of one column (16 bytes of the transposed
+// matrix, the sixteen rows of the block 64 bytes); row pitch mod 64 words is 4, so the 64 lanes of such a read fall
+// on 64 different banks.
 template <class C, bool OUT_F32, bool GUARD>
 __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x4_t (&acc)[C::FM][C::FN], char* lds, int wave,
                                                   int lane, int m_base, int n_base, int64_t batch, float alpha,
@@ -323,6 +327,13 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x4_t (
         float* o = reinterpret_cast<float*>(p.Out) + batch * p.o_bs + (int64_t)m * p.ldo + n;
         lo *= p.out_scale;
         hi *= p.out_scale;
+        if constexpr (!GUARD) {
+          if (p.out_transposed) {
+            *reinterpret_cast<f32x4_t*>(reg + row * ROWB + cc * 4) = lo;
+            *reinterpret_cast<f32x4_t*>(reg + row * ROWB + cc * 4 + 16) = hi;
+            continue;
+          }
+        }
         if (p.out_accum != 0.0f) {  // in-place update of a float32 matrix (optimizer step folded into the epilogue)
           const f32x4_t olo = *reinterpret_cast<const f32x4_t*>(o), ohi = *reinterpret_cast<const f32x4_t*>(o + 4);
 #pragma unroll
@@ -338,6 +349,24 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x4_t (
         const uint2 a = __builtin_bit_cast(uint2, __builtin_convertvector(lo, bf16x4_t));
         const uint2 b = __builtin_bit_cast(uint2, __builtin_convertvector(hi, bf16x4_t));
         *reinterpret_cast<uint4*>(o) = make_uint4(a.x, a.y, b.x, b.y);
+      }
+    }
+    if constexpr (OUT_F32 && !GUARD && MI == 16) {
+      if (p.out_transposed) {
+        const int col = lane & 15, g4 = 4 * (lane >> 4);
+#pragma unroll
+        for (int t = 0; t < TN / 16; ++t) {
+          f32x4_t w;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w[e] = *reinterpret_cast<const float*>(reg + (g4 + e) * ROWB + (16 * t + col) * 4);
+          float* o = reinterpret_cast<float*>(p.Out) + batch * p.o_bs + (int64_t)(n_base + 16 * t + col) * p.ldo + m_base + i * MI + g4;
+          if (p.out_accum != 0.0f) {
+            const f32x4_t old = *reinterpret_cast<const f32x4_t*>(o);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = __builtin_fmaf(p.out_accum, old[e], w[e]);
+          }
+          *reinterpret_cast<f32x4_t*>(o) = w;
+        }
       }
     }
   }

@@ -177,6 +177,7 @@ int launch_head_apply(const GemmParams& p, int64_t batch, int splits, float* gra
   if (!head_apply_supported(p, batch, splits))
     return fail(MI_ERR_UNSUPPORTED_SHAPE, "internal: per-head product on %d x %d (K = %d), %d slices", p.M, p.N, p.K, splits);
   if (out_f32 && gram_next != nullptr) return fail(MI_ERR_BAD_ARG, "internal: the Gram partials need the bf16 result");
+  if (p.out_transposed) return fail(MI_ERR_UNSUPPORTED_SHAPE, "internal: the slab kernel has no transposed output");
   GemmParams q = p;
   if (q.slot_stride == 0) q.slot_stride = splits;
   if (int rc = check_slots(q, splits)) return rc;

@@ -24,6 +24,7 @@ int launch_one(const GemmParams& p, int64_t batch, hipStream_t stream) {
     if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "hipFuncSetAttribute(%d B LDS): %s", LDS_BYTES, hipGetErrorString(e));
     attr_set = true;
   }
+  if (p.out_transposed) return fail(MI_ERR_UNSUPPORTED_SHAPE, "internal: the general kernel has no transposed output");
   GemmParams q = p;
   q.tiles_m = (p.M + BM - 1) / BM;
   q.tiles_n = (p.N + BN - 1) / BN;
@@ -55,6 +56,10 @@ int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream, int64_t 
   if (p.K < C::BK || p.K % C::BK != 0)
     return fail(MI_ERR_UNSUPPORTED_SHAPE, "internal: K = %d is not a multiple of %d", p.K, C::BK);
   if (p.M <= 0 || p.N <= 0 || batch <= 0) return MI_OK;
+  // transposed output: only the staged epilogue of the GEMM mode writes it, and only for whole tiles
+  constexpr bool STAGED_GEMM = MODE == MODE_GEMM && OUT_F32 && C::MI == 16 && (C::TN == 32 || C::TN == 64 || C::TN == 128);
+  if (p.out_transposed && !(STAGED_GEMM && p.M % C::TILE_M == 0 && p.N % C::TILE_N == 0 && p.ldo >= p.M && p.ldo % 4 == 0))
+    return fail(MI_ERR_UNSUPPORTED_SHAPE, "internal: no transposed output for this product (%d x %d)", p.M, p.N);
   GemmParams q = p;
   q.tiles_m = (p.M + C::TILE_M - 1) / C::TILE_M;
   q.tiles_n = (p.N + C::TILE_N - 1) / C::TILE_N;

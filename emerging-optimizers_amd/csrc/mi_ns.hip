@@ -190,6 +190,14 @@ static bool gemm_prefers_half_tiles(int64_t m, int64_t n, int64_t batch) {
   return (double)ceil_div(2 * tiles, cus) * 0.5 * 1.27 < (double)ceil_div(tiles, cus);
 }
 
+// Whether the float32 GEMM+AXPY of an (m x m) by (m x n) product runs on kernels that can write their result
+// transposed (the staged epilogue of the fast kernel; mirrors the choices of launch_class below).
+static bool gemm_transposed_out_ok(int64_t m, int64_t n) {
+  if (m % 64 != 0 || m < 64) return false;
+  if (m >= 1024 && n >= 1024 && m % 256 == 0 && n % 256 == 0) return true;
+  return m % 128 == 0 && m < 1024 && n % 256 == 0 && n >= 256;
+}
+
 template <bool P_KS, bool Q_KS, int MODE, bool OUT_F32>
 static int launch_class(TileClass tc, const GemmParams& p, int64_t batch, hipStream_t stream) {
   const bool k_ok = p.K % 64 == 0 && p.K >= 64;
@@ -380,7 +388,7 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
                           int64_t x_ld, int x_trans, void* Xout, int64_t o_bs, int64_t o_ld, int64_t batch,
                           int64_t m, int64_t n, float alpha, float beta, int out_fp32, float out_scale,
                           hipStream_t stream, const ShiftArgs* sh = nullptr, float out_accum = 0.0f, int head_splits = 0,
-                          float* head_gram_next = nullptr, bool* head_used = nullptr) {
+                          float* head_gram_next = nullptr, bool* head_used = nullptr, int out_transposed = 0) {
   if (!Bm || !X || !Xout) return fail(MI_ERR_BAD_ARG, "mi_gemm_axpy_bf16: null pointer");
   if (batch < 0 || m < 0 || n < 0) return fail(MI_ERR_BAD_ARG, "mi_gemm_axpy_bf16: negative extent");
   if (m % 8 || n % 8) return fail(MI_ERR_UNSUPPORTED_SHAPE, "M and N must be multiples of 8, got M=%lld, N=%lld", (long long)m, (long long)n);
@@ -389,7 +397,9 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
   if (!aligned16(Bm) || !aligned16(X) || !aligned16(Xout))
     return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_gemm_axpy_bf16: pointers must be 16-byte aligned");
   const int64_t x_inner = x_trans ? m : n;
-  if (b_ld < m || x_ld < x_inner || o_ld < x_inner) return fail(MI_ERR_BAD_ARG, "mi_gemm_axpy_bf16: leading dimension too small");
+  if (out_transposed && (x_trans || !out_fp32)) return fail(MI_ERR_BAD_ARG, "internal: transposed output of this product");
+  if (b_ld < m || x_ld < x_inner || o_ld < (out_transposed ? m : x_inner))
+    return fail(MI_ERR_BAD_ARG, "mi_gemm_axpy_bf16: leading dimension too small");
   if (m > (1 << 30) || n > (1 << 30)) return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_gemm_axpy_bf16: extent too large");
   if (batch == 0 || m == 0 || n == 0) return MI_OK;
 
@@ -405,6 +415,7 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
   p.beta = beta;
   p.out_scale = out_scale;
   p.out_accum = out_fp32 ? out_accum : 0.0f;
+  p.out_transposed = out_transposed;
   if (sh) sh->apply(p);
   TileClass tc = pick_class(m);
   if (!x_trans) {
@@ -451,13 +462,13 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
           pt.N = (int)tail_cols;
           pt.Q = p.Q + main_cols;  // K-strided operand: column offset
           if (pt.Cin) pt.Cin = p.Cin + main_cols;
-          out_off = main_cols;
+          out_off = out_transposed ? main_cols * p.ldo : main_cols;
         } else {
           pm.M = (int)main_rows;
           pt.M = (int)tail_rows;
           pt.P = p.P + main_rows * p.ldp;
           if (pt.Cin) pt.Cin = p.Cin + main_rows * p.ldc;
-          out_off = main_rows * p.ldo;
+          out_off = out_transposed ? main_rows : main_rows * p.ldo;
         }
         pt.Out = out_fp32 ? static_cast<void*>(static_cast<float*>(p.Out) + out_off)
                           : static_cast<void*>(static_cast<uint16_t*>(p.Out) + out_off);
@@ -1440,7 +1451,11 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
   const int64_t m = tall ? cols : rows, n = tall ? rows : cols;
   const int64_t ld = n;
   const int64_t x_bs = numel, g_bs = m * m;
-  float* result = tall ? reinterpret_cast<float*>(ws + w.result) : out;
+  // (where the last product can write its float32 result transposed, a tall input needs neither the staging copy
+  // nor the transposing pass at the end)
+  const char* tall_env = getenv("MI_TALL_DIRECT");  // "0": staging copy and transposing pass for every tall input (A/B runs, tests)
+  const bool direct_t = tall && gemm_transposed_out_ok(m, n) && !(w.gram_splits > 0 && m == CH_M) && !(tall_env && tall_env[0] == '0');
+  float* result = (tall && !direct_t) ? reinterpret_cast<float*>(ws + w.result) : out;
   // The input is cast to bf16 by the pass that sums its squares (transposing, if it is tall), and the divide by the
   // norm is folded into the first Gram product and the first B X product: one pass over the float32 input, not two.
   float* xscale = reinterpret_cast<float*>(ws + w.xscale);
@@ -1571,9 +1586,11 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
     {
       ProfScope prof(PROF_APPLY, stream);
       bool head_used = false;
-      rc = gemm_axpy_impl(mult, g_bs, m, xbuf[cur], x_bs, ld, trans, dst, x_bs, ld, batch, m, n, alpha, taken > 1 ? 1.0f : a,
-                          last ? 1 : 0, last ? out_scale : 1.0f, stream, &sh_apply, (last && !tall) ? out_accum : 0.0f,
-                          chain ? w.gram_splits : 0, reinterpret_cast<float*>(ws + w.gpart), &head_used);
+      const bool write_t = last && direct_t;
+      rc = gemm_axpy_impl(mult, g_bs, m, xbuf[cur], x_bs, ld, trans, dst, x_bs, write_t ? m : ld, batch, m, n, alpha,
+                          taken > 1 ? 1.0f : a, last ? 1 : 0, last ? out_scale : 1.0f, stream, &sh_apply,
+                          (last && (!tall || direct_t)) ? out_accum : 0.0f, chain ? w.gram_splits : 0,
+                          reinterpret_cast<float*>(ws + w.gpart), &head_used, write_t ? 1 : 0);
       have_partials = head_used && !last;
     }
     if (rc != MI_OK) return rc;
@@ -1581,7 +1598,7 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
     cur ^= 1;
     s += taken;
   }
-  if (tall) {
+  if (tall && !direct_t) {
     ProfScope prof(PROF_NORMALIZE, stream);
     dim3 gridt((unsigned)((n + 63) / 64), (unsigned)((m + 63) / 64), (unsigned)batch), blockt(256);
     hipLaunchKernelGGL(transpose_f32_kernel, gridt, blockt, 0, stream, result, m, n, out, out_accum);

@@ -144,8 +144,9 @@ size_t mi_frob_partials_len(int64_t batch, int64_t numel);
  *
  * x, out: float32, batch matrices of (rows, cols) row-major contiguous.  The iteration always runs on
  * the orientation with the smaller leading dimension (muon_utils.py:205-208): a tall input is transposed
- * while it is cast to bf16 (into the workspace) and the float32 result is transposed back into `out`, so
- * the MFMA kernels always see the wide layout.  out must not alias x.
+ * while it is cast to bf16 (into the workspace) and the float32 result is written transposed into `out` (by the
+ * last product itself, or by a transposing pass over a staging copy in the workspace), so the MFMA kernels
+ * always see the wide layout.  out must not alias x.
  * abc: HOST array of 3*steps floats (a, b, c per step, already expanded by the coefficient iterator).
  * steps == 0 returns the normalised input.  rows and cols must be multiples of 8.
  * workspace: device scratch of at least mi_newton_schulz_workspace_bytes(batch, rows, cols) bytes,
@@ -205,7 +206,7 @@ int mi_newton_schulz_schedule(int64_t batch, int64_t rows, int64_t cols, const f
  * together with Muon's closure (muon.py:117-132): param_decay = 1 - wd*lr (decoupled), 1 - wd (independent),
  * 1 - wd*lr^2 (palm), 1 (no decay); update_scale = -lr * get_muon_scale_factor(...) * extra_scale_factor.
  * The momentum update, the sum of squares and the bf16 cast of d share one pass over grad and momentum, and the
- * last GEMM epilogue (or the final transpose of a tall parameter) updates param in place.  param, grad, momentum: float32 (batch, rows, cols) row-major contiguous, distinct
+ * last GEMM epilogue (transposed for a tall parameter) updates param in place.  param, grad, momentum: float32 (batch, rows, cols) row-major contiguous, distinct
  * buffers.  Other arguments and the workspace as for mi_newton_schulz_bf16; steps >= 1; param_decay != 0.
  */
 int mi_muon_update_bf16(float* param, const float* grad, float* momentum, int64_t batch, int64_t rows, int64_t cols,

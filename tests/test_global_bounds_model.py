@@ -701,3 +701,60 @@ def test_head_front_global_accesses(batch, n):
                     seen[r, c:c + 8] += 1
         assert (seen == 1).all()
         assert 0 <= b * splits + s < batch * splits
+
+
+def transposed_store_elements(cfg, m0, n0, ldo, base):
+    """Element offsets (into the transposed float32 result, element (m, n) at n * ldo + m) of the 16-byte stores that
+    the staged GEMM epilogue issues for the tile at (m0, n0) when p.out_transposed is set: per wavefront and 16-row
+    block, lane l takes rows 4 (l / 16) .. + 3 of column 16 t + l % 16."""
+    tile_m, tile_n, wgm, wgn, _ = CFGS[cfg]
+    tm, tn = tile_m // wgm, tile_n // wgn
+    col, g4 = LANES & 15, 4 * (LANES >> 4)
+    out = []
+    for wave in range(NW):
+        wm, wn = wave % wgm, wave // wgm
+        for i in range(tm // MI):
+            for t in range(tn // 16):
+                out.append(base + (n0 + wn * tn + 16 * t + col) * ldo + m0 + wm * tm + i * MI + g4)
+    return np.concatenate(out)
+
+
+@pytest.mark.parametrize("m,n,batch", [(4096, 14336, 1), (1792, 4096, 8), (1024, 1024, 1), (1024, 2304, 2), (256, 512, 3)])
+def test_transposed_output_of_the_staged_gemm_epilogue(m, n, batch):
+    """Tall inputs: the last product writes its float32 result transposed, (n x m) row-major.  Over the launches of
+    one product (one, or a main and a tail launch whose output pointer is advanced by main_cols * ldo or by main_rows
+    elements) every element of every transposed matrix is written exactly once, by a 16-byte aligned store."""
+    cus, ldo = 256, m
+    tm, tn = m // 256, n // 256
+    launches = []  # (cfg, rows, cols, element offset of the launch's output inside a batch entry)
+    if m >= 1024:
+        rem = (tm * tn * batch) % cus
+        tail_cols = tail_rows = 0
+        if rem > 0 and rem * 2 <= cus:
+            if rem % (tm * batch) == 0 and rem // (tm * batch) < tn:
+                tail_cols = rem // (tm * batch) * 256
+            elif rem % (tn * batch) == 0 and rem // (tn * batch) < tm:
+                tail_rows = rem // (tn * batch) * 256
+        if tail_cols:
+            launches = [("CfgBig", m, n - tail_cols, 0), ("CfgHalfN", m, tail_cols, (n - tail_cols) * ldo)]
+        elif tail_rows:
+            launches = [("CfgBig", m - tail_rows, n, 0), ("CfgHalfN", tail_rows, n, m - tail_rows)]
+        else:
+            launches = [("CfgBig", m, n, 0)]
+        assert (m, n, batch) != (4096, 14336, 1) or tail_cols == 2048
+        assert (m, n, batch) != (1792, 4096, 8) or tail_rows == 256
+    else:
+        launches = [("CfgM128", m, n, 0)]
+    b = batch - 1
+    written = np.zeros(n * m, dtype=np.int32)
+    for cfg, rows, cols, off in launches:
+        tile_m, tile_n = CFGS[cfg][:2]
+        assert rows % tile_m == 0 and cols % tile_n == 0 and ldo >= m and ldo % 4 == 0
+        for m0 in range(0, rows, tile_m):
+            for n0 in range(0, cols, tile_n):
+                at = transposed_store_elements(cfg, m0, n0, ldo, off)
+                assert (at % 4 == 0).all() and (at >= 0).all() and (at + 4 <= n * m).all()
+                for e in range(4):
+                    np.add.at(written, at + e, 1)
+    assert (written == 1).all()
+    assert (b * n * m + n * m) <= batch * n * m

@@ -541,6 +541,31 @@ def test_per_head_input_pass_with_a_momentum_source(gpu, monkeypatch, nesterov):
     assert float(rel_fro(_np((res["1"][0] - (1 - wd * lr) * p0) / (-lr)), _np(ns_fp32_torch(direction, SIMPLE5)))) <= TOL_FP32
 
 
+@pytest.mark.parametrize("shape", [(3584, 1024), (2048, 1024), (512, 256), (2, 2304, 1024), (8, 4096, 1792), (14336, 4096)])
+def test_tall_input_result_written_transposed_by_the_last_product(gpu, monkeypatch, shape):
+    """Tall inputs are iterated in the transposed orientation.  Where the last product runs on kernels with the staged
+    epilogue, it writes its float32 result transposed, straight into the output; MI_TALL_DIRECT=0 restores the
+    float32 staging copy and the transposing pass.  Same arithmetic, so the two agree bit for bit -- also for the
+    fused optimizer update, where the epilogue reads the parameter it updates in the transposed pattern."""
+    gen = torch.Generator(device=gpu).manual_seed(9)
+    x = torch.randn(*shape, device=gpu, generator=gen) * 1e-3
+    p0 = torch.randn(*shape, device=gpu, generator=gen) * 0.02
+    buf0 = torch.randn(*shape, device=gpu, generator=gen) * 1e-3
+    res = {}
+    for direct in ("1", "0"):
+        monkeypatch.setenv("MI_TALL_DIRECT", direct)
+        with utils.fp32_matmul_precision("medium"):
+            out = muon_utils.newton_schulz(x, steps=5, coefficient_type="simple", use_syrk=True)
+        p, buf = p0.clone(), buf0.clone()
+        hip_kernels.fused_muon_update(p, x, buf, SIMPLE5, beta=0.95, nesterov=True, param_decay=0.999, update_scale=-0.02)
+        res[direct] = (out, p, buf)
+    assert torch.isfinite(res["1"][0]).all()
+    for a, b in zip(res["1"], res["0"]):
+        assert torch.equal(a, b)
+    if shape != (14336, 4096):
+        assert rel_fro(_np(res["1"][0]), _np(ns_fp32_torch(x, SIMPLE5))) <= TOL_FP32
+
+
 @pytest.mark.parametrize("shape", [(32, 128, 4096), (1024, 4096)])
 def test_fused_call_replays_from_a_hip_graph(gpu, shape):
     """The single-call driver allocates nothing and records no memset: captured into a HIP graph (its workspace

@@ -469,3 +469,22 @@ def test_chain_kernel_lower_triangle_then_mirror():
                     a = ch_elem(16 * bi + 4 * patch + (i16 >> 2), 16 * bj + 4 * (i16 & 3))
                     banks += [(a // 4) % 64, (a // 4 + 1) % 64]
                 assert max(banks.count(x) for x in set(banks)) <= 2
+
+
+@pytest.mark.parametrize("tn", [64, 128])
+def test_transposed_reads_of_the_gemm_staging_rows_are_conflict_free(tn):
+    """Transposed float32 output of the staged GEMM epilogue: a 16-row block of a wavefront sits in LDS as float32 rows
+    of tn values padded by 16 bytes; lane l reads rows 4 (l / 16) + e, e = 0 .. 3, of column 16 t + l % 16, four bytes
+    at a time.  For every (t, e) the 64 lanes hit 64 different banks (4-byte banks, 64 of them), and together the reads
+    cover every element of the block once."""
+    rowb = tn * 4 + 16
+    seen = [[0] * tn for _ in range(16)]
+    for t in range(tn // 16):
+        for e in range(4):
+            banks = set()
+            for lane in range(64):
+                row, col = 4 * (lane >> 4) + e, 16 * t + (lane & 15)
+                banks.add(((row * rowb + col * 4) // 4) % 64)
+                seen[row][col] += 1
+            assert len(banks) == 64
+    assert all(v == 1 for r in seen for v in r)
