@@ -1299,6 +1299,14 @@ static int small_chain(const uint16_t* X, int64_t batch, int64_t n, int splits, 
 
 static size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
+// Tall input iterated as (m x n), m < n: does the last product write the float32 result transposed, straight into the
+// output?  (Not on the slab kernel of 128-row matrices.  MI_TALL_DIRECT=0, read by the workspace query and by the
+// call alike: staging copy and transposing pass for every tall input -- A/B runs, tests.)
+static bool tall_writes_direct(int64_t m, int64_t n, int gram_splits) {
+  const char* env = getenv("MI_TALL_DIRECT");
+  return gemm_transposed_out_ok(m, n) && !(gram_splits > 0 && m == CH_M) && !(env && env[0] == '0');
+}
+
 struct NsWorkspace {
   size_t x0, x1, a, b, t, d2, partials, norm, slots, shift, xscale, result, gpart, total;
   int gram_splits;  // > 0: split-K Gram path of short, wide batches
@@ -1360,10 +1368,10 @@ static NsWorkspace ns_layout(int64_t batch, int64_t rows, int64_t cols) {
   w.slots = off; off += align_up((size_t)batch * w.max_slots * sizeof(float), 256);
   w.shift = off; off += align_up((size_t)batch * sizeof(float), 256);
   w.xscale = off; off += align_up((size_t)batch * sizeof(float), 256);
-  // tall inputs iterate on the transposed orientation; their float32 result is staged here before the
-  // final transpose into `out`
+  // tall inputs iterate on the transposed orientation; where the last product cannot write its float32 result
+  // transposed, it is staged here before the final transpose into `out`
   w.result = off;
-  if (rows > cols) off += align_up((size_t)batch * rows * cols * sizeof(float), 256);
+  if (rows > cols && !tall_writes_direct(cols, rows, w.gram_splits)) off += align_up((size_t)batch * rows * cols * sizeof(float), 256);
   // float32 partial Gram matrices of the split-K path
   w.gpart = off;
   off += align_up((size_t)batch * w.gram_splits * m * m * sizeof(float), 256);
@@ -1453,8 +1461,7 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
   const int64_t x_bs = numel, g_bs = m * m;
   // (where the last product can write its float32 result transposed, a tall input needs neither the staging copy
   // nor the transposing pass at the end)
-  const char* tall_env = getenv("MI_TALL_DIRECT");  // "0": staging copy and transposing pass for every tall input (A/B runs, tests)
-  const bool direct_t = tall && gemm_transposed_out_ok(m, n) && !(w.gram_splits > 0 && m == CH_M) && !(tall_env && tall_env[0] == '0');
+  const bool direct_t = tall && tall_writes_direct(m, n, w.gram_splits);
   float* result = (tall && !direct_t) ? reinterpret_cast<float*>(ws + w.result) : out;
   // The input is cast to bf16 by the pass that sums its squares (transposing, if it is tall), and the divide by the
   // norm is folded into the first Gram product and the first B X product: one pass over the float32 input, not two.
