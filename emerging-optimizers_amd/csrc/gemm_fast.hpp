@@ -257,7 +257,9 @@ __device__ __forceinline__ void gemm_tile_of(int pid, int tiles_m, int tiles_n, 
 // second time down the columns, a lane taking four consecutive rows of one column (16 bytes of the transposed
 // matrix, the sixteen rows of the block 64 bytes); row pitch mod 64 words is 4, so the 64 lanes of such a read fall
 // on 64 different banks.
-template <class C, bool OUT_F32, bool GUARD>
+// RMW: the kernel variant for p.out_accum != 0, a compile-time flag so that the plain write-out carries none of its
+// registers and branches (with a run-time flag the plain float32 product of 4096 x 14336 took 7 us longer).
+template <class C, bool OUT_F32, bool GUARD, bool RMW>
 __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x4_t (&acc)[C::FM][C::FN], char* lds, int wave,
                                                   int lane, int m_base, int n_base, int64_t batch, float alpha,
                                                   float beta, float* red) {
@@ -278,23 +280,53 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x4_t (
   // now), so the global-load latency is paid once instead of once per piece.
   // (register budget: a workgroup of four wavefronts leaves each lane 512 registers, 256 of them free here)
   constexpr bool PREFETCH_ALL = C::FM * NIT * 4 <= (C::NW <= 4 ? 160 : 64);  // else one MI-row block at a time
-  uint4 cin[C::FM][NIT];
+  // blocks in flight (a block's registers are refilled when it has been consumed); the in-place variant of a large tile
+  // shares the registers with the old values
+  constexpr int CW = !PREFETCH_ALL ? 1 : ((RMW && C::FM * NIT * 4 > 64 && C::FM > 4) ? 4 : C::FM);
+  uint4 cin[CW][NIT];
   auto load_cin = [&](int i) {
 #pragma unroll
     for (int t = 0; t < NIT; ++t) {
       const int m = m_base + i * MI + t * RPI + rr, n = n_base + cc;
-      cin[i][t] = make_uint4(0u, 0u, 0u, 0u);
-      if (use_c && (!GUARD || (m < p.M && n < p.N))) cin[i][t] = *reinterpret_cast<const uint4*>(Cb + (int64_t)m * p.ldc + n);
+      cin[i % CW][t] = make_uint4(0u, 0u, 0u, 0u);
+      if (use_c && (!GUARD || (m < p.M && n < p.N))) cin[i % CW][t] = *reinterpret_cast<const uint4*>(Cb + (int64_t)m * p.ldc + n);
     }
   };
-  if (PREFETCH_ALL) {
 #pragma unroll
-    for (int i = 0; i < C::FM; ++i) load_cin(i);
-  }
+  for (int i = 0; i < CW && i < C::FM; ++i) load_cin(i);
+  // In-place update of a float32 matrix (out_accum != 0): the old values of a 16-row block are requested one block
+  // ahead (loaded where they are used, every one of the FM * NIT pieces waits out a memory latency of its own:
+  // measured 22 us per 256 x 256 tile against 12 this way).
+  constexpr int OW = 2;  // blocks in flight (three and four: no faster, and the 256 x 256 tile starts to spill)
+  // (A kernel of its own, not two copies of the epilogue behind a branch in one kernel: that made the 256 x 256 tile
+  // spill 548 bytes per lane.)
+  static_assert(!RMW || OUT_F32, "in-place update of a float32 matrix");
+  const bool rmw_t = RMW && !GUARD && p.out_transposed;
+  f32x4_t oldv[RMW ? OW : 1][RMW ? (NIT * 2 > TN / 16 ? NIT * 2 : TN / 16) : 1];
+  auto load_old = [&](int i) {
+    if constexpr (RMW) {
+      if (rmw_t) {
+#pragma unroll
+        for (int t = 0; t < TN / 16; ++t)
+          oldv[i % OW][t] = *reinterpret_cast<const f32x4_t*>(
+              reinterpret_cast<const float*>(p.Out) + batch * p.o_bs + (int64_t)(n_base + 16 * t + (lane & 15)) * p.ldo + m_base + i * MI + 4 * (lane >> 4));
+      } else {
+#pragma unroll
+        for (int t = 0; t < NIT; ++t) {
+          const int m = m_base + i * MI + t * RPI + rr, n = n_base + cc;
+          if (GUARD && (m >= p.M || n >= p.N)) continue;
+          const float* o = reinterpret_cast<const float*>(p.Out) + batch * p.o_bs + (int64_t)m * p.ldo + n;
+          oldv[i % OW][2 * t] = *reinterpret_cast<const f32x4_t*>(o);
+          oldv[i % OW][2 * t + 1] = *reinterpret_cast<const f32x4_t*>(o + 4);
+        }
+      }
+    }
+  };
+#pragma unroll
+  for (int i = 0; RMW && i < OW && i < C::FM; ++i) load_old(i);
   float ssq = 0.0f;
 #pragma unroll
   for (int i = 0; i < C::FM; ++i) {
-    if (!PREFETCH_ALL) load_cin(i);
     char* reg = lds + (wave * NREG + i % NREG) * (MI * ROWB);
 #pragma unroll
     for (int j = 0; j < C::FN; ++j)
@@ -312,7 +344,7 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x4_t (
       lo *= alpha;
       hi *= alpha;
       if (use_c) {
-        const uint32_t w[4] = {cin[i][t].x, cin[i][t].y, cin[i][t].z, cin[i][t].w};
+        const uint32_t w[4] = {cin[i % CW][t].x, cin[i % CW][t].y, cin[i % CW][t].z, cin[i % CW][t].w};
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
           lo[2 * e] = __builtin_fmaf(beta, __uint_as_float(w[e] << 16), lo[2 * e]);
@@ -334,8 +366,8 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x4_t (
             continue;
           }
         }
-        if (p.out_accum != 0.0f) {  // in-place update of a float32 matrix (optimizer step folded into the epilogue)
-          const f32x4_t olo = *reinterpret_cast<const f32x4_t*>(o), ohi = *reinterpret_cast<const f32x4_t*>(o + 4);
+        if constexpr (RMW) {  // in-place update of a float32 matrix (optimizer step folded into the epilogue)
+          const f32x4_t olo = oldv[i % OW][2 * t], ohi = oldv[i % OW][2 * t + 1];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             lo[e] = __builtin_fmaf(p.out_accum, olo[e], lo[e]);
@@ -360,8 +392,8 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x4_t (
 #pragma unroll
           for (int e = 0; e < 4; ++e) w[e] = *reinterpret_cast<const float*>(reg + (g4 + e) * ROWB + (16 * t + col) * 4);
           float* o = reinterpret_cast<float*>(p.Out) + batch * p.o_bs + (int64_t)(n_base + 16 * t + col) * p.ldo + m_base + i * MI + g4;
-          if (p.out_accum != 0.0f) {
-            const f32x4_t old = *reinterpret_cast<const f32x4_t*>(o);
+          if constexpr (RMW) {
+            const f32x4_t old = oldv[i % OW][t];
 #pragma unroll
             for (int e = 0; e < 4; ++e) w[e] = __builtin_fmaf(p.out_accum, old[e], w[e]);
           }
@@ -369,6 +401,9 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x4_t (
         }
       }
     }
+    // this block's registers take the pieces of a later block
+    if (i + CW < C::FM) load_cin(i + CW);
+    if (RMW && i + OW < C::FM) load_old(i + OW);
   }
   if (p.slots_out != nullptr) {
     const float total = block_sum_f32<C::NT>(ssq, red);
@@ -664,7 +699,9 @@ constexpr int waitcnt_imm(int vmcnt, int lgkmcnt) {
 constexpr int SK_TILE = 256, SK_NT = 256, SK_FN = 8;                       // the tile, threads and fragment columns of SK_PARTS
 constexpr int64_t SK_IMAGE_FLOATS = (int64_t)SK_TILE * SK_TILE;            // one accumulator image
 enum { SK_NONE = 0, SK_FINISH = 2, SK_PARTS = 3 };
-template <class C, bool P_KS, bool Q_KS, int MODE, bool OUT_F32, bool EDGE, int STREAMK = 0>
+// RMW: GEMM mode with float32 output only, the variant that launch_fast takes for p.out_accum != 0 (see
+// gemm_epilogue_lds).
+template <class C, bool P_KS, bool Q_KS, int MODE, bool OUT_F32, bool EDGE, int STREAMK = 0, bool RMW = false>
 __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   constexpr int NS = C::NS, FM = C::FM, FN = C::FN, P_BYTES = C::P_BYTES, NT = C::NT;
   // The ring of operand slots; every LDS access of the K loop names its slot statically (ring[u] is a constant
@@ -680,6 +717,7 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: everything derived from it stays in SGPRs
   const int wm = wave % C::WGM, wn = wave / C::WGM;
+  static_assert(!RMW || (MODE == MODE_GEMM && OUT_F32 && !EDGE && (C::TN == 32 || C::TN == 64 || C::TN == 128)), "in-place variant: staged GEMM epilogue");
   static_assert(!STREAMK || (MODE == MODE_SYRK && !P_KS && !Q_KS && !EDGE && !OUT_F32 && C::NW == 4), "stream-K variant");
   static_assert(!STREAMK || (STREAMK == SK_FINISH ? (C::TILE_M == 128 && C::WGM == 2) : (C::TILE_M == SK_TILE && C::NT == SK_NT && C::FN == SK_FN)),
                 "SK_PARTS on 256 x 256 tiles, SK_FINISH on their 128 x 128 quarters");
@@ -928,8 +966,8 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
     const bool diag = (MODE == MODE_SYRK) && (tm == tn);
     if constexpr (MODE == MODE_GEMM && (C::TN == 32 || C::TN == 64 || C::TN == 128)) {
       __syncthreads();  // every wavefront has finished reading the ring: it can be reused as staging space
-      gemm_epilogue_lds<C, OUT_F32, EDGE>(p, acc, &ring[0][0], wave, lane, m0 + wm * C::TM, n0 + wn * C::TN, batch, alpha,
-                                          beta, red);
+      gemm_epilogue_lds<C, OUT_F32, EDGE, RMW>(p, acc, &ring[0][0], wave, lane, m0 + wm * C::TM, n0 + wn * C::TN, batch, alpha,
+                                               beta, red);
     } else if constexpr (SYRK_STAGED) {
       syrk_epilogue_lds<C, EDGE>(p, acc, &ring[0][0], lane, wm, wn, m0, n0, batch, diag, alpha, beta, beta2, shift, cin_pre);
     } else {

@@ -93,7 +93,15 @@ int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream, int64_t 
     else
       return fail(MI_ERR_UNSUPPORTED_SHAPE, "internal: %d x %d is not a whole number of %d x %d tiles", p.M, p.N, C::TILE_M, C::TILE_N);
   } else {
-    hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, false>), grid, block, 0, stream, q);
+    constexpr bool HAS_RMW_VARIANT = MODE == MODE_GEMM && OUT_F32 && (C::TN == 32 || C::TN == 64 || C::TN == 128);
+    if constexpr (HAS_RMW_VARIANT) {
+      if (p.out_accum != 0.0f)
+        hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, false, 0, true>), grid, block, 0, stream, q);
+      else
+        hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, false>), grid, block, 0, stream, q);
+    } else {
+      hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, false>), grid, block, 0, stream, q);
+    }
   }
   g_last_launch = LastLaunch{(int)grid.x, C::TILE_M, C::TILE_N, 1};
   hipError_t e = hipGetLastError();
