@@ -444,6 +444,9 @@ struct SyrkStage {
 // instruction touches MI rows with 32 contiguous bytes each -- whole 32-byte sectors, so nothing is fetched twice.
 // Issued before the K loop (first addend) or at the start of the epilogue (second), so that the burst of all
 // workgroups does not sit on the critical path.
+// Exactly NQUAD load instructions, whatever the position of the tile: the K loop that follows counts them in its
+// vmcnt waits.  Quads beyond the matrix (GUARD) therefore read a clamped, valid address instead of being skipped; the
+// values they deliver belong to outputs that are never stored.
 template <class C, bool GUARD>
 __device__ __forceinline__ void syrk_addend_fetch(const GemmParams& p, const uint16_t* __restrict__ Cb, int lane, int m_base,
                                                   int n_base, uint2 (&pre)[SyrkStage<C>::NQUAD]) {
@@ -454,10 +457,12 @@ __device__ __forceinline__ void syrk_addend_fetch(const GemmParams& p, const uin
 #pragma unroll
     for (int j = 0; j < C::FN; ++j)
 {
-        const int m = m_base + i * MI + frow, n = n_base + j * MI + 4 * fk;
-        uint2 v = make_uint2(0u, 0u);
-        if (!GUARD || (m < p.M && n < p.N)) v = *reinterpret_cast<const uint2*>(Cb + (int64_t)m * p.ldc + n);
-        pre[i * C::FN + j] = v;
+        int m = m_base + i * MI + frow, n = n_base + j * MI + 4 * fk;
+        if constexpr (GUARD) {
+          m = m < p.M ? m : p.M - 1;
+          n = n + 4 <= p.N ? n : p.N - 4;
+        }
+        pre[i * C::FN + j] = *reinterpret_cast<const uint2*>(Cb + (int64_t)m * p.ldc + n);
       }
 }
 
@@ -888,8 +893,12 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   };
   // `steady` (a compile-time flag) marks tiles in the middle of the K loop: tile kt+NS exists (so the vacated
   // slot is refilled and NS-2 younger tiles stay in flight at the wait), and the tile body is branch free.
-  auto k_tile = [&](auto steady, int kt, int cur_slot, const char* cur, const char* nxt) {
+  // `extra` (compile time) and `with_extra` (run time, uniform): register loads issued between this wavefront's loads
+  // of tile kt+1 and the wait below (the addend fetch in front of tile 0) that the wait must not sit out.
+  auto k_tile = [&](auto steady, int kt, int cur_slot, const char* cur, const char* nxt, auto extra, bool with_extra) {
     constexpr bool STEADY = decltype(steady)::value;
+    constexpr int EXTRA = decltype(extra)::value;
+    static_assert((NS - 2) * LOADS_PER_TILE + EXTRA < 64, "vmcnt is a 6-bit counter");
     const int prev_slot = (cur_slot + NS - 1) % NS;  // receives the later parts of tile kt-1+NS
     if (!STEADY && PARTS > 1 && kt + NS - 1 < nk) issue_parts(prev_slot, 1, PARTS);
 #pragma unroll
@@ -903,7 +912,10 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
       }
     }
     // own loads of tile kt+1 have landed; own reads of `cur` are done
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(STEADY ? (NS - 2) * LOADS_PER_TILE : 0, 0));
+    if (STEADY && EXTRA > 0 && with_extra)
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm((NS - 2) * LOADS_PER_TILE + EXTRA, 0));
+    else
+      __builtin_amdgcn_s_waitcnt(waitcnt_imm(STEADY ? (NS - 2) * LOADS_PER_TILE : 0, 0));
     __syncthreads();
     if (STEADY) {
       k_step(std::true_type{}, std::integral_constant<int, 0>{}, (NQ - 1) & 1, nxt, 0, cur_slot);
@@ -930,12 +942,18 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
     else
       __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
     __syncthreads();
+    // The first addend is requested here, behind the loads of the first tiles and in front of everything the K loop
+    // issues.  The wait at the end of tile 0 (for tile 1, whose loads are older) lets these NQUAD loads stay in
+    // flight: sat out there, the burst of all workgroups cost 4 us per launch.  From tile 1 on every wait is for loads
+    // that are younger than the addend, so it has arrived by then whatever the count says.
+    bool addend_in_flight = false;
     if constexpr (CIN_EARLY) {
-      // these loads are older than every direct-to-LDS load issued from here on, so the vmcnt waits of the K
-      // loop cover them as well
-      if (p.Cin != nullptr)
+      if (p.Cin != nullptr) {
         syrk_addend_fetch<C, EDGE>(p, p.Cin + batch * p.c_bs, lane, m0 + wm * C::TM, n0 + wn * C::TN, cin_pre);
+        addend_in_flight = true;
+      }
     }
+    constexpr int ADDEND_LOADS = CIN_EARLY ? SyrkStage<C>::NQUAD : 0;
     if (idle_wave) {
       for (int kt = 0; kt < nk; ++kt) {
         const int cur_slot = kt % NS, prev_slot = (cur_slot + NS - 1) % NS;
@@ -948,13 +966,15 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
       fetch(ring[0], 0, 0);
       int kt = 0;
       for (; kt + 2 * NS - 1 < nk; kt += NS) {  // every tile of this round is a steady one
+        k_tile(std::true_type{}, kt, 0, ring[0], ring[1 % NS], std::integral_constant<int, ADDEND_LOADS>{}, addend_in_flight && kt == 0);
 #pragma unroll
-        for (int u = 0; u < NS; ++u) k_tile(std::true_type{}, kt + u, u, ring[u], ring[(u + 1) % NS]);
+        for (int u = 1; u < NS; ++u)
+          k_tile(std::true_type{}, kt + u, u, ring[u], ring[(u + 1) % NS], std::integral_constant<int, 0>{}, false);
       }
       for (; kt < nk; kt += NS) {
 #pragma unroll
         for (int u = 0; u < NS; ++u)
-          if (kt + u < nk) k_tile(std::false_type{}, kt + u, u, ring[u], ring[(u + 1) % NS]);
+          if (kt + u < nk) k_tile(std::false_type{}, kt + u, u, ring[u], ring[(u + 1) % NS], std::integral_constant<int, 0>{}, false);
       }
     }
     mfma_drain();

@@ -76,7 +76,8 @@ def accumulator_hazards(lines):
         if not t.startswith("v_mfma"):
             continue
         for x in text[k + 1:k + 13]:
-            if x.startswith("v_mfma") or x.startswith("s_nop 7"):
+            # (what follows an unconditional branch in the text does not follow it at run time)
+            if x.startswith("v_mfma") or x.startswith("s_nop 7") or x.startswith("s_branch") or x.startswith("s_endpgm"):
                 break
             if touches(x):
                 bad.append(f"after MFMA, before the drain: {x}")
@@ -104,6 +105,14 @@ def test_detector_flags_swaps_and_spills():
 	v_accvgpr_read_b32 v1, a0
 """.splitlines()
     assert accumulator_hazards(spill) == ["after MFMA, before the drain: scratch_store_dwordx4 off, a[232:235], off offset:100"]
+    other_path = """
+	v_mfma_f32_16x16x32_bf16 a[48:51], v[14:17], v[46:49], a[48:51]
+	s_cbranch_scc1 .LBB0_9
+	s_branch .LBB0_1
+.LBB0_8:
+	v_accvgpr_write_b32 a48, 0
+""".splitlines()
+    assert accumulator_hazards(other_path) == []  # the block after the unconditional branch is entered from elsewhere
     clean = """
 .LBB0_1:
 	v_mfma_f32_16x16x32_bf16 a[0:3], v[14:17], v[46:49], a[0:3]
