@@ -249,9 +249,12 @@ def syrk_epilogue_accesses(cfg, M, m0, n0, diag, guard, skip_upper, addends, out
             for j in range(fm):
                 m = m0 + wm * tm + i * MI + (LANES & 15)
                 n = n0 + wn * tm + j * MI + 4 * (LANES >> 4)
-                on = (m < M) & (n < M) if guard else np.ones(64, bool)
+                if guard:
+                    # every lane loads (the K loop counts these loads in its vmcnt waits): quads beyond the matrix
+                    # read a clamped address
+                    m, n = np.minimum(m, M - 1), np.where(n + 4 <= M, n, M - 4)
                 if addends:
-                    cmat.check(m[on], n[on], 4, "addend fetch")
+                    cmat.check(m, n, 4, "addend fetch")
     # store counts in the tile's own window (rows from m0, columns from n0) and in the mirrored window
     direct = np.zeros((tile, tile), dtype=np.int32)
     mirror = direct if diag else np.zeros((tile, tile), dtype=np.int32)

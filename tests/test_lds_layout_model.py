@@ -488,3 +488,72 @@ def test_transposed_reads_of_the_gemm_staging_rows_are_conflict_free(tn):
                 seen[row][col] += 1
             assert len(banks) == 64
     assert all(v == 1 for r in seen for v in r)
+
+
+@pytest.mark.parametrize("ns,lpt,nquad", [(3, 12, 36), (3, 8, 16), (2, 8, 16)])
+@pytest.mark.parametrize("nk", [1, 2, 3, 5, 6, 7, 8, 9, 12, 13, 64])
+@pytest.mark.parametrize("addend", [False, True])
+def test_vmcnt_waits_of_the_k_loop(ns, lpt, nquad, nk, addend):
+    """The K loop of the fast kernel tracks its direct-to-LDS loads with s_waitcnt vmcnt(N): vector memory loads come
+    back in the order they were issued, so "at most N outstanding" means "everything but the N youngest has landed".
+    This replays, per wavefront, the order in which the kernel issues the loads of its K tiles (cut into parts) and the
+    register loads of the first addend of a lower-triangle product (nquad loads, issued between the prologue and
+    tile 0), and every wait with its count, and asserts that at the wait that ends tile kt all loads of tile kt + 1
+    have landed -- and that the wait of tile 0 does not sit out the addend (the reason for its larger count), while
+    the addend has landed at the wait of tile 1."""
+    nq = 2                                             # k-steps per tile (BK / 32)
+    parts = nq if ns >= 3 and lpt % nq == 0 else 1
+    pl = lpt // parts
+    issued = []                                        # tags in issue order
+    landed = 0                                         # loads [0, landed) have come back
+
+    def issue(tag, count):
+        issued.extend([tag] * count)
+
+    def wait(n):
+        nonlocal landed
+        landed = max(landed, len(issued) - n)
+
+    def tile_landed(t):
+        return all(i < landed for i, tag in enumerate(issued) if tag == t)
+
+    for t in range(ns - 1):
+        if t < nk:
+            issue(t, lpt)
+    if ns - 1 < nk:
+        issue(ns - 1, pl)
+    wait((ns - 2) * lpt + pl if nk >= ns else 0)
+    assert tile_landed(0)
+    if addend:
+        issue("addend", nquad)
+    kt = 0
+    while kt + 2 * ns - 1 < nk:                        # steady rounds
+        for u in range(ns):
+            t = kt + u
+            for q in range(nq - 1):
+                if parts > 1:
+                    issue(t - 1 + ns, pl)              # part q + 1 of tile t - 1 + NS
+            extra = nquad if (addend and t == 0) else 0
+            assert (ns - 2) * lpt + extra < 64         # 6-bit counter
+            wait((ns - 2) * lpt + extra)
+            assert tile_landed(t + 1)
+            if addend and t == 0:
+                assert not all(i < landed for i, tag in enumerate(issued) if tag == "addend")
+            if addend and t == 1:
+                assert tile_landed("addend")
+            issue(t + ns, pl)                          # part 0 of tile t + NS into the slot just vacated
+        kt += ns
+    while kt < nk:                                     # the rounds that are not all steady
+        for u in range(ns):
+            t = kt + u
+            if t >= nk:
+                break
+            if parts > 1 and t + ns - 1 < nk:
+                issue(t - 1 + ns, (parts - 1) * pl)
+            wait(0)
+            assert t + 1 >= nk or tile_landed(t + 1)
+            if t + ns < nk:
+                issue(t + ns, pl)
+        kt += ns
+    assert landed == len(issued)
+    assert all(issued.count(t) == lpt for t in range(nk))  # every tile loaded once, completely
