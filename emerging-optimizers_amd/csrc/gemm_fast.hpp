@@ -106,7 +106,10 @@ __device__ __forceinline__ void dma16_sv(uint64_t sbase, uint32_t voff, uint32_t
 //     lanes' offsets inside a block repeat with a short period in b (the swizzle phase), so the loader keeps
 //     one scalar base plus NV lane-offset registers.
 //   CLAMP = true: rows beyond `rows_valid` are redirected to the last valid row (they only feed output rows
-//     that the epilogue never stores); every load keeps its own per-lane pointer.
+//     that the epilogue never stores); every load keeps its own lane-offset register (32 bits, relative to the
+//     first row of the tile: the launcher refuses leading dimensions for which TILE rows do not fit), the base
+//     is the same scalar as above.  (With a 64-bit pointer per load, advanced by vector adds in every K tile, the
+//     lower-triangle product of 4096 rows -- 192 does not divide them -- was 3 % slower than that of 4224 rows.)
 template <class C, bool KS, int ROWS, bool CLAMP>
 struct FastLoader {
   static constexpr int LPT = ROWS * C::BK * 2 / 1024 / C::NW;
@@ -115,17 +118,16 @@ struct FastLoader {
   // period of the swizzle phase in the block index
   static constexpr int PERIOD = KS ? (KS_CHUNKS / KS_ROWS_PER_KB > 0 ? KS_CHUNKS / KS_ROWS_PER_KB : 1) : (C::BK == 64 ? 2 : 1);
   static constexpr bool PERIODIC = LPT % PERIOD == 0;  // then the phase of load i is i % PERIOD for every wavefront
-  static constexpr int NV = CLAMP ? 1 : (PERIODIC ? (PERIOD < LPT ? PERIOD : LPT) : LPT);
+  static constexpr int NV = CLAMP ? LPT : (PERIODIC ? (PERIOD < LPT ? PERIOD : LPT) : LPT);
   static_assert(!KS || ROWS == 256 || ROWS == 128, "K-strided LDS layout is laid out for 128/256-wide tiles");
   // (a K-strided tile at the edge of its operand would need clamping along the contiguous dimension, which a
   // 16-byte load cannot do per element: the launcher never sends such a tile here)
   static_assert(!(KS && CLAMP), "edge tiles of K-strided operands are not served by the fast kernel");
 
-  const uint16_t* gp[CLAMP ? LPT : 1];  // CLAMP: per-load pointers
-  uint32_t voff[NV];                    // !CLAMP: per-lane byte offsets inside a block
-  uint64_t base;                        // !CLAMP: byte address of this wavefront's first block (uniform)
+  uint32_t voff[NV];                    // per-lane byte offsets: inside a block (!CLAMP), from the tile's first row (CLAMP)
+  uint64_t base;                        // byte address of this wavefront's first block (!CLAMP) or of the tile (CLAMP); uniform
   int64_t block_step;                   // !CLAMP: bytes between consecutive blocks (uniform)
-  int64_t step;                         // advance per K tile: elements (CLAMP) or bytes (!CLAMP)
+  int64_t step;                         // advance per K tile in bytes
 
   // lane's element offset inside block b, relative to the block's first element
   static __device__ __forceinline__ int64_t lane_part(int b, int64_t ld, int lane) {
@@ -149,9 +151,11 @@ struct FastLoader {
         const int c = kc_slot<C::BK>(row, lane % C::CPR);
         int gr = row0 + row;
         gr = gr < rows_valid ? gr : rows_valid - 1;
-        gp[i] = opbase + (int64_t)gr * ld + c * 8;
+        voff[i] = (uint32_t)(2 * ((int64_t)(gr - row0) * ld + c * 8));
       }
-      step = C::BK;
+      base = (uint64_t)(uintptr_t)(opbase + (int64_t)row0 * ld);
+      block_step = 0;
+      step = 2 * (int64_t)C::BK;
     } else {
       const int b0 = wave * LPT;
 #pragma unroll
@@ -166,18 +170,11 @@ struct FastLoader {
   // in the target ring slot.  advance() moves on to the next K tile once all LPT loads are out.
   __device__ __forceinline__ void issue_one(uint32_t lds_tile, int wave, int i) {
     if constexpr (CLAMP)
-      dma16(gp[i], lds_tile + (wave * LPT + i) * 1024);
+      dma16_sv(base, voff[i], lds_tile + (wave * LPT + i) * 1024);
     else
       dma16_sv(base + (uint64_t)(i * block_step), voff[PERIODIC ? i % NV : i], lds_tile + (wave * LPT + i) * 1024);
   }
-  __device__ __forceinline__ void advance() {
-    if constexpr (CLAMP) {
-#pragma unroll
-      for (int i = 0; i < LPT; ++i) gp[i] += step;
-    } else {
-      base += step;
-    }
-  }
+  __device__ __forceinline__ void advance() { base += step; }
 };
 
 // MFMA fragment (8 bf16 along k per lane) of a K-contiguous tile for 16 consecutive rows starting at `row_base`,
@@ -966,10 +963,16 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
       fetch(ring[0], 0, 0);
       int kt = 0;
       for (; kt + 2 * NS - 1 < nk; kt += NS) {  // every tile of this round is a steady one
-        k_tile(std::true_type{}, kt, 0, ring[0], ring[1 % NS], std::integral_constant<int, ADDEND_LOADS>{}, addend_in_flight && kt == 0);
+        if constexpr (ADDEND_LOADS > 0) {
+          k_tile(std::true_type{}, kt, 0, ring[0], ring[1 % NS], std::integral_constant<int, ADDEND_LOADS>{}, addend_in_flight && kt == 0);
 #pragma unroll
-        for (int u = 1; u < NS; ++u)
-          k_tile(std::true_type{}, kt + u, u, ring[u], ring[(u + 1) % NS], std::integral_constant<int, 0>{}, false);
+          for (int u = 1; u < NS; ++u)
+            k_tile(std::true_type{}, kt + u, u, ring[u], ring[(u + 1) % NS], std::integral_constant<int, 0>{}, false);
+        } else {
+#pragma unroll
+          for (int u = 0; u < NS; ++u)
+            k_tile(std::true_type{}, kt + u, u, ring[u], ring[(u + 1) % NS], std::integral_constant<int, 0>{}, false);
+        }
       }
       for (; kt < nk; kt += NS) {
 #pragma unroll

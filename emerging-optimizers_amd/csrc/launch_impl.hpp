@@ -84,6 +84,9 @@ int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream, int64_t 
     grid = dim3((unsigned)tiles, (unsigned)batch, 1);
   }
   const bool edge = (p.M % C::TILE_M) != 0 || (p.N % C::TILE_N) != 0;
+  // (the loaders of an edge tile address its rows with 32-bit byte offsets from the tile's first row)
+  if (edge && ((int64_t)C::TILE_M * p.ldp >= ((int64_t)1 << 31) || (int64_t)C::TILE_N * p.ldq >= ((int64_t)1 << 31)))
+    return fail(MI_ERR_UNSUPPORTED_SHAPE, "internal: leading dimension too large for an edge tile");
   // Only the lower-triangle product of K-contiguous operands has a variant for tiles that overhang the matrix
   // (rows clamped in the loaders, guarded epilogue).
   constexpr bool HAS_EDGE_VARIANT = MODE == MODE_SYRK && !P_KS && !Q_KS;

@@ -204,7 +204,10 @@ static int launch_class(TileClass tc, const GemmParams& p, int64_t batch, hipStr
   // Lower-triangle products of 256 rows and more whose rows are whole 128-row tiles also take the direct-to-LDS
   // kernels (general kernel 1.25 - 2.45x slower over 129 shapes, n = 256 .. 768, batch 1 .. 64); other small
   // matrices stay on the general kernel.
-  const bool big = (p.M >= 1024 && p.N >= 1024) || (MODE == MODE_SYRK && p.M >= 256 && p.M % 128 == 0);
+  // (leading dimensions beyond 4M elements -- a 4096-row bf16 operand of more than 32 GB -- stay on the general kernel:
+  // the fast loaders address the rows of a tile with 32-bit byte offsets)
+  const bool ld_ok = p.ldp < (1 << 22) && p.ldq < (1 << 22);
+  const bool big = ld_ok && ((p.M >= 1024 && p.N >= 1024) || (MODE == MODE_SYRK && p.M >= 256 && p.M % 128 == 0));
   if (k_ok && big) {
     if constexpr (MODE == MODE_SYRK) {
       static_assert(P_KS == Q_KS, "the lower-triangle product reads one operand in one layout");
