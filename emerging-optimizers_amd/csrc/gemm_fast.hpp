@@ -507,19 +507,42 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, f32x4_t (
     // Both addends arrive in accumulator layout: the first was requested before the K loop, the second is
     // requested now and consumed after the first.
     uint2 c2[S::NQUAD];
-    if (use_c2) syrk_addend_fetch<C, GUARD>(p, Cb2, lane, m0 + mw, n0 + nw, c2);
+    if (use_c2) {
+      syrk_addend_fetch<C, GUARD>(p, Cb2, lane, m0 + mw, n0 + nw, c2);
+      // while those loads are on their way (a burst of all workgroups: 4 - 5 us), alpha and the first addend go into
+      // the accumulators; the same operations in the same order as below, so the result does not change
 #pragma unroll
-    for (int i = 0; i < FM; ++i)
+      for (int i = 0; i < FM; ++i)
 #pragma unroll
-      for (int j = 0; j < FN; ++j) {
-        const int ml = mw + i * MI + frow, nl = nw + j * MI + 4 * fk;
-        f32x4_t v;
+        for (int j = 0; j < FN; ++j) {
+          f32x4_t v;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][r];
-        if (use_c) add(v, cin_pre[i * FN + j], beta);
-        if (use_c2) add(v, c2[i * FN + j], beta2);
-        val[i][j] = finish(v, ml, nl);
-      }
+          for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][r];
+          if (use_c) add(v, cin_pre[i * FN + j], beta);
+          acc[i][j] = v;
+        }
+      asm volatile("" ::: "memory");  // (keeps the uses of c2 behind this block)
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+          f32x4_t v = acc[i][j];
+          add(v, c2[i * FN + j], beta2);
+          val[i][j] = finish(v, mw + i * MI + frow, nw + j * MI + 4 * fk);
+        }
+    } else {
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+          const int ml = mw + i * MI + frow, nl = nw + j * MI + 4 * fk;
+          f32x4_t v;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) v[r] = alpha * acc[i][j][r];
+          if (use_c) add(v, cin_pre[i * FN + j], beta);
+          val[i][j] = finish(v, ml, nl);
+        }
+    }
     __syncthreads();  // every wavefront has left the K loop: the ring can be reused as staging space
   } else {
     // Large tile: every addend tile goes through the staging area.  The workgroup copies it there row by row (16 bytes
