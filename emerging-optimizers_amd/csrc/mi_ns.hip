@@ -103,7 +103,8 @@ int device_cus() {
 //                               L      F      s      s0     s1
 //      128 x 128, one per CU   12.1    5.5   0.48   0.29   0.11     (n % 128 == 0)
 //      128 x 128, two per CU    8.9    7.4   0.84   0.43   0.45     (n % 128 == 0; per pair of tiles)
-//      192 x 192               14.6   10.8   0.81   0.50   0.26
+//      192 x 192               14.6   10.8   0.79   0.50   0.26     (s was 0.81 in the fit; the loaders of edge tiles,
+//                                                                 which most of the fitted shapes have, got cheaper since)
 //      256 x 256               12.3   12.9   1.32   0.88   0.43     (n % 256 == 0)
 //    Short K or few tiles favour the small tiles, long K with many tiles the 192 x 192 tile, and shapes whose
 //    256 x 256 tiles fill whole rounds (8 x 1792: 224 tiles) or that 192 divides badly the 256 x 256 tile.
@@ -115,7 +116,7 @@ struct TileCost {
   }
 };
 static constexpr TileCost COST_128{12.1, 5.5, 0.48, 0.29, 0.11}, COST_128X2{8.9, 7.4, 0.84, 0.43, 0.45},
-    COST_192{14.6, 10.8, 0.81, 0.50, 0.26}, COST_256{12.3, 12.9, 1.32, 0.88, 0.43};
+    COST_192{14.6, 10.8, 0.79, 0.50, 0.26}, COST_256{12.3, 12.9, 1.32, 0.88, 0.43};
 enum SyrkTile { SYRK_TILE_NONE, SYRK_TILE_128, SYRK_TILE_128X2, SYRK_TILE_192, SYRK_TILE_256 };
 // `k_strided`: the operand is stored transposed; its LDS layout exists for 128- and 256-row tiles only, and not for
 // tiles that overhang the matrix, so there may be no fast tile at all.
