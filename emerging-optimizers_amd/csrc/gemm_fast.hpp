@@ -548,32 +548,29 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, f32x4_t (
     // Large tile: every addend tile goes through the staging area.  The workgroup copies it there row by row (16 bytes
     // per lane, whole rows per 32 lanes), each lane adds its quads to its accumulators, and the next addend or the
     // finished values overwrite it.
+    // All NCH 16-byte pieces of an addend tile are requested at once (in batches of eight with a wait after each, every
+    // batch sat out a memory latency of its own: 7 us per addend and tile), the first addend before the accumulators
+    // are scaled, the second as soon as the first has left its registers for the staging area, so that it is on its
+    // way while the first is added.
+    uint4 buf[NCH];
+    auto request = [&](const uint16_t* __restrict__ src) {
 #pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-      for (int j = 0; j < FN; ++j)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) acc[i][j][r] *= alpha;
-    auto stage_addend = [&](const uint16_t* __restrict__ src, float coef) {
-      __syncthreads();  // nobody reads the area any more (the ring, or the previous addend)
-      constexpr int BATCH = 8;
-      static_assert(NCH % BATCH == 0, "addend copy goes in batches");
-#pragma unroll 1
-      for (int it0 = 0; it0 < NCH; it0 += BATCH) {
-        uint4 buf[BATCH];
-#pragma unroll
-        for (int u = 0; u < BATCH; ++u) {
-          const int c = tid + (it0 + u) * C::NT, row = c / CPRW, c8 = c % CPRW;
-          const int gr = m0 + row, gc = n0 + c8 * 8;
-          buf[u] = make_uint4(0u, 0u, 0u, 0u);
-          if (!GUARD || (gr < p.M && gc < p.N)) buf[u] = *reinterpret_cast<const uint4*>(src + (int64_t)gr * p.ldc + gc);
-        }
-#pragma unroll
-        for (int u = 0; u < BATCH; ++u) {
-          const int c = tid + (it0 + u) * C::NT, row = c / CPRW, c8 = c % CPRW;
-          *reinterpret_cast<uint4*>(lds + (row * LDT + c8 * 8) * 2) = buf[u];
-        }
+      for (int u = 0; u < NCH; ++u) {
+        const int c = tid + u * C::NT, row = c / CPRW, c8 = c % CPRW;
+        const int gr = m0 + row, gc = n0 + c8 * 8;
+        buf[u] = make_uint4(0u, 0u, 0u, 0u);
+        if (!GUARD || (gr < p.M && gc < p.N)) buf[u] = *reinterpret_cast<const uint4*>(src + (int64_t)gr * p.ldc + gc);
       }
+    };
+    auto park = [&]() {  // registers -> staging area (behind a barrier: nobody reads the area any more)
+      __syncthreads();
+#pragma unroll
+      for (int u = 0; u < NCH; ++u) {
+        const int c = tid + u * C::NT, row = c / CPRW, c8 = c % CPRW;
+        *reinterpret_cast<uint4*>(lds + (row * LDT + c8 * 8) * 2) = buf[u];
+      }
+    };
+    auto add_staged = [&](float coef) {
       __syncthreads();
       if (active) {
 #pragma unroll
@@ -585,8 +582,23 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, f32x4_t (
           }
       }
     };
-    if (use_c) stage_addend(Cb, beta);
-    if (use_c2) stage_addend(Cb2, beta2);
+    if (use_c) request(Cb);
+    else if (use_c2) request(Cb2);
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[i][j][r] *= alpha;
+    if (use_c) {
+      park();
+      if (use_c2) request(Cb2);
+      add_staged(beta);
+    }
+    if (use_c2) {
+      park();
+      add_staged(beta2);
+    }
     __syncthreads();  // the area is free for the finished values
   }
   // finished bf16 quad (i, j) of this lane
