@@ -42,8 +42,8 @@ TOL = 1e-2
 # (2 x X X^T, 14 m x m products), and of one GEMM+AXPY (both launches): FETCH_SIZE and WRITE_SIZE of two
 # `rocprofv3 --pmc` runs of this file (KiB per dispatch), each scaled by what the same counter reads for sumsq_kernel
 # of the same run, whose traffic is known (229 376 KiB read, 114 696 KiB written): factors 1.9994 and 0.9998.
-TRI_KERNEL_TRAFFIC_BYTES = int((129187.8 * 1.9994 + 32768.0 * 0.9998) * 1024)
-GEMM_AXPY_TRAFFIC_BYTES = int(((406675.4 + 146813.2) * 1.9994 + (98328.0 + 16392.0) * 0.9998) * 1024)
+TRI_KERNEL_TRAFFIC_BYTES = int((129117.8 * 1.9994 + 32768.0 * 0.9998) * 1024)
+GEMM_AXPY_TRAFFIC_BYTES = int(((407572.7 + 146821.6) * 1.9994 + (98328.0 + 16392.0) * 0.9998) * 1024)
 M, N, NS_STEPS = 4096, 14336, 5
 COEFFS = [(3.4445, -4.7750, 2.0315)] * NS_STEPS  # "simple" table cycled
 MIN_WARMUP, MIN_TIMED = 3, 20
