@@ -4,9 +4,11 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -26,6 +28,54 @@ int fail(int code, const char* fmt, ...) {
   va_end(ap);
   g_last_error = buf;
   return code;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Process-wide options (mi_set_option / mi_get_option).  Each is one atomic integer; its initial value comes from an
+// environment variable that is read once, when the first option is looked up.  Nothing on the call path reads the
+// environment.
+// ---------------------------------------------------------------------------------------------
+enum Opt { OPT_STREAMK = 0, OPT_SYRK_TRANSPOSE, OPT_HEAD_APPLY, OPT_HEAD_FRONT, OPT_TALL_DIRECT, OPT_NS_PAIRS, OPT_COUNT };
+struct OptDesc {
+  const char* name;
+  const char* env;
+  int lo, hi, initial;
+};
+static constexpr OptDesc OPT_TABLE[OPT_COUNT] = {
+    {"streamk", "MI_STREAMK", -1, 1, -1},                // -1 by the cost model, 0 never, 1 whenever the shape qualifies
+    {"syrk_transpose", "MI_SYRK_TRANSPOSE", -1, 1, -1},  // -1 by the cost model, 0 never, 1 whenever the shape qualifies
+    {"head_apply", "MI_HEAD_APPLY", 0, 1, 1},            // slab kernel for the B X product of 128-row matrices
+    {"head_front", "MI_HEAD_FRONT", 0, 1, 1},            // input pass of 128-row matrices that leaves the Gram partials
+    {"tall_direct", "MI_TALL_DIRECT", 0, 1, 1},          // last product of a tall input writes the result transposed
+    {"ns_pairs", "MI_NS_PAIRS", -1, 2, -1},              // -1 by shape, 0 single steps, 1 never three at once, 2 pairs at every size
+};
+static std::atomic<int> g_opt[OPT_COUNT];
+static std::once_flag g_opt_once;
+
+static void opt_init() {
+  std::call_once(g_opt_once, [] {
+    for (int i = 0; i < OPT_COUNT; ++i) {
+      int v = OPT_TABLE[i].initial;
+      if (const char* e = getenv(OPT_TABLE[i].env)) {
+        // numbers as they are; for MI_NS_PAIRS also the words "pairs" (1) and "force" (2)
+        if (e[0] == 'p') v = 1;
+        else if (e[0] == 'f') v = 2;
+        else if ((e[0] >= '0' && e[0] <= '9') || e[0] == '-') v = atoi(e);
+        if (v < OPT_TABLE[i].lo || v > OPT_TABLE[i].hi) v = OPT_TABLE[i].initial;
+      }
+      g_opt[i].store(v, std::memory_order_relaxed);
+    }
+  });
+}
+static int opt(Opt o) {
+  opt_init();
+  return g_opt[o].load(std::memory_order_relaxed);
+}
+static int opt_index(const char* name) {
+  if (name)
+    for (int i = 0; i < OPT_COUNT; ++i)
+      if (strcmp(name, OPT_TABLE[i].name) == 0) return i;
+  return -1;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -172,12 +222,12 @@ static bool streamk_wanted(int64_t n, int64_t batch, int64_t k, bool k_strided, 
   *plan = StreamKPlan{0, 0, 0};
   const int cus = streamk_cus();
   if (k_strided || n < 1024 || n % 256 != 0 || k % 64 != 0 || k < 64 || cus < 8) return false;
-  const char* env = getenv("MI_STREAMK");  // "0": never, "1": whenever the shape qualifies (tests), else by the model
-  if (env && env[0] == '0') return false;
+  const int mode = opt(OPT_STREAMK);  // 0: never, 1: whenever the shape qualifies (tests), else by the model
+  if (mode == 0) return false;
   const int64_t t = n / 256, tiles = t * (t + 1) / 2 * batch, kt = k / 64;
   if (tiles / cus > 4096) return false;
   *plan = streamk_plan(tiles, (int)kt, cus);
-  if (env && env[0] == '1') return true;
+  if (mode == 1) return true;
   if (plan->splits < 2) return false;
   double best = 0.0;
   pick_syrk_tile(n, batch, k, false, &best);
@@ -195,6 +245,7 @@ static bool gemm_prefers_half_tiles(int64_t m, int64_t n, int64_t batch) {
 // transposed (the staged epilogue of the fast kernel; mirrors the choices of launch_class below).
 static bool gemm_transposed_out_ok(int64_t m, int64_t n) {
   if (m % 64 != 0 || m < 64) return false;
+  if (m >= (1 << 22) || n >= (1 << 22)) return false;  // (launch_class: such leading dimensions stay on the general kernel)
   if (m >= 1024 && n >= 1024 && m % 256 == 0 && n % 256 == 0) return true;
   return m % 128 == 0 && m < 1024 && n % 256 == 0 && n >= 256;
 }
@@ -322,10 +373,10 @@ __global__ void __launch_bounds__(256) transpose_bf16_kernel(const uint16_t* __r
 // 4 TB/s (read + write).  Bytes of scratch the copy needs, or 0 when the model expects no gain.
 static size_t transposed_copy_bytes(int64_t n, int64_t batch, int64_t k) {
   if (n < 1024 || k % 64 != 0) return 0;  // (below, both layouts go to the general kernel)
-  const char* env = getenv("MI_SYRK_TRANSPOSE");  // "0": never, "1": always (tests), else by the model
-  if (env && env[0] == '0') return 0;
+  const int mode = opt(OPT_SYRK_TRANSPOSE);  // 0: never, 1: always (tests), else by the model
+  if (mode == 0) return 0;
   const size_t bytes = ((size_t)batch * n * k * 2 + 255) / 256 * 256;
-  if (env && env[0] == '1') return bytes;
+  if (mode == 1) return bytes;
   if (n < 2048) return 0;  // (launches of a few dozen small tiles: the model is too coarse there, measured no gain)
   double strided = 0.0, contiguous = 0.0;
   if (pick_syrk_tile(n, batch, k, true, &strided) == SYRK_TILE_NONE) return bytes;
@@ -334,13 +385,10 @@ static size_t transposed_copy_bytes(int64_t n, int64_t batch, int64_t k) {
   return contiguous + copy < 0.95 * strided ? bytes : 0;
 }
 
-// `other` != null computes alpha * A other^T (symmetric in exact arithmetic; the lower triangle is computed and
-// mirrored), and `C2` is a second addend laid out like C whose coefficient a SHIFT_GROUP_* mode supplies.
-static int syrk_impl(const void* A, int64_t batch, int64_t n, int64_t k, int64_t a_bs, int64_t a_ld, int a_trans,
-                     const void* C, int64_t c_bs, int64_t c_ld, float alpha, float beta, void* D, int64_t d_bs,
-                     int64_t d_ld, int skip_upper, hipStream_t stream, const ShiftArgs* sh = nullptr,
-                     const void* other = nullptr, const void* C2 = nullptr, void* workspace = nullptr,
-                     size_t workspace_bytes = 0) {
+// Argument checks of the lower-triangle product, shared by every entry that leads to it: nothing is launched for a
+// call that fails one of them.
+static int syrk_validate(const void* A, int64_t batch, int64_t n, int64_t k, int64_t a_bs, int64_t a_ld, int a_trans,
+                         const void* C, int64_t c_bs, int64_t c_ld, float beta, const void* D, int64_t d_bs, int64_t d_ld) {
   if (!A || !D) return fail(MI_ERR_BAD_ARG, "mi_syrk_bf16: A and D must not be null");
   if (batch < 0 || n < 0 || k < 0) return fail(MI_ERR_BAD_ARG, "mi_syrk_bf16: negative extent");
   if (beta != 0.0f && !C) return fail(MI_ERR_BAD_ARG, "mi_syrk_bf16: C is null but beta != 0");
@@ -351,6 +399,17 @@ static int syrk_impl(const void* A, int64_t batch, int64_t n, int64_t k, int64_t
     return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_syrk_bf16: pointers must be 16-byte aligned");
   if (a_ld < (a_trans ? n : k) || d_ld < n || (C && c_ld < n)) return fail(MI_ERR_BAD_ARG, "mi_syrk_bf16: leading dimension too small");
   if (n > (1 << 30) || k > (1 << 30)) return fail(MI_ERR_UNSUPPORTED_SHAPE, "mi_syrk_bf16: extent too large");
+  return MI_OK;
+}
+
+// `other` != null computes alpha * A other^T (symmetric in exact arithmetic; the lower triangle is computed and
+// mirrored), and `C2` is a second addend laid out like C whose coefficient a SHIFT_GROUP_* mode supplies.
+static int syrk_impl(const void* A, int64_t batch, int64_t n, int64_t k, int64_t a_bs, int64_t a_ld, int a_trans,
+                     const void* C, int64_t c_bs, int64_t c_ld, float alpha, float beta, void* D, int64_t d_bs,
+                     int64_t d_ld, int skip_upper, hipStream_t stream, const ShiftArgs* sh = nullptr,
+                     const void* other = nullptr, const void* C2 = nullptr, void* workspace = nullptr,
+                     size_t workspace_bytes = 0) {
+  if (int rc = syrk_validate(A, batch, n, k, a_bs, a_ld, a_trans, C, c_bs, c_ld, beta, D, d_bs, d_ld)) return rc;
   if (batch == 0 || n == 0) return MI_OK;
 
   GemmParams p{};
@@ -434,8 +493,8 @@ static int gemm_axpy_impl(const void* Bm, int64_t b_bs, int64_t b_ld, const void
     p.N = (int)n;
     // 128-row matrices inside the driver: one workgroup per 512-column slice does product, addend and the next
     // group's partial Gram matrices on slabs it keeps in LDS
-    const char* head_env = getenv("MI_HEAD_APPLY");  // "0": the general GEMM+AXPY kernels also for 128-row matrices (A/B runs, tests)
-    if (head_splits > 0 && !(head_env && head_env[0] == '0') && head_apply_supported(p, batch, head_splits)) {
+    // (option "head_apply" = 0: the general GEMM+AXPY kernels also for 128-row matrices -- A/B runs, tests)
+    if (head_splits > 0 && opt(OPT_HEAD_APPLY) != 0 && head_apply_supported(p, batch, head_splits)) {
       if (head_used) *head_used = true;
       return launch_head_apply(p, batch, head_splits, out_fp32 ? nullptr : head_gram_next, out_fp32 != 0, stream);
     }
@@ -1304,11 +1363,10 @@ static int small_chain(const uint16_t* X, int64_t batch, int64_t n, int splits, 
 static size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 // Tall input iterated as (m x n), m < n: does the last product write the float32 result transposed, straight into the
-// output?  (Not on the slab kernel of 128-row matrices.  MI_TALL_DIRECT=0, read by the workspace query and by the
-// call alike: staging copy and transposing pass for every tall input -- A/B runs, tests.)
+// output?  (Not on the slab kernel of 128-row matrices.  Option "tall_direct" = 0, read by the workspace query and by
+// the call alike: staging copy and transposing pass for every tall input -- A/B runs, tests.)
 static bool tall_writes_direct(int64_t m, int64_t n, int gram_splits) {
-  const char* env = getenv("MI_TALL_DIRECT");
-  return gemm_transposed_out_ok(m, n) && !(gram_splits > 0 && m == CH_M) && !(env && env[0] == '0');
+  return gemm_transposed_out_ok(m, n) && !(gram_splits > 0 && m == CH_M) && opt(OPT_TALL_DIRECT) != 0;
 }
 
 struct NsWorkspace {
@@ -1322,16 +1380,16 @@ struct NsWorkspace {
 // 2 = pairs, and the first three steps as one group.  A group of g steps trades g - 1 X X^T and g - 1 B X products
 // (3 m^2 n multiply-adds each time) for 4 (g - 1) products of m x m matrices, which pays for wide matrices only; on
 // a square matrix it would also sit close to the 1e-2 tolerance; below 1024 rows the kernels are launch-bound and a
-// group has more launches, except on the split-K Gram path.  MI_NS_PAIRS=0 switches grouping off, MI_NS_PAIRS=pairs
-// keeps the rule but never takes three steps at once, MI_NS_PAIRS=force pairs wherever the kernels allow it (used
-// by the tests to reach the pair kernels with small matrices).
+// group has more launches, except on the split-K Gram path.  Option "ns_pairs": 0 switches grouping off, 1 keeps the
+// rule but never takes three steps at once, 2 pairs wherever the kernels allow it (used by the tests to reach the
+// pair kernels with small matrices), -1 (default) the rule as described.
 static int ns_pairs_enabled(int64_t m, int64_t n, int gram_splits) {
-  const char* env = getenv("MI_NS_PAIRS");
-  if (env && env[0] == '0') return 0;
-  if (env && env[0] == 'f') return 1;
+  const int mode = opt(OPT_NS_PAIRS);
+  if (mode == 0) return 0;
+  if (mode == 2) return 1;
   // (the split-K Gram path serves short matrices at least four times as wide as tall: a group there trades passes
   // over X for tiny products at no more launches)
-  if (gram_splits > 0 || (m >= 1024 && n >= 2 * m)) return (env && env[0] == 'p') ? 1 : 2;
+  if (gram_splits > 0 || (m >= 1024 && n >= 2 * m)) return mode == 1 ? 1 : 2;
   return 0;
 }
 
@@ -1472,10 +1530,9 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
   float* xscale = reinterpret_cast<float*>(ws + w.xscale);
   int rc;
   // 128-row matrices whose first group goes through the chain kernel: the input pass also leaves the partial Gram
-  // matrices of its bf16 copy (MI_HEAD_FRONT=0: the general passes and a Gram kernel of its own).
-  const char* front_env = getenv("MI_HEAD_FRONT");
+  // matrices of its bf16 copy (option "head_front" = 0: the general passes and a Gram kernel of its own).
   const bool head_front = w.gram_splits > 0 && m == CH_M && !tall && !accumulate_fp64 && abc[2] != 0.0f &&
-                          w.gram_splits == n / 512 && w.gram_splits <= NORM_MAX_BLOCKS && !(front_env && front_env[0] == '0') &&
+                          w.gram_splits == n / 512 && w.gram_splits <= NORM_MAX_BLOCKS && opt(OPT_HEAD_FRONT) != 0 &&
                           head_front_supported(x, batch, n, mom);
   {
     ProfScope prof(PROF_NORMALIZE, stream);
@@ -1647,8 +1704,10 @@ int mi_syrk_bf16_ws(const void* A, int64_t batch, int64_t n, int64_t k, int64_t 
                     int64_t d_batch_stride, int64_t d_ld, int skip_upper, void* workspace, size_t workspace_bytes,
                     void* stream) {
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (a_trans && A && workspace && batch > 0 && n > 0 && k > 0 && n % 8 == 0 && k % 8 == 0 && a_ld % 8 == 0 &&
-      a_batch_stride % 8 == 0 && a_ld >= n && aligned16(A) && !(reinterpret_cast<uintptr_t>(workspace) & 255u)) {
+  // every argument is checked before the transposing copy below: an invalid call launches nothing
+  if (int rc = syrk_validate(A, batch, n, k, a_batch_stride, a_ld, a_trans, C, c_batch_stride, c_ld, beta, D, d_batch_stride, d_ld))
+    return rc;
+  if (a_trans && workspace && batch > 0 && n > 0 && k > 0 && !(reinterpret_cast<uintptr_t>(workspace) & 255u)) {
     const size_t copy = transposed_copy_bytes(n, batch, k);
     if (copy > 0 && workspace_bytes >= copy && n < (1 << 30) && k < (1 << 30) && batch <= 65535) {
       // the operand, K-contiguous, in the first part of the workspace; the rest serves the product itself
@@ -1774,6 +1833,23 @@ int mi_muon_update_bf16(float* param, const float* grad, float* momentum, int64_
   return ns_impl(grad, param, batch, rows, cols, abc, steps, eps, accumulate_fp64, update_scale, workspace,
                  workspace_bytes, static_cast<hipStream_t>(stream), MomentumSrc{momentum, beta, nesterov ? 1 : 0},
                  param_decay);
+}
+
+int mi_set_option(const char* name, int value) {
+  const int i = opt_index(name);
+  if (i < 0) return fail(MI_ERR_BAD_ARG, "mi_set_option: unknown option '%s'", name ? name : "(null)");
+  if (value < OPT_TABLE[i].lo || value > OPT_TABLE[i].hi)
+    return fail(MI_ERR_BAD_ARG, "mi_set_option: %s takes %d .. %d, got %d", name, OPT_TABLE[i].lo, OPT_TABLE[i].hi, value);
+  opt_init();
+  g_opt[i].store(value, std::memory_order_relaxed);
+  return MI_OK;
+}
+
+int mi_get_option(const char* name, int* value) {
+  const int i = opt_index(name);
+  if (i < 0 || !value) return fail(MI_ERR_BAD_ARG, "mi_get_option: unknown option '%s' or null output", name ? name : "(null)");
+  *value = opt(static_cast<Opt>(i));
+  return MI_OK;
 }
 
 int mi_debug_last_launch(int* tiles, int* tile_m, int* tile_n, int* fast) {

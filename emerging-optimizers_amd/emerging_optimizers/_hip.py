@@ -57,6 +57,8 @@ EXPORTS = (
     ("mi_profile_begin", _int, ()),
     ("mi_profile_end", _int, (_vp, _vp)),
     ("mi_debug_last_launch", _int, (_vp, _vp, _vp, _vp)),
+    ("mi_set_option", _int, (ctypes.c_char_p, _int)),
+    ("mi_get_option", _int, (ctypes.c_char_p, _vp)),
 )
 
 _lock = threading.Lock()
@@ -97,11 +99,37 @@ def lib() -> ctypes.CDLL:
     return _lib
 
 
+_gfx950: dict[int, bool] = {}
+
+
+def device_is_gfx950(device: torch.device) -> bool:
+    """Whether ``device`` is the part the kernels are compiled for (cached per device index)."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    hit = _gfx950.get(idx)
+    if hit is None:
+        arch = getattr(torch.cuda.get_device_properties(idx), "gcnArchName", "")
+        hit = _gfx950[idx] = arch.startswith("gfx950")
+    return hit
+
+
 def last_launch() -> dict:
     """Tile shape and workgroup count of the last product this thread launched (see ``mi_debug_last_launch``)."""
     vals = [ctypes.c_int(0) for _ in range(4)]
     check(lib().mi_debug_last_launch(*[ctypes.byref(v) for v in vals]))
     return dict(zip(("tiles", "tile_m", "tile_n", "fast"), (v.value for v in vals)))
+
+
+def set_option(name: str, value: int) -> int:
+    """Sets a process-wide option of the library (see ``mi_set_option``); returns the previous value."""
+    prev = get_option(name)
+    check(lib().mi_set_option(name.encode(), int(value)))
+    return prev
+
+
+def get_option(name: str) -> int:
+    out = ctypes.c_int(0)
+    check(lib().mi_get_option(name.encode(), ctypes.byref(out)))
+    return out.value
 
 
 def last_error() -> str:

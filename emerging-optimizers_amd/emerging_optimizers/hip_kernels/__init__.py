@@ -2,17 +2,16 @@
 
 from .. import _hip
 from .batched_syrk import batched_tsyrk_ex, can_use_batched_tsyrk
-from .newton_schulz import frob_normalize, fused_muon_update, fused_newton_schulz, fused_supported, gemm_axpy
+from .newton_schulz import (
+    frob_normalize,
+    fused_muon_update,
+    fused_newton_schulz,
+    fused_supported,
+    gemm_axpy,
+    on_kernel_device,
+    require_library,
+)
 from .syrk import tsyrk_ex, tsyrk_ex_small_matrix
-
-
-def _device_ready() -> bool:
-    import torch
-
-    if not _hip.available() or not torch.cuda.is_available():
-        return False
-    arch = getattr(torch.cuda.get_device_properties(0), "gcnArchName", "")
-    return arch.startswith("gfx950")
 
 
 #: True when libmi_ns.so is loadable.  The reference's call sites test ``HAS_TRITON_340`` before taking
@@ -30,6 +29,8 @@ __all__ = [
     "fused_newton_schulz",
     "fused_supported",
     "gemm_axpy",
+    "on_kernel_device",
+    "require_library",
     "tsyrk_ex",
     "tsyrk_ex_small_matrix",
 ]

@@ -11,7 +11,19 @@ from .. import _hip
 from . import _launch
 
 
-__all__ = ["gemm_axpy", "fused_newton_schulz", "fused_supported", "fused_muon_update"]
+__all__ = ["gemm_axpy", "fused_newton_schulz", "fused_supported", "fused_muon_update", "on_kernel_device", "require_library"]
+
+
+def require_library() -> None:
+    """Raises ``RuntimeError`` unless ``libmi_ns.so`` is loaded: GPU operands that the kernels serve never take
+    another path silently."""
+    _hip.lib()
+
+
+def on_kernel_device(t: torch.Tensor) -> bool:
+    """``t`` lives on a gfx950 GPU, the only part the kernels are compiled for.  Tensors on any other GPU stay on
+    torch's own operators, as the reference does for GPUs that its kernels do not support (muon.py:101-115)."""
+    return t.is_cuda and _hip.device_is_gfx950(t.device)
 
 
 def gemm_axpy(
@@ -63,16 +75,19 @@ def gemm_axpy(
 
 
 def fused_supported(x: torch.Tensor) -> bool:
-    """True when :func:`fused_newton_schulz` can take ``x``: GPU float32, 2-D/3-D, both dims multiples of 8."""
-    return (
-        _hip.available()
-        and x.is_cuda
+    """True when :func:`fused_newton_schulz` can take ``x``: GPU float32, 2-D/3-D, both dims multiples of 8.
+    Raises ``RuntimeError`` for such a tensor when ``libmi_ns.so`` is missing (no silent slow path on the GPU)."""
+    if not (
+        on_kernel_device(x)
         and x.dtype == torch.float32
         and x.dim() in (2, 3)
         and x.shape[-1] % 8 == 0
         and x.shape[-2] % 8 == 0
         and x.numel() > 0
-    )
+    ):
+        return False
+    require_library()
+    return True
 
 
 def frob_normalize(

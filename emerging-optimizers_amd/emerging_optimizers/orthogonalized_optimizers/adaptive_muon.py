@@ -9,7 +9,8 @@ Behaviour follows the reference's ``AdaptiveMuon`` (orthogonalized_optimizers/ad
   ``M`` the matrix handed to Newton-Schulz.
 
 ``O`` is the raw Newton-Schulz output; Muon's scale factor multiplies the normalised update afterwards.
-``use_syrk`` is an addition (the reference fixes False): True runs Newton-Schulz on the gfx950 kernels.
+``use_syrk`` is an addition (the reference fixes False); it is handed to ``newton_schulz``, which under matmul
+precision "medium" runs float32 matrices on a gfx950 GPU on the kernels for either value.
 """
 
 from __future__ import annotations
@@ -48,7 +49,7 @@ class AdaptiveMuon(OrthogonalizedOptimizer):
         moment2_method: "adamuon", "normuon" or "namo" (see the module docstring)
         beta2: EMA coefficient of the second moment
         eps: stabiliser of the division
-        use_syrk: use the SYRK kernels for the orthogonalisation
+        use_syrk: forwarded to ``newton_schulz``
     """
 
     def __init__(

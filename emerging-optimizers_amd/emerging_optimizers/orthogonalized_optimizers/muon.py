@@ -1,9 +1,14 @@
 """Muon (MomentUm Orthogonalized by Newton-schulz) on top of :class:`OrthogonalizedOptimizer`.
 
 Constructor arguments, defaults, read-only properties and the scale-factor rules follow the reference's
-``Muon`` (orthogonalized_optimizers/muon.py:37-216).  ``use_syrk=True`` routes the orthogonalisation
-through the gfx950 kernels; the reference whitelists NVIDIA SM versions at that point (muon.py:101-115),
-here the condition is "a gfx950 device and a loadable libmi_ns.so".
+``Muon`` (orthogonalized_optimizers/muon.py:37-216).
+
+A float32 parameter on a gfx950 GPU with both dims multiples of 8 is orthogonalised on the hand-written kernels
+under the default matmul precision "medium", whatever ``use_syrk`` says (see ``muon_utils.newton_schulz``): the
+reference's flag chooses between two library back ends for the same products, here the kernel library makes that
+choice itself.  ``use_syrk=True`` keeps its checks: the reference whitelists NVIDIA SM versions at that point
+(muon.py:101-115), here the condition is "a gfx950 device and a loadable libmi_ns.so", and a GPU without the
+library is an error rather than a downgrade.
 """
 
 from __future__ import annotations
@@ -82,7 +87,9 @@ class Muon(OrthogonalizedOptimizer[HookStateT]):
         num_ns_steps: number of Newton-Schulz iterations (at least 1).
         scale_mode: see :func:`get_muon_scale_factor`.
         extra_scale_factor: further multiplier of the update (0.2 roughly matches AdamW's update RMS).
-        use_syrk: run the iteration on the hand-written SYRK/GEMM kernels.
+        use_syrk: ask for the lower-triangle (SYRK) kernels explicitly; raises when a GPU is present but the kernel
+            library is not.  The default False gives the same results on a gfx950 GPU (the library chooses its
+            kernels by shape); the flag still selects the ``*_tsyrk`` step functions where steps run one by one.
         group_same_shape: one batched orthogonalisation per distinct parameter shape (see the base class).
     """
 
@@ -150,11 +157,11 @@ class Muon(OrthogonalizedOptimizer[HookStateT]):
     ) -> bool:
         """Whole update of one 2-D parameter in a single library call, when nothing needs the intermediates.
 
-        Taken for GPU float32 parameters with both dims multiples of 8 under ``use_syrk`` and matmul precision
-        "medium", with the library's own ``newton_schulz``, no subclass or weight-update hooks, and a weight
-        decay that only scales the parameter (every method except ``"l2"``, which modifies the gradient).
+        Taken for float32 parameters on a gfx950 GPU with both dims multiples of 8 under matmul precision "medium",
+        with the library's own ``newton_schulz``, no subclass or weight-update hooks, and a weight decay that only
+        scales the parameter (every method except ``"l2"``, which modifies the gradient).
         """
-        if not (FUSED_MUON_STEP and self._use_syrk and self.fp32_matmul_prec == "medium" and p.ndim == 2):
+        if not (FUSED_MUON_STEP and self.fp32_matmul_prec == "medium" and p.ndim == 2 and p.is_cuda):
             return False
         if self.scaled_orthogonalize_fn is not self._own_scaled_orthogonalize_fn or not self._update_is_plain():
             return False

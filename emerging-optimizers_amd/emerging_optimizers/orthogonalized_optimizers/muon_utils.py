@@ -4,14 +4,20 @@ Public surface and behaviour follow ``emerging_optimizers/orthogonalized_optimiz
 reference (function names, arguments, exception types/messages, the late-bound step functions), so callers
 and tests written against it run unchanged.  What differs is where the work goes:
 
-* float32 GPU input, matmul precision ``"medium"``, ``use_syrk=True``, both dims multiples of 8
-  -> one call into ``libmi_ns.so`` (normalise, bf16 cast, all steps, float32 result) -- the hot path.
-* the ``*_tsyrk`` step functions -> HIP SYRK + HIP GEMM/AXPY kernels, one product each.
-* everything else (CPU tensors, float32 arithmetic, shapes that are not multiples of 8) -> the same
-  torch operators the reference uses; these are not accelerated and not part of the hot path.
+* float32 GPU input, matmul precision ``"medium"``, both dims multiples of 8 -> one call into
+  ``libmi_ns.so`` (normalise, bf16 cast, all steps, float32 result) -- the hot path.  ``use_syrk`` does not
+  select it: in the reference that flag only picks between two library back ends for the same products
+  (its default ``False`` means cuBLAS GEMMs); here the library itself decides which of its kernels forms
+  a product, so both values of the flag give the same, bit-identical, result on such input.
+* the four step functions on bf16 GPU operands with both dims multiples of 8 -> HIP lower-triangle product +
+  HIP GEMM/AXPY kernels, one launch per product, with the reference's rounding points (every product
+  accumulated in float32 and rounded to bf16 once).
+* everything else (CPU tensors, float32 arithmetic under "highest"/"high", shapes that are not multiples
+  of 8) -> the same torch operators the reference uses; these are not accelerated and not part of the
+  hot path.
 
-GPU tensors never fall back silently: if the kernels are requested and ``libmi_ns.so`` is missing, the
-call raises.
+GPU tensors never fall back silently: where the kernels apply and ``libmi_ns.so`` is missing, the call
+raises.
 """
 
 from __future__ import annotations
@@ -155,7 +161,9 @@ def _normalize(x: torch.Tensor, eps: float, in_double: bool) -> torch.Tensor:
 
 
 def _fused_path_ok(x: torch.Tensor, transpose: bool, tp_group: Any) -> bool:
-    """The single-call kernel path applies when nothing asks for per-step Python control."""
+    """The single-call kernel path applies when nothing asks for per-step Python control.
+
+    Raises ``RuntimeError`` when the input qualifies but ``libmi_ns.so`` cannot be loaded."""
     if tp_group is not None or not hip_kernels.fused_supported(x):
         return False
     if transpose != (x.size(-2) > x.size(-1)):
@@ -187,9 +195,17 @@ def newton_schulz(
     Args mirror the reference (muon_utils.py:149-274): ``coefficient_type`` one of ``NSCoeffT`` (``"custom"``
     needs ``custom_coefficient_sets``; ``"cubic5"`` needs ``steps == 5``), ``eps`` guards the float32 norm,
     ``transpose`` overrides the orientation choice, ``tp_group`` marks ``x`` as sharded along the long
-    dimension, ``use_syrk`` selects the SYRK kernels (effective only under matmul precision ``"medium"``
-    and for dims that are multiples of 8), ``normalize_in_double`` reduces the norm in float64 so tiny
-    inputs do not underflow.  ``_out_scale`` (private) is folded into the last kernel's epilogue.
+    dimension, ``use_syrk`` selects the ``*_tsyrk`` step functions where the steps run one by one (effective
+    only under matmul precision ``"medium"`` and for dims that are multiples of 8), ``normalize_in_double``
+    reduces the norm in float64 so tiny inputs do not underflow.  ``_out_scale`` (private) is folded into the
+    last kernel's epilogue.
+
+    GPU input under ``"medium"`` with both dims multiples of 8 is orthogonalised by one library call whatever
+    ``use_syrk`` says: normalisation in one pass, steps on the diagonal-shifted rounding schedule (the stored
+    Gram matrix is ``A - (tr A / m) I``, so the bf16 rounding of its diagonal does not dominate the error),
+    consecutive steps of wide matrices on one shared Gram matrix, float32 result without a last bf16 rounding.
+    That schedule sits 3e-3 .. 7e-3 (relative Frobenius) from float32 Newton-Schulz where the reference's
+    bf16 schedule -- which the step functions keep -- sits around 1e-2.
 
     Returns a new float32 tensor shaped like ``x``.
     """
@@ -201,7 +217,7 @@ def newton_schulz(
         transpose = x.size(-2) > x.size(-1)
 
     medium = torch.get_float32_matmul_precision() == "medium"
-    if medium and use_syrk and x.is_cuda and _fused_path_ok(x, transpose, tp_group):
+    if medium and x.is_cuda and _fused_path_ok(x, transpose, tp_group):
         coeffs = _schedule(steps, coefficient_type, custom_coefficient_sets)
         _log_first_n(logging.INFO, "bf16", 1, "Using BF16 I/O kernels for Newton-Schulz iteration.")
         return hip_kernels.fused_newton_schulz(x, coeffs, eps, normalize_in_double, _out_scale)
@@ -278,12 +294,41 @@ def _allreduce_gram(A: torch.Tensor, tp_group: Any) -> None:
         torch.distributed.all_reduce(A, op=torch.distributed.ReduceOp.SUM, group=tp_group)
 
 
+def _kernels_take(X: torch.Tensor) -> bool:
+    """bf16 GPU operand of a step whose products the HIP kernels form: both dims multiples of 8 (16-byte rows),
+    stored row-major or as its transpose.  Raises when such an operand arrives and ``libmi_ns.so`` is missing."""
+    if not (hip_kernels.on_kernel_device(X) and X.dtype == torch.bfloat16 and X.numel() > 0):
+        return False
+    if X.size(-1) % 8 or X.size(-2) % 8 or not (X.is_contiguous() or X.mT.is_contiguous()):
+        return False
+    hip_kernels.require_library()
+    return True
+
+
+def _kernel_step(X: torch.Tensor, a: float, b: float, c: float, tp_group: Any) -> torch.Tensor:
+    """One iteration on the HIP kernels, 2-D or batched: ``A = X X^T`` and ``B = c A A^T + b A`` on the
+    lower-triangle kernel (``A`` is symmetric, so ``A A^T = A A``; the mirror image is written bit for bit), then
+    ``a X + B X`` as one GEMM with the AXPY in its epilogue.  Three launches, each product accumulated in float32
+    and rounded to bf16 once: the rounding points of ``X @ X.mT`` / ``addmm`` / ``baddbmm`` on bf16 operands."""
+    syrk = triton_kernels.batched_tsyrk_ex if X.ndim == 3 else triton_kernels.tsyrk_ex
+    A = syrk(X)
+    _allreduce_gram(A, tp_group)
+    if c == 0.0:
+        return hip_kernels.gemm_axpy(A, X, alpha=b, beta=a)
+    B = syrk(A, A, alpha=c, beta=b)
+    return hip_kernels.gemm_axpy(B, X, alpha=1.0, beta=a)
+
+
 def newton_schulz_step(X: torch.Tensor, a: float, b: float, c: float, tp_group: Any = None) -> torch.Tensor:
-    """One iteration on a 2-D ``X`` with library matmuls (any device/dtype): ``a X + (b A + c A A) X``.
+    """One iteration on a 2-D ``X``: ``a X + (b A + c A A) X`` (reference: muon_utils.py:348-378).
 
     ``c == 0`` takes the cubic form ``a X + b A X`` and skips the ``A A`` product.  With ``tp_group`` the Gram
-    matrix is summed over the group, i.e. ``X`` is a shard along the contraction dimension.
+    matrix is summed over the group, i.e. ``X`` is a shard along the contraction dimension.  bf16 GPU operands
+    with both dims multiples of 8 run on the HIP kernels (:func:`_kernel_step`); any other device, dtype or shape
+    on torch's matmuls, as in the reference.
     """
+    if _kernels_take(X):
+        return _kernel_step(X, a, b, c, tp_group)
     A = X @ X.mT
     _allreduce_gram(A, tp_group)
     if c == 0.0:
@@ -292,7 +337,10 @@ def newton_schulz_step(X: torch.Tensor, a: float, b: float, c: float, tp_group: 
 
 
 def batched_newton_schulz_step(X: torch.Tensor, a: float, b: float, c: float, tp_group: Any = None) -> torch.Tensor:
-    """:func:`newton_schulz_step` for ``(B, M, N)`` input, every batch entry iterated independently (``baddbmm``)."""
+    """:func:`newton_schulz_step` for ``(B, M, N)`` input, every batch entry iterated independently (reference:
+    muon_utils.py:381-411, ``baddbmm``); on the HIP kernels each product of the batch is one grouped launch."""
+    if _kernels_take(X):
+        return _kernel_step(X, a, b, c, tp_group)
     A = X @ X.mT
     _allreduce_gram(A, tp_group)
     if c == 0.0:
@@ -308,12 +356,7 @@ def newton_schulz_step_tsyrk(X: torch.Tensor, a: float, b: float, c: float, tp_g
     """One iteration on a 2-D bf16 ``X`` with the HIP kernels: two SYRKs (``X X^T`` and, ``A`` being symmetric,
     ``c A A^T + b A``) and one GEMM whose epilogue applies ``a X +``."""
     _require_kernels()
-    A = triton_kernels.tsyrk_ex(X)
-    _allreduce_gram(A, tp_group)
-    if c == 0.0:
-        return hip_kernels.gemm_axpy(A, X, alpha=b, beta=a)
-    B = triton_kernels.tsyrk_ex(A, A, alpha=c, beta=b)
-    return hip_kernels.gemm_axpy(B, X, alpha=1.0, beta=a)
+    return _kernel_step(X, a, b, c, tp_group)
 
 
 def batched_newton_schulz_step_tsyrk(
@@ -321,12 +364,7 @@ def batched_newton_schulz_step_tsyrk(
 ) -> torch.Tensor:
     """:func:`newton_schulz_step_tsyrk` for ``(B, M, N)`` bf16 input; each product is one grouped launch."""
     _require_kernels()
-    A = triton_kernels.batched_tsyrk_ex(X)
-    _allreduce_gram(A, tp_group)
-    if c == 0.0:
-        return hip_kernels.gemm_axpy(A, X, alpha=b, beta=a)
-    B = triton_kernels.batched_tsyrk_ex(A, A, alpha=c, beta=b)
-    return hip_kernels.gemm_axpy(B, X, alpha=1.0, beta=a)
+    return _kernel_step(X, a, b, c, tp_group)
 
 
 _ORIGINAL_STEP_FNS = {

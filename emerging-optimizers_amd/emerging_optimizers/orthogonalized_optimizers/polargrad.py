@@ -3,7 +3,8 @@
 Behaviour follows the reference's ``PolarGrad`` class (orthogonalized_optimizers/polargrad.py:33-118): the update
 is ``msign(G) * <msign(G), G> * extra_scale_factor``; the inner product equals the nuclear norm of ``G`` when the
 orthogonalisation is exact.  Default matmul precision is "highest", as in the reference; ``num_ns_steps = 0`` is
-allowed (the update is then ``G/||G|| * <G/||G||, G>``).  ``use_syrk`` is an addition (effective under "medium").
+allowed (the update is then ``G/||G|| * <G/||G||, G>``).  ``use_syrk`` is an addition, handed to ``newton_schulz``
+(the kernels run under "medium" only).
 The eigendecomposition-based one-sided variants of that file are not part of this package.
 """
 
@@ -31,7 +32,7 @@ class PolarGrad(OrthogonalizedOptimizer):
         coefficient_type: Newton-Schulz coefficient family
         num_ns_steps: Newton-Schulz iterations (0 skips the iteration, for exact-match tests)
         extra_scale_factor: extra multiplier of the update (0.2 roughly matches AdamW's update RMS, arXiv:2502.16982)
-        use_syrk: use the SYRK kernels for the orthogonalisation (not in the reference)
+        use_syrk: forwarded to ``newton_schulz`` (not in the reference)
     """
 
     def __init__(

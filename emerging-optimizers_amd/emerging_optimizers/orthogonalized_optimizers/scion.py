@@ -4,8 +4,8 @@ Constructor arguments and behaviour follow the reference's ``Scion``
 (orthogonalized_optimizers/scion.py:31-106): no Nesterov blend, and the Frank-Wolfe step is obtained from the
 base class by fixing decoupled weight decay at 1, so each step is
 ``p <- (1 - lr) p - lr * spectral_radius * sqrt(out / in) * msign(momentum)``.
-``use_syrk`` is an addition: the reference always takes its GEMM path here; True routes the orthogonalisation
-through the gfx950 kernels exactly as :class:`Muon` does.
+``use_syrk`` is an addition (the reference fixes False); it is handed to ``newton_schulz``, which under matmul
+precision "medium" runs float32 matrices on a gfx950 GPU on the kernels for either value.
 """
 
 from __future__ import annotations
@@ -38,7 +38,7 @@ class Scion(OrthogonalizedOptimizer):
         coefficient_type: Newton-Schulz coefficient family
         num_ns_steps: Newton-Schulz iterations (at least 1)
         spectral_radius: radius of the spectral-norm ball the LMO is scaled to
-        use_syrk: use the SYRK kernels for the orthogonalisation (not in the reference, which fixes False)
+        use_syrk: forwarded to ``newton_schulz`` (not in the reference, which fixes False)
     """
 
     def __init__(

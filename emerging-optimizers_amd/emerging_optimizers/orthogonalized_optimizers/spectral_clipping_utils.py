@@ -4,7 +4,8 @@ Same functions and arithmetic as the reference's ``spectral_clipping_utils``
 (orthogonalized_optimizers/spectral_clipping_utils.py:24-98), after
 https://leloykun.github.io/ponder/spectral-clipping/: ``clip(s, a, b) = ((a + b) + (a - s) sign(a - s)
 - (b - s) sign(b - s)) / 2`` lifted to singular values, with ``msign`` from 8 "polar_express" steps.
-``use_syrk`` is an addition: under matmul precision "medium" it sends the Newton-Schulz calls to the gfx950 kernels.
+``use_syrk`` is an addition (the reference fixes False); it is handed to ``newton_schulz``, which under matmul
+precision "medium" runs float32 matrices on a gfx950 GPU on the kernels for either value.
 """
 
 from __future__ import annotations

@@ -3,7 +3,8 @@
 Behaviour follows the reference's ``Spel`` (orthogonalized_optimizers/spel.py:31-129): the momentum is
 orthogonalised without any scale factor, the weight takes the usual step, and the updated weight is itself
 re-orthogonalised in place, ``x <- msign((1 - lr wd) x - lr msign(momentum))``.  Two Newton-Schulz calls per
-parameter and step.  ``use_syrk`` is an addition (the reference fixes False).
+parameter and step.  ``use_syrk`` is an addition (the reference fixes False); it is handed to ``newton_schulz``, which under matmul
+precision "medium" runs float32 matrices on a gfx950 GPU on the kernels for either value.
 """
 
 from __future__ import annotations
@@ -32,7 +33,7 @@ class Spel(OrthogonalizedOptimizer):
         {_args_doc}
         coefficient_type: Newton-Schulz coefficient family, used for both projections
         num_ns_steps: Newton-Schulz iterations of each projection (at least 1)
-        use_syrk: use the SYRK kernels for both projections (not in the reference, which fixes False)
+        use_syrk: forwarded to both ``newton_schulz`` calls (not in the reference, which fixes False)
     """
 
     def __init__(

@@ -81,10 +81,10 @@ int mi_syrk_bf16(const void* A, int64_t batch, int64_t n, int64_t k,
  * K loop: 4096 x 14336 transposed runs in 1.15x the time of the K-contiguous call instead of 1.6x.  Bit-identical to
  * the direct route on integer-valued inputs; on general inputs the tile size, hence the order of the float32
  * additions, may differ.
- * Environment: MI_STREAMK=0 never splits, MI_STREAMK=1 splits whenever the shape qualifies (n a multiple of 256,
+ * Options (mi_set_option): "streamk" = 0 never splits, 1 splits whenever the shape qualifies (n a multiple of 256,
  * n >= 1024, k a multiple of 64, A not transposed or copied, skip_upper == 0) and tiles are left over after the whole
- * rounds; MI_SYRK_TRANSPOSE=0 never copies a transposed operand, MI_SYRK_TRANSPOSE=1 always does (n >= 1024,
- * k a multiple of 64).
+ * rounds; "syrk_transpose" = 0 never copies a transposed operand, 1 always does (n >= 1024, k a multiple of 64).
+ * Every argument is checked before the first launch, the transposing copy included.
  */
 size_t mi_syrk_workspace_bytes(int64_t batch, int64_t n, int64_t k, int a_trans);
 int mi_syrk_bf16_ws(const void* A, int64_t batch, int64_t n, int64_t k,
@@ -158,9 +158,9 @@ size_t mi_frob_partials_len(int64_t batch, int64_t numel);
  *  - for matrices with at least 1024 rows and twice as many columns, consecutive quintic steps share one Gram
  *    matrix (all factors are polynomials of X X^T and commute): the first three when at least two more follow and
  *    (a_1 a_2)^2 <= 400, otherwise two at a time alternating with single steps, so 5 steps run as 3 + 2 or
- *    2 + 1 + 2; the same holds for 128/256-row matrices at least four times as wide.  The environment variable
- *    MI_NS_PAIRS, read at every call (and by mi_newton_schulz_workspace_bytes), overrides this: "0" = one step at a
- *    time, "pairs" = never three at once, "force" = pairs at every size.
+ *    2 + 1 + 2; the same holds for 128/256-row matrices at least four times as wide.  The option "ns_pairs"
+ *    (mi_set_option; read by the call and by mi_newton_schulz_workspace_bytes, so set it before both) overrides
+ *    this: 0 = one step at a time, 1 = never three at once, 2 = pairs at every size.
  */
 int mi_newton_schulz_bf16(const float* x, float* out, int64_t batch, int64_t rows, int64_t cols,
                           const float* abc, int steps, float eps, int accumulate_fp64,
@@ -225,6 +225,28 @@ int mi_muon_update_bf16(float* param, const float* grad, float* momentum, int64_
  */
 int mi_profile_begin(void);
 int mi_profile_end(float* ms_by_kind, int* launches_by_kind);
+
+/*
+ * Process-wide switches of kernel choice and step grouping, for A/B measurements and for tests that must reach a
+ * particular kernel variant (no counterpart in the reference, whose Triton autotuner is steered by the presence of
+ * absl.testing in sys.modules, triton_kernels/syrk.py:138-140).  An option is an integer; -1 means "decide by
+ * shape / cost model" where that exists.
+ *   "streamk"         -1 | 0 | 1   split-tail launch of mi_syrk_bf16_ws: by the model | never | whenever it applies
+ *   "syrk_transpose"  -1 | 0 | 1   transposing copy of a K-strided operand in mi_syrk_bf16_ws: likewise
+ *   "head_apply"       0 | 1       slab kernel for the B X product of 128-row matrices (default 1)
+ *   "head_front"       0 | 1       input pass of 128-row matrices that also leaves the Gram partials (default 1)
+ *   "tall_direct"      0 | 1       last product of a tall input writes the float32 result transposed (default 1)
+ *   "ns_pairs"        -1 | 0 | 1 | 2   steps sharing a Gram matrix: by shape | never | never three at once | pairs
+ *                                      at every size
+ * Initial values come from the environment variables MI_STREAMK, MI_SYRK_TRANSPOSE, MI_HEAD_APPLY, MI_HEAD_FRONT,
+ * MI_TALL_DIRECT, MI_NS_PAIRS (numbers as above; MI_NS_PAIRS also "pairs" = 1, "force" = 2), read once when the
+ * first option is looked up; no call reads the environment after that.  mi_set_option is atomic per option but not
+ * ordered against calls in flight on other host threads: "ns_pairs" and "tall_direct" change the workspace size,
+ * so set them before mi_newton_schulz_workspace_bytes and leave them alone until the call that uses that size
+ * has returned.  Unknown names and out-of-range values return MI_ERR_BAD_ARG.
+ */
+int mi_set_option(const char* name, int value);
+int mi_get_option(const char* name, int* value);
 
 /*
  * What the last product launched from this host thread used (for tests that must know which kernel variant served

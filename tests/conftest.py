@@ -25,6 +25,23 @@ def _seed():
     torch.set_float32_matmul_precision(prev)
 
 
+@pytest.fixture
+def mi_option():
+    """``mi_option(name, value)`` sets a process-wide option of libmi_ns.so for the rest of the test; every option
+    touched is put back afterwards."""
+    from emerging_optimizers import _hip
+
+    saved = {}
+
+    def set_option(name, value):
+        prev = _hip.set_option(name, value)
+        saved.setdefault(name, prev)
+
+    yield set_option
+    for name, value in saved.items():
+        _hip.set_option(name, value)
+
+
 @pytest.fixture(scope="session")
 def gpu():
     import torch

@@ -100,15 +100,12 @@ def test_python_validation_messages_cpu():
 
 
 @pytest.mark.parametrize("env", [None, "0", "pairs", "force"])
-def test_step_grouping_rule_matches_the_oracle_model(monkeypatch, env):
+def test_step_grouping_rule_matches_the_oracle_model(mi_option, env):
     """The host-side rule of the driver (which steps share a Gram matrix) against the oracle's restatement of it,
     over shapes on both sides of every threshold and every coefficient family."""
     from oracle import ns_oracle as O
 
-    if env is None:
-        monkeypatch.delenv("MI_NS_PAIRS", raising=False)
-    else:
-        monkeypatch.setenv("MI_NS_PAIRS", env)
+    mi_option("ns_pairs", {None: -1, "0": 0, "pairs": 1, "force": 2}[env])
     lib = _hip.lib()
     shapes = [(1, 4096, 14336), (1, 14336, 4096), (8, 4096, 14336), (1, 4096, 4096), (1, 4096, 8184), (1, 4096, 8192),
               (1, 1024, 2048), (1, 1016, 4096), (32, 128, 4096), (2, 256, 1536), (4, 128, 1000), (1, 384, 4096), (1, 8, 16)]
@@ -126,3 +123,51 @@ def test_step_grouping_rule_matches_the_oracle_model(monkeypatch, env):
             count = lib.mi_newton_schulz_schedule(batch, rows, cols, abc, steps, out, 16)
             assert list(out[:count]) == O.group_schedule(coeffs, mode), (env, batch, rows, cols, kind, steps)
     assert lib.mi_newton_schulz_schedule(1, 64, 64, None, 5, (ctypes.c_int * 4)(), 4) == _hip.MI_ERR_BAD_ARG
+
+
+def test_options_are_set_once_and_read_back(mi_option):
+    """mi_set_option / mi_get_option: ranges, unknown names, and that the step-grouping option steers both the
+    schedule query and the workspace size (two more m x m buffers where steps share a Gram matrix)."""
+    lib = _hip.lib()
+    assert _hip.get_option("ns_pairs") == -1 and _hip.get_option("streamk") == -1 and _hip.get_option("tall_direct") == 1
+    assert lib.mi_set_option(b"no_such_option", 1) == _hip.MI_ERR_BAD_ARG and "unknown option" in _hip.last_error()
+    assert lib.mi_set_option(b"ns_pairs", 3) == _hip.MI_ERR_BAD_ARG and "-1 .. 2" in _hip.last_error()
+    assert lib.mi_set_option(b"head_apply", -1) == _hip.MI_ERR_BAD_ARG
+    assert lib.mi_get_option(b"ns_pairs", None) == _hip.MI_ERR_BAD_ARG
+    assert _hip.get_option("ns_pairs") == -1  # a refused value changes nothing
+    grouped = lib.mi_newton_schulz_workspace_bytes(1, 4096, 14336)
+    mi_option("ns_pairs", 0)
+    assert _hip.get_option("ns_pairs") == 0
+    assert grouped - lib.mi_newton_schulz_workspace_bytes(1, 4096, 14336) == 2 * 4096 * 4096 * 2
+    # tall inputs whose last product writes the result transposed need no float32 staging copy
+    direct = lib.mi_newton_schulz_workspace_bytes(1, 14336, 4096)
+    mi_option("tall_direct", 0)
+    assert lib.mi_newton_schulz_workspace_bytes(1, 14336, 4096) - direct == 14336 * 4096 * 4
+
+
+def test_tall_input_beyond_the_fast_loaders_keeps_its_staging_copy():
+    """The direct-to-LDS loaders address a tile's rows with 32-bit byte offsets and leave leading dimensions of 4M
+    elements and more to the general kernel, which cannot write its result transposed: such a tall input must be given
+    the float32 staging copy by the workspace layout (it was once laid out without, and the refusal came after the first
+    kernel had run)."""
+    lib = _hip.lib()
+    rows, cols = (1 << 22) + 1024, 1024
+    wide = lib.mi_newton_schulz_workspace_bytes(1, cols, rows)
+    tall = lib.mi_newton_schulz_workspace_bytes(1, rows, cols)
+    assert tall - wide == rows * cols * 4
+    rows = (1 << 22) - 1024  # just inside: written directly, no staging copy
+    assert lib.mi_newton_schulz_workspace_bytes(1, rows, cols) == lib.mi_newton_schulz_workspace_bytes(1, cols, rows)
+
+
+def test_syrk_with_workspace_validates_before_it_copies():
+    """mi_syrk_bf16_ws refuses a bad call before its transposing copy of a K-strided operand (nothing is launched: this
+    runs without a GPU)."""
+    lib = _hip.lib()
+    buf = (ctypes.c_char * 8192)()
+    p = ctypes.cast((ctypes.addressof(buf) + 255) & ~255, ctypes.c_void_p)
+    args = lambda D, c_ld, beta, C: (p, 1, 2048, 4096, 2048 * 4096, 2048, 1, C, 2048 * 2048, c_ld, 1.0, beta, D, 2048 * 2048, 2048, 0,
+                                     p, 1 << 40, None)
+    assert lib.mi_syrk_bf16_ws(*args(None, 2048, 0.0, None)) == _hip.MI_ERR_BAD_ARG  # D missing
+    assert lib.mi_syrk_bf16_ws(*args(p, 2048, 0.5, None)) == _hip.MI_ERR_BAD_ARG     # beta without C
+    assert lib.mi_syrk_bf16_ws(*args(p, 2044, 0.5, p)) == _hip.MI_ERR_UNSUPPORTED_SHAPE  # c_ld not a multiple of 8
+    assert lib.mi_syrk_bf16_ws(*args(p, 1024, 0.5, p)) == _hip.MI_ERR_BAD_ARG        # c_ld too small

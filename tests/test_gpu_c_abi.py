@@ -196,11 +196,11 @@ SYRK_VARIANTS = [
 
 
 @pytest.mark.parametrize("n,k,trans,tile", SYRK_VARIANTS)
-def test_syrk_variants_integer_exact(gpu, monkeypatch, n, k, trans, tile):
+def test_syrk_variants_integer_exact(gpu, mi_option, n, k, trans, tile):
     """Both operand layouts on the direct-to-LDS kernels (a transposed operand has 128- and 256-row tiles and no
     variant for tiles that overhang the matrix: 1096 rows go to the general kernel there)."""
-    monkeypatch.setenv("MI_SYRK_TRANSPOSE", "0")  # the K-strided kernels themselves, not the transposing copy
-    monkeypatch.setenv("MI_STREAMK", "0")
+    mi_option("syrk_transpose", 0)  # the K-strided kernels themselves, not the transposing copy
+    mi_option("streamk", 0)
     a = _int_bf16((k, n) if trans else (n, k), -3, 3, gpu, seed=n + k)
     if trans:
         a = a.T
@@ -247,12 +247,12 @@ def test_syrk_lower_triangle_only(gpu, n, k, batch, trans):
 # ---------------------------------------------------------------- split-tail (stream-K) launch of the lower-triangle kernel
 @pytest.mark.parametrize("batch,n,k", [(16, 2048, 8192), (1, 1024, 8192), (3, 1280, 1024), (2, 1536, 4096), (5, 1024, 448),
                                        (30, 1024, 128), (26, 1024, 256)])
-def test_syrk_stream_k_integer_exact(gpu, monkeypatch, batch, n, k):
+def test_syrk_stream_k_integer_exact(gpu, mi_option, batch, n, k):
     """Whole rounds of 256 x 256 tiles, then the left-over tiles with their K range split between workgroups that
     park float32 accumulators in the workspace, then a launch that adds them and writes those tiles.  Small integers
     make every float32 sum exact, so the result must equal the ordinary launch bit for bit.  30 x 1024 x 128: 300
     tiles, 44 left over, 2 K tiles each (the split is capped by K); 26 x 1024 x 256: 260 tiles, 4 left over, 4 K tiles."""
-    monkeypatch.setenv("MI_STREAMK", "1")
+    mi_option("streamk", 1)
     a = _int_bf16((batch, n, k), -2, 3, gpu, seed=n + k)
     print(f"stream-K {batch}x{n}x{k}", flush=True)
     d = triton_kernels.batched_tsyrk_ex(a)
@@ -265,23 +265,23 @@ def test_syrk_stream_k_integer_exact(gpu, monkeypatch, batch, n, k):
     d2 = triton_kernels.batched_tsyrk_ex(a, s, alpha=0.25, beta=0.5)
     assert _hip.last_launch()["fast"] == 2
     assert torch.equal(d2, torch.baddbmm(s.float(), a.float(), a.float().mT, alpha=0.25, beta=0.5).to(BF))
-    monkeypatch.setenv("MI_STREAMK", "0")
+    mi_option("streamk", 0)
     d3 = triton_kernels.batched_tsyrk_ex(a)
     assert _hip.last_launch()["fast"] == 1 and torch.equal(d3, d)
     if batch * n <= 1280:
         assert np.array_equal(d[0].float().cpu().numpy(), O.syrk(a[0].float().cpu().numpy()))
 
 
-def test_syrk_stream_k_random_inputs_and_model_choice(gpu, monkeypatch):
+def test_syrk_stream_k_random_inputs_and_model_choice(gpu, mi_option):
     """Gaussian operands: the stream-K launch adds the same products in another order (float32), so it agrees with the
     ordinary launch to bf16 rounding of near-ties; which launch the cost model picks for the benchmark shapes."""
-    monkeypatch.delenv("MI_STREAMK", raising=False)
+    mi_option("streamk", -1)
     a = torch.randn(16, 2048, 8192, device=gpu, generator=torch.Generator(device=gpu).manual_seed(5)).to(BF)
     d = triton_kernels.batched_tsyrk_ex(a)
     chosen = _hip.last_launch()
     if torch.cuda.get_device_properties(0).multi_processor_count == 256:
         assert chosen["fast"] == 2, chosen  # 576 tiles of 256 x 256 = 2.25 rounds of 256 CUs
-    monkeypatch.setenv("MI_STREAMK", "0")
+    mi_option("streamk", 0)
     d0 = triton_kernels.batched_tsyrk_ex(a)
     assert _hip.last_launch()["fast"] == 1
     diff = (d.float() - d0.float()).abs()
@@ -290,7 +290,7 @@ def test_syrk_stream_k_random_inputs_and_model_choice(gpu, monkeypatch):
     assert float((diff > 0).float().mean()) < 0.02
     ref = a[3].float() @ a[3].float().T
     assert rel_fro_t(d[3].float(), ref) < 3e-3
-    monkeypatch.delenv("MI_STREAMK", raising=False)
+    mi_option("streamk", -1)
     x = torch.randn(4096, 14336, device=gpu).to(BF)
     triton_kernels.tsyrk_ex(x)
     assert _hip.last_launch()["fast"] == 1  # 253 tiles of 192 x 192: one round already
@@ -298,16 +298,16 @@ def test_syrk_stream_k_random_inputs_and_model_choice(gpu, monkeypatch):
 
 # ---------------------------------------------------------------- K-strided operand through a transposed copy
 @pytest.mark.parametrize("batch,n,k", [(1, 1024, 512), (2, 1096, 192), (1, 4096, 14336), (3, 1280, 4096), (16, 2048, 8192)])
-def test_syrk_transposed_copy_integer_exact(gpu, monkeypatch, batch, n, k):
+def test_syrk_transposed_copy_integer_exact(gpu, mi_option, batch, n, k):
     """A K-strided operand is first copied, transposed, into the workspace and then multiplied by the K-contiguous
     kernels (which have a 192 x 192 tile and the faster K loop).  Bit-equal to the K-strided kernels on small integers.
     4096 x 14336 is a shape where the model itself chooses the copy (elsewhere it is forced here); 16 x 2048 x 8192
     adds the split-tail launch behind it, both parts of the workspace in use."""
     forced = (n, k) != (4096, 14336)
     if forced:
-        monkeypatch.setenv("MI_SYRK_TRANSPOSE", "1")
+        mi_option("syrk_transpose", 1)
     else:
-        monkeypatch.delenv("MI_SYRK_TRANSPOSE", raising=False)
+        mi_option("syrk_transpose", -1)
     a = _int_bf16((batch, k, n), -2, 3, gpu, seed=n + k + 1).mT  # stored as k rows of n
     assert a.stride(-2) == 1
     print(f"transposed copy {batch}x{n}x{k}", flush=True)
@@ -324,6 +324,6 @@ def test_syrk_transposed_copy_integer_exact(gpu, monkeypatch, batch, n, k):
     s = s + s.mT
     d2 = triton_kernels.batched_tsyrk_ex(a, s, alpha=0.25, beta=0.5)
     assert torch.equal(d2, torch.baddbmm(s.float(), a.float(), a.float().mT, alpha=0.25, beta=0.5).to(BF))
-    monkeypatch.setenv("MI_SYRK_TRANSPOSE", "0")
+    mi_option("syrk_transpose", 0)
     assert torch.equal(triton_kernels.batched_tsyrk_ex(a), d)
     assert lib.mi_syrk_workspace_bytes(batch, n, k, 1) < batch * n * k * 2

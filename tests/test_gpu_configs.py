@@ -83,6 +83,39 @@ def test_muon_step_full_size_zero_and_warmed_buffer(gpu, shape):
     assert torch.isfinite(p).all()
 
 
+@pytest.mark.parametrize("shape", [(4096, 14336), (14336, 4096), (4096, 4096)])
+def test_default_muon_runs_on_the_kernels_full_size(gpu, monkeypatch, shape):
+    """`Muon(params)` with every argument at the reference's default (use_syrk=False, "quintic", no Nesterov, matmul
+    precision "medium"): each step is one fused library call, and the update is within 1e-2 of the same optimizer
+    run statement by statement in float32."""
+    from emerging_optimizers import hip_kernels
+
+    calls = []
+    real = hip_kernels.fused_muon_update
+    monkeypatch.setattr(hip_kernels, "fused_muon_update", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    w0 = torch.randn(shape, generator=torch.Generator().manual_seed(2)) * 0.02
+    p, q = nn.Parameter(w0.clone().to(gpu)), nn.Parameter(w0.clone().to(gpu))
+    fast = muon.Muon([p])
+    slow = muon.Muon([q], fp32_matmul_prec="highest")
+    assert not fast.use_syrk
+    lr, wd = fast.param_groups[0]["lr"], fast.param_groups[0]["weight_decay"]
+    for step in range(1, 3):
+        g = llama_grad(shape, seed=400 + step).to(gpu)
+        p.grad, q.grad = g.clone(), g.clone()
+        before_p, before_q = p.detach().clone(), q.detach().clone()
+        fast.step()
+        slow.step()
+        assert len(calls) == step
+        # (the parameter moves by lr = 3e-4 times an O(1) update: the difference of two float32 values of size 0.02
+        # carries their rounding, 1e-9 against an update of 3e-4 -- far below the tolerance)
+        upd_fast = p.detach() - before_p * (1 - lr * wd)
+        upd_slow = q.detach() - before_q * (1 - lr * wd)
+        err = float((upd_fast - upd_slow).norm() / upd_slow.norm())
+        print(f"\n  default Muon {shape} step {step}: update rel_fro vs float32 statements = {err:.3e}")
+        assert err <= TOL_FP32
+    torch.testing.assert_close(fast.state[p]["momentum_buffer"], slow.state[q]["momentum_buffer"], rtol=2e-6, atol=5e-9)
+
+
 def test_grouped_muon_step_against_the_oracle(gpu):
     """Same-shape parameters orthogonalised in one batched call (group_same_shape=True), on the kernels, against the
     numpy oracle's optimizer step with its float32 Newton-Schulz."""

@@ -26,22 +26,124 @@ def _np(t):
 
 
 # ---------------------------------------------------------------- step functions
+def _torch_step(x, a, b, c):
+    """The operator sequence of the reference's GEMM steps (muon_utils.py:370-377, 403-410 there), on torch's matmuls."""
+    A = x @ x.mT
+    add = torch.baddbmm if x.ndim == 3 else torch.addmm
+    if c == 0.0:
+        return add(x, A, x, alpha=b, beta=a)
+    return add(x, add(A, A, A, alpha=c, beta=b), x, alpha=1.0, beta=a)
+
+
+@pytest.fixture
+def kernel_calls(monkeypatch):
+    """Counts the products that reach the HIP kernels through the step functions."""
+    calls = {"syrk": 0, "gemm": 0}
+    real_gemm = hip_kernels.gemm_axpy
+    real = {"tsyrk_ex": muon_utils.triton_kernels.tsyrk_ex, "batched_tsyrk_ex": muon_utils.triton_kernels.batched_tsyrk_ex}
+
+    def counted(kind, fn):
+        def run(*args, **kw):
+            calls[kind] += 1
+            return fn(*args, **kw)
+
+        return run
+
+    monkeypatch.setattr(hip_kernels, "gemm_axpy", counted("gemm", real_gemm))
+    for name, fn in real.items():
+        monkeypatch.setattr(muon_utils.triton_kernels, name, counted("syrk", fn))
+    return calls
+
+
+# the integer cases of the reference's own step tests (tests/test_muon_utils.py:503-524 there)
 @pytest.mark.parametrize("shape", [(32, 32), (32, 64), (2, 32, 32), (4, 32, 64), (8, 16, 128)])
-def test_tsyrk_step_bit_equal_to_gemm_step_and_oracle(gpu, shape):
+def test_gemm_and_tsyrk_steps_bit_equal_to_torch_and_oracle(gpu, kernel_calls, shape):
     x = torch.randint(-2, 3, shape, device=gpu).to(BF)
     a, b, c = 2**-1, 2**-2, 2**-3
-    if len(shape) == 2:
-        got = muon_utils.newton_schulz_step_tsyrk(x, a, b, c)
-        ref = muon_utils.newton_schulz_step(x, a, b, c)
-    else:
-        got = muon_utils.batched_newton_schulz_step_tsyrk(x, a, b, c)
-        ref = muon_utils.batched_newton_schulz_step(x, a, b, c)
-        per = torch.stack([muon_utils.newton_schulz_step_tsyrk(x[i], a, b, c) for i in range(shape[0])])
-        assert torch.equal(got, per)
-    assert got.dtype == BF and torch.equal(got, ref)
+    batched = len(shape) == 3
+    tsyrk = muon_utils.batched_newton_schulz_step_tsyrk if batched else muon_utils.newton_schulz_step_tsyrk
+    gemm = muon_utils.batched_newton_schulz_step if batched else muon_utils.newton_schulz_step
+    got = tsyrk(x, a, b, c)
+    assert kernel_calls == {"syrk": 2, "gemm": 1}
+    via_gemm_step = gemm(x, a, b, c)
+    assert kernel_calls == {"syrk": 4, "gemm": 2}  # the GEMM step runs on the HIP kernels as well
+    assert got.dtype == BF and torch.equal(got, via_gemm_step)
+    assert torch.equal(got, _torch_step(x, a, b, c))  # hipBLASLt through torch: same rounding points, exact sums
     assert np.array_equal(_np(got), O.newton_schulz_step(_np(x), a, b, c, bf16=True))
-    cubic = (muon_utils.newton_schulz_step_tsyrk if len(shape) == 2 else muon_utils.batched_newton_schulz_step_tsyrk)(x, 2.0, -0.5, 0.0)
-    assert np.array_equal(_np(cubic), O.newton_schulz_step(_np(x), 2.0, -0.5, 0.0, bf16=True))
+    if batched:
+        per = torch.stack([muon_utils.newton_schulz_step(x[i], a, b, c) for i in range(shape[0])])
+        assert torch.equal(via_gemm_step, per)
+    for step in (tsyrk, gemm):  # cubic form: one lower-triangle product, one GEMM
+        cubic = step(x, 2.0, -0.5, 0.0)
+        assert np.array_equal(_np(cubic), O.newton_schulz_step(_np(x), 2.0, -0.5, 0.0, bf16=True))
+        assert torch.equal(cubic, _torch_step(x, 2.0, -0.5, 0.0))
+    # an operand stored transposed (what a tall parameter is after the `.mT` view of the driver)
+    xt = x.mT.contiguous().mT
+    assert not xt.is_contiguous() and torch.equal(gemm(xt, a, b, c), got)
+
+
+@pytest.mark.parametrize("shape", [(1024, 2048), (2, 1024, 1280), (256, 768), (4, 128, 1024), (2048, 1024)])
+def test_gemm_step_on_the_kernels_matches_torch_operators(gpu, kernel_calls, shape):
+    """Sizes that reach the direct-to-LDS kernels: random operands, so the float32 sums differ in order from
+    hipBLASLt's and a bf16 rounding flips here and there -- agreement to bf16 resolution, as the reference asks of its
+    own SYRK against cuBLAS (rtol 0.05 in tests/test_triton_kernels.py:138-204 there), and much tighter in norm."""
+    x = torch.randn(*shape, device=gpu)
+    x = (x / x.norm(dim=(-2, -1), keepdim=True)).to(BF)
+    if shape[-2] > shape[-1]:
+        x = x.mT  # the driver iterates on the wide orientation: the operand of the step is a transposed view
+    step = muon_utils.batched_newton_schulz_step if x.ndim == 3 else muon_utils.newton_schulz_step
+    a, b, c = 3.4445, -4.7750, 2.0315
+    got = step(x, a, b, c)
+    assert kernel_calls == {"syrk": 2, "gemm": 1}
+    ref = _torch_step(x.contiguous(), a, b, c)
+    assert got.shape == ref.shape and got.dtype == BF
+    assert rel_fro(got.float().cpu(), ref.float().cpu()) <= 3e-3
+    exact = _torch_step(x.float(), a, b, c)  # float32 arithmetic on the same bf16 operand
+    assert rel_fro(got.float().cpu(), exact.cpu()) <= 1.2 * rel_fro(ref.float().cpu(), exact.cpu()) + 1e-4
+
+
+def test_gemm_step_keeps_torch_for_what_the_kernels_do_not_take(gpu, kernel_calls):
+    """float32 operands, dims that are not multiples of 8 and CPU tensors stay on torch's matmuls (the reference's
+    path); nothing reaches the kernels."""
+    for x in (torch.randn(64, 128, device=gpu), torch.randn(12, 40, device=gpu).to(BF), torch.randn(2, 12, 40, device=gpu).to(BF),
+              torch.randn(16, 32).to(BF), torch.randn(64, 128, device=gpu).to(BF)[::2]):
+        step = muon_utils.batched_newton_schulz_step if x.ndim == 3 else muon_utils.newton_schulz_step
+        got = step(x, 0.5, 0.25, 0.125)
+        assert torch.equal(got, _torch_step(x, 0.5, 0.25, 0.125))
+    assert kernel_calls == {"syrk": 0, "gemm": 0}
+
+
+@pytest.mark.parametrize("shape", [(256, 512), (512, 256), (3, 128, 384), (1024, 2560), (4, 128, 1024)])
+def test_default_flags_take_the_single_call_driver(gpu, monkeypatch, shape):
+    """`newton_schulz(..., use_syrk=False)` -- the reference's default -- on GPU float32 input under "medium": the same
+    single library call as with use_syrk=True, bit for bit; and the per-step loop (forced here by replacing a step
+    function) reaches the kernels through the GEMM step functions."""
+    x = torch.randn(*shape, device=gpu)
+    calls = []
+    real = hip_kernels.fused_newton_schulz
+    monkeypatch.setattr(hip_kernels, "fused_newton_schulz", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    with utils.fp32_matmul_precision("medium"):
+        default = muon_utils.newton_schulz(x, steps=5)
+        syrk = muon_utils.newton_schulz(x, steps=5, use_syrk=True)
+    assert len(calls) == 2 and torch.equal(default, syrk)
+    assert rel_fro(default.cpu(), O.newton_schulz(x.cpu().numpy(), 5, "quintic")) <= TOL_FP32
+    # "highest": float32 arithmetic on torch, as in the reference
+    with utils.fp32_matmul_precision("highest"):
+        hi = muon_utils.newton_schulz(x, steps=5)
+    assert len(calls) == 2
+    assert rel_fro(hi.cpu(), O.newton_schulz(x.cpu().numpy(), 5, "quintic")) <= 1e-4
+
+
+def test_stepwise_loop_with_default_flags_runs_on_the_kernels(gpu, monkeypatch, kernel_calls):
+    x = torch.randn(256, 512, device=gpu)
+    original = muon_utils.newton_schulz_step
+    seen = []
+    monkeypatch.setattr(muon_utils, "newton_schulz_step", lambda X, a, b, c, tp_group=None: (seen.append(X.dtype), original(X, a, b, c, tp_group))[1])
+    with utils.fp32_matmul_precision("medium"):
+        out = muon_utils.newton_schulz(x, steps=5, coefficient_type="simple")
+    assert seen == [BF] * 5 and kernel_calls == {"syrk": 10, "gemm": 5}
+    want = O.newton_schulz(x.cpu().numpy(), 5, "simple", precision="medium")  # the reference's bf16 rounding schedule
+    assert rel_fro(out.cpu(), want) < 6e-3
 
 
 # ---------------------------------------------------------------- fused driver, small shapes vs the numpy oracle
@@ -69,10 +171,10 @@ def test_fused_matches_oracle(gpu, shape, kind, steps):
 
 
 @pytest.fixture
-def forced_pairs(monkeypatch):
+def forced_pairs(mi_option):
     """Makes the driver take steps two at a time on one Gram matrix wherever its kernels allow it (by itself it
     does so only for matrices with at least 1024 rows and twice as many columns)."""
-    monkeypatch.setenv("MI_NS_PAIRS", "force")
+    mi_option("ns_pairs", 2)
 
 
 # (1024, 2048) and (2, 1024, 2304) pair up by the driver's own rule (no override needed)
@@ -97,17 +199,17 @@ def test_paired_steps_match_oracle(gpu, forced_pairs, shape, kind, steps):
         assert rel_fro(model, single) > 1e-5
 
 
-def test_group_rule_by_shape(gpu, monkeypatch):
-    """Wide matrices take 5 quintic steps as 3 + 2 by default, as 2 + 1 + 2 under MI_NS_PAIRS=pairs, one at a time
-    under MI_NS_PAIRS=0; every variant stays within tolerance and follows its rounding model."""
+PAIRS_OPTION = {None: -1, "auto": -1, "0": 0, "pairs": 1, "force": 2}  # values of the library option "ns_pairs"
+
+
+def test_group_rule_by_shape(gpu, mi_option):
+    """Wide matrices take 5 quintic steps as 3 + 2 by default, as 2 + 1 + 2 with the option ns_pairs = 1, one at a time
+    with ns_pairs = 0; every variant stays within tolerance and follows its rounding model."""
     x = torch.randn(1024, 2560)
     want32 = O.newton_schulz(x.numpy(), 5, "quintic")
     outs = {}
     for env, mode in ((None, 2), ("pairs", 1), ("0", 0)):
-        if env is None:
-            monkeypatch.delenv("MI_NS_PAIRS", raising=False)
-        else:
-            monkeypatch.setenv("MI_NS_PAIRS", env)
+        mi_option("ns_pairs", PAIRS_OPTION[env])
         with utils.fp32_matmul_precision("medium"):
             outs[env] = muon_utils.newton_schulz(x.to(gpu), steps=5, coefficient_type="quintic", use_syrk=True).cpu()
         assert rel_fro(outs[env], want32) <= TOL_FP32
@@ -115,7 +217,7 @@ def test_group_rule_by_shape(gpu, monkeypatch):
     assert rel_fro(outs[None], O.newton_schulz_shifted_bf16(x.numpy(), 5, "quintic")) <= 6e-3  # the model's own rule
     assert not torch.equal(outs[None], outs["pairs"]) and not torch.equal(outs["pairs"], outs["0"])
     # polar_express opens with a large coefficient: no three steps at once there
-    monkeypatch.delenv("MI_NS_PAIRS", raising=False)
+    mi_option("ns_pairs", -1)
     with utils.fp32_matmul_precision("medium"):
         got = muon_utils.newton_schulz(x.to(gpu), steps=5, coefficient_type="polar_express", use_syrk=True).cpu()
     assert rel_fro(got, O.newton_schulz_shifted_bf16(x.numpy(), 5, "polar_express", pairs=1)) <= 6e-3
@@ -151,7 +253,7 @@ def _spectrum_cases():
 
 
 @pytest.mark.parametrize("kind", ["simple", "quintic", "aol", "polar_express"])
-def test_grouped_steps_are_as_accurate_as_single_steps(gpu, monkeypatch, kind):
+def test_grouped_steps_are_as_accurate_as_single_steps(gpu, mi_option, kind):
     """Ill-conditioned inputs are far from float32 under any bf16 schedule (the reference's included); what must
     hold is that taking steps in groups (the driver's own rule: 3 + 2 or 2 + 1 + 2; pairs only) does not add to
     that."""
@@ -159,7 +261,7 @@ def test_grouped_steps_are_as_accurate_as_single_steps(gpu, monkeypatch, kind):
         want32 = O.newton_schulz(x.numpy(), 5, kind, compute_dtype=np.float64)
         err = {}
         for env in ("auto", "pairs", "0"):
-            monkeypatch.setenv("MI_NS_PAIRS", env)
+            mi_option("ns_pairs", PAIRS_OPTION[env])
             with utils.fp32_matmul_precision("medium"):
                 got = muon_utils.newton_schulz(x.to(gpu), steps=5, coefficient_type=kind, use_syrk=True).cpu()
             err[env] = rel_fro(got, want32)
@@ -468,9 +570,9 @@ def test_muon_step_keeps_the_statement_path_when_something_watches_the_update(gp
 
 @pytest.mark.parametrize("shape", [(32, 128, 4096), (3, 128, 1024), (1, 128, 2048), (5, 4096, 128)])
 @pytest.mark.parametrize("coefficient_type", ["simple", "quintic", "polar_express"])
-def test_per_head_slab_kernel_against_the_general_kernels(gpu, monkeypatch, shape, coefficient_type):
+def test_per_head_slab_kernel_against_the_general_kernels(gpu, mi_option, shape, coefficient_type):
     """128-row matrices: the product that ends a group of steps, and the partial Gram matrices of its result, come from
-    the slab kernel (inst_head_apply.hip).  MI_HEAD_APPLY=0 sends the same call through the general GEMM+AXPY kernel
+    the slab kernel (inst_head_apply.hip).  The option head_apply = 0 sends the same call through the general GEMM+AXPY kernel
     and a separate Gram kernel.  The two differ in how the sum of squares behind the diagonal shift is split into
     partial sums (one per 512-column slice against one per 256-column tile), i.e. in the last bits of the shift, which
     moves a few bf16 roundings: measured 0 to 6e-5 apart for the "simple" and "quintic" coefficients and up to 2.7e-3
@@ -478,10 +580,10 @@ def test_per_head_slab_kernel_against_the_general_kernels(gpu, monkeypatch, shap
     float32, not bit for bit.  A batch entry equals the matrix computed alone, bit for bit."""
     x = torch.randn(*shape, device=gpu, generator=torch.Generator(device=gpu).manual_seed(21)) * 3e-3
     with utils.fp32_matmul_precision("medium"):
-        monkeypatch.delenv("MI_HEAD_APPLY", raising=False)
+        mi_option("head_apply", 1)
         new = muon_utils.newton_schulz(x, steps=5, coefficient_type=coefficient_type, use_syrk=True)
         alone = muon_utils.newton_schulz(x[-1], steps=5, coefficient_type=coefficient_type, use_syrk=True)
-        monkeypatch.setenv("MI_HEAD_APPLY", "0")
+        mi_option("head_apply", 0)
         old = muon_utils.newton_schulz(x, steps=5, coefficient_type=coefficient_type, use_syrk=True)
     assert torch.isfinite(new).all()
     diff = rel_fro(new, old)
@@ -492,9 +594,9 @@ def test_per_head_slab_kernel_against_the_general_kernels(gpu, monkeypatch, shap
 
 @pytest.mark.parametrize("shape", [(32, 128, 4096), (3, 128, 1024), (1, 128, 2048)])
 @pytest.mark.parametrize("magnitude", [3e-3, 1e-17, 1e15])
-def test_per_head_input_pass_against_the_general_passes(gpu, monkeypatch, shape, magnitude):
+def test_per_head_input_pass_against_the_general_passes(gpu, mi_option, shape, magnitude):
     """128-row matrices: the pass over the float32 input also leaves the partial Gram matrices of its bf16 copy
-    (head_front_kernel in inst_head_apply.hip).  MI_HEAD_FRONT=0 sends the same call through the general sum-of-squares
+    (head_front_kernel in inst_head_apply.hip).  The option head_front = 0 sends the same call through the general sum-of-squares
     pass and a Gram kernel of its own.  The two add the squares in a different order, so the norm may differ in its last
     bit, which moves a few bf16 roundings: the results agree to 2e-4 and either is as far from float32 as the other.
     The magnitudes 1e-17 and 1e15 put the norm outside the range where the divide by it may be left to the consumers:
@@ -502,10 +604,10 @@ def test_per_head_input_pass_against_the_general_passes(gpu, monkeypatch, shape,
     equals the matrix computed alone, bit for bit."""
     x = torch.randn(*shape, device=gpu, generator=torch.Generator(device=gpu).manual_seed(33)) * magnitude
     with utils.fp32_matmul_precision("medium"):
-        monkeypatch.delenv("MI_HEAD_FRONT", raising=False)
+        mi_option("head_front", 1)
         new = muon_utils.newton_schulz(x, steps=5, coefficient_type="simple", use_syrk=True)
         alone = muon_utils.newton_schulz(x[-1], steps=5, coefficient_type="simple", use_syrk=True)
-        monkeypatch.setenv("MI_HEAD_FRONT", "0")
+        mi_option("head_front", 0)
         old = muon_utils.newton_schulz(x, steps=5, coefficient_type="simple", use_syrk=True)
     assert torch.isfinite(new).all()
     diff = rel_fro(new, old)
@@ -518,10 +620,10 @@ def test_per_head_input_pass_against_the_general_passes(gpu, monkeypatch, shape,
 
 
 @pytest.mark.parametrize("nesterov", [True, False])
-def test_per_head_input_pass_with_a_momentum_source(gpu, monkeypatch, nesterov):
+def test_per_head_input_pass_with_a_momentum_source(gpu, mi_option, nesterov):
     """The fused optimizer update on 128-row matrices: the input pass that leaves the Gram partials also updates the
     momentum buffer and orthogonalises the direction it defines.  Against the same call through the general passes
-    (MI_HEAD_FRONT=0): the buffer bit for bit (the same elementwise formula), the parameter to rounding noise."""
+    (option head_front = 0): the buffer bit for bit (the same elementwise formula), the parameter to rounding noise."""
     shape, lr, beta, wd = (8, 128, 2048), 0.02, 0.95, 0.1
     gen = torch.Generator().manual_seed(11)
     p0 = (torch.randn(shape, generator=gen) * 0.02).to(gpu)
@@ -529,7 +631,7 @@ def test_per_head_input_pass_with_a_momentum_source(gpu, monkeypatch, nesterov):
     g = (torch.randn(shape, generator=gen) * 1e-2).to(gpu)
     res = {}
     for front in ("1", "0"):
-        monkeypatch.setenv("MI_HEAD_FRONT", front)
+        mi_option("head_front", int(front))
         p, buf = p0.clone(), buf0.clone()
         hip_kernels.fused_muon_update(p, g, buf, SIMPLE5, beta=beta, nesterov=nesterov, param_decay=1 - wd * lr, update_scale=-lr)
         res[front] = (p, buf)
@@ -542,9 +644,9 @@ def test_per_head_input_pass_with_a_momentum_source(gpu, monkeypatch, nesterov):
 
 
 @pytest.mark.parametrize("shape", [(3584, 1024), (2048, 1024), (512, 256), (2, 2304, 1024), (8, 4096, 1792), (14336, 4096)])
-def test_tall_input_result_written_transposed_by_the_last_product(gpu, monkeypatch, shape):
+def test_tall_input_result_written_transposed_by_the_last_product(gpu, mi_option, shape):
     """Tall inputs are iterated in the transposed orientation.  Where the last product runs on kernels with the staged
-    epilogue, it writes its float32 result transposed, straight into the output; MI_TALL_DIRECT=0 restores the
+    epilogue, it writes its float32 result transposed, straight into the output; the option tall_direct = 0 restores the
     float32 staging copy and the transposing pass.  Same arithmetic, so the two agree bit for bit -- also for the
     fused optimizer update, where the epilogue reads the parameter it updates in the transposed pattern."""
     gen = torch.Generator(device=gpu).manual_seed(9)
@@ -553,7 +655,7 @@ def test_tall_input_result_written_transposed_by_the_last_product(gpu, monkeypat
     buf0 = torch.randn(*shape, device=gpu, generator=gen) * 1e-3
     res = {}
     for direct in ("1", "0"):
-        monkeypatch.setenv("MI_TALL_DIRECT", direct)
+        mi_option("tall_direct", int(direct))
         with utils.fp32_matmul_precision("medium"):
             out = muon_utils.newton_schulz(x, steps=5, coefficient_type="simple", use_syrk=True)
         p, buf = p0.clone(), buf0.clone()

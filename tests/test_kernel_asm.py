@@ -9,6 +9,10 @@ inside the loop; the result is then wrong in a few elements only.  This test com
 rejects, for every fast kernel,
   * any ``v_accvgpr_*`` move or AGPR spill inside an innermost loop that contains MFMAs,
   * any such instruction between an MFMA and the drain that follows it.
+A second check counts loads.  The lower-triangle kernels of 128- and 192-row tiles request their first addend with
+ordinary loads between the prologue and the K loop, and the wait at the end of K tile 0 leaves exactly that many more
+loads in flight; were the compiler to merge, drop or move some of them, that wait would let a load of K tile 1 slip.
+The test reads the number of those loads and the wait's immediate off the compiled code of every such kernel.
 No GPU is involved.
 """
 import os
@@ -125,12 +129,15 @@ def test_detector_flags_swaps_and_spills():
     assert accumulator_hazards(clean) == []  # a151 is no accumulator here: a value the compiler parked in a free AGPR
 
 
-@pytest.mark.skipif(shutil.which("hipcc") is None, reason="hipcc not available")
-def test_no_accumulator_traffic_next_to_mfma(tmp_path):
-    # the Makefile's own flags, one assembly file per translation unit
-    subprocess.run(["make", "-j8", "-C", CSRC, "asm", f"ASMDIR={tmp_path}"], check=True, capture_output=True, timeout=900)
+@pytest.fixture(scope="module")
+def compiled_kernels(tmp_path_factory):
+    """name -> assembly lines of every kernel of the library, compiled with the Makefile's own flags."""
+    if shutil.which("hipcc") is None:
+        pytest.skip("hipcc not available")
+    out = tmp_path_factory.mktemp("asm")
+    subprocess.run(["make", "-j8", "-C", CSRC, "asm", f"ASMDIR={out}"], check=True, capture_output=True, timeout=900)
     kernels, name = {}, None
-    for asm in sorted(tmp_path.glob("*.s")):
+    for asm in sorted(out.glob("*.s")):
         for line in asm.read_text().splitlines():
             m = re.match(r"^(_ZN2mi\S+):\s", line)
             if m:
@@ -140,10 +147,50 @@ def test_no_accumulator_traffic_next_to_mfma(tmp_path):
                 kernels[name].append(line)
                 if line.startswith(".Lfunc_end"):  # (not the first s_endpgm: a kernel may return early)
                     name = None
-    fast = {n: ls for n, ls in kernels.items() if "gemm_fast_kernel" in n or "small_chain_kernel" in n}
+    return kernels
+
+
+def test_no_accumulator_traffic_next_to_mfma(compiled_kernels):
+    fast = {n: ls for n, ls in compiled_kernels.items() if "gemm_fast_kernel" in n or "small_chain_kernel" in n}
     # (the finishing kernel of a split-tail launch, split-tail role 2, has an epilogue and no K loop)
     no_mfma = [n for n, ls in fast.items() if not any("v_mfma" in x for x in ls)]
     assert len(fast) >= 20 and all(n.endswith("ELi2ELb0EEEvNS_10GemmParamsE") for n in no_mfma) and len(no_mfma) <= 1, no_mfma
     report = {n: accumulator_hazards(ls) for n, ls in fast.items()}
     report = {n: b for n, b in report.items() if b}
     assert not report, "\n".join(f"{n}: {len(b)} hazards, e.g. {b[0]}" for n, b in report.items())
+
+
+# gemm_fast_kernel<FastCfg<TILE_M, WGM, WGN, BK, NS, TILE_N>, P_KS, Q_KS, MODE, OUT_F32, EDGE, STREAMK, RMW>
+FAST_NAME = re.compile(r"gemm_fast_kernelINS_7FastCfgILi(\d+)ELi(\d+)ELi(\d+)ELi(\d+)ELi(\d+)ELi(\d+)EEE"
+                       r"Lb([01])ELb([01])ELi(\d)ELb([01])ELb([01])ELi(\d)ELb([01])E")
+
+
+def early_addend_loads(lines):
+    """(8-byte global loads in front of the first MFMA, immediates of the vmcnt waits of the kernel)."""
+    text = [t for _, t in instructions(lines)]
+    first_mfma = next(k for k, t in enumerate(text) if t.startswith("v_mfma"))
+    loads = sum(1 for t in text[:first_mfma] if re.match(r"global_load_dwordx2\s", t))
+    wider = sum(1 for t in text[:first_mfma] if re.match(r"global_load_dwordx[34]\s", t))
+    waits = {int(m.group(1)) for t in text for m in [re.match(r"s_waitcnt vmcnt\((\d+)\)", t)] if m}
+    return loads, wider, waits
+
+
+def test_first_addend_is_requested_with_the_counted_number_of_loads(compiled_kernels):
+    """SyrkStage::NQUAD loads of 8 bytes per lane, none merged into wider ones, and the wait at the end of K tile 0 that
+    leaves (NS - 2) * LOADS_PER_TILE + NQUAD loads in flight (k_tile's EXTRA in gemm_fast.hpp)."""
+    seen = 0
+    for name, lines in compiled_kernels.items():
+        m = FAST_NAME.search(name)
+        if not m:
+            continue
+        tile_m, wgm, wgn, bk, ns, tile_n, p_ks, q_ks, mode, out_f32, edge, streamk, rmw = map(int, m.groups())
+        nquad = (tile_m // wgm // 16) * (tile_n // wgn // 16)
+        # the variants that hold the first addend in registers across the K loop (SyrkStage::CIN_EARLY), K loop included
+        if mode != 0 or out_f32 or wgm * wgn != 4 or 2 * nquad > 80 or streamk == 2:
+            continue
+        loads_per_tile = (tile_m + tile_n) * bk * 2 // 1024 // (wgm * wgn)
+        loads, wider, waits = early_addend_loads(lines)
+        assert (loads, wider) == (nquad, 0), (name, loads, wider, nquad)
+        assert (ns - 2) * loads_per_tile + nquad in waits, (name, sorted(waits))
+        seen += 1
+    assert seen >= 6  # 128 x 128 (two ring depths) and 192 x 192 tiles, whole and edge variants, both operand layouts

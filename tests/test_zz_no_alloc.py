@@ -32,11 +32,20 @@ def _both(x, steps=5, out_scale=1.0):
     want = torch.full_like(x, float("nan"))
     _hip.check(lib.mi_newton_schulz_bf16(_vp(x), _vp(want), batch, rows, cols, abc, steps, 1e-15, 0, out_scale, _vp(ws), nbytes, stream))
     got = torch.full_like(x, float("nan"))
-    before = torch.cuda.memory_allocated(x.device)
+    # A first call looks up the buffer's address (once per device) and makes the runtime load the code of the kernels
+    # this shape uses; the call that is measured comes after it.  Free device memory as the driver reports it
+    # (hipMemGetInfo) sees every allocation of the process, torch's own and any the library might make.
+    _hip.check(lib.mi_newton_schulz_bf16_noalloc(_vp(x), _vp(got), batch, rows, cols, abc, steps, 1e-15, 0, out_scale, stream))
+    torch.cuda.synchronize()
+    got.fill_(float("nan"))
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info(x.device)[0]
+    torch_before = torch.cuda.memory_allocated(x.device)
     rc = lib.mi_newton_schulz_bf16_noalloc(_vp(x), _vp(got), batch, rows, cols, abc, steps, 1e-15, 0, out_scale, stream)
     _hip.check(rc)
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated(x.device) == before
+    assert torch.cuda.mem_get_info(x.device)[0] == free_before
+    assert torch.cuda.memory_allocated(x.device) == torch_before
     return got, want
 
 
