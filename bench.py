@@ -16,7 +16,14 @@ one such orthogonalisation.  The run prints ONE JSON line:
                X X^T and every m x m product): algorithmic (symmetric-halved) FLOP per launch over its average launch
                duration, taken from HIP events the library records on the launch stream; `frac_executed` prices the
                MFMA work the launches really issue (whole tiles, idle quarter of diagonal tiles left out)
-  cpu_baseline the same operator sequence in float32 torch on the host cores (a baseline, not a target)
+  cpu_baseline the same operator sequence in float32 torch on the host cores (a baseline, not a target); timed first,
+               so that the GPU work ends the run
+Stated baselines beside the kernels (never targets), timed in the same process with the same warm-up and iteration
+counts: every Newton-Schulz row carries `torch_bf16_path_ms`, the reference's own operator sequence with
+use_syrk=False (normalise, bf16 cast, X @ X.mT / addmm / addmm per step, float32 cast) on torch's GPU operators --
+what the reference executes on this GPU, whose SYRK gate admits NVIDIA parts only; every SYRK row carries
+`torch_bmm_ms` (and `torch_baddbmm_ms` for its beta variant) and `loop_single_ms`, a Python loop of single-matrix
+calls, as the reference's SYRK benchmark times them (benchmarks/bench_batched_syrk.py:71-96 there).
 A parity gate that fails (relative Frobenius error against float32 above 1e-2, or a SYRK result that is not bitwise
 symmetric) is reported in the line and makes the process exit with status 1.  This build runs on one GPU; --gpus
 above 1 is refused.
@@ -42,6 +49,8 @@ TOL = 1e-2
 # (2 x X X^T, 14 m x m products), and of one GEMM+AXPY (both launches): FETCH_SIZE and WRITE_SIZE of two
 # `rocprofv3 --pmc` runs of this file (KiB per dispatch), each scaled by what the same counter reads for sumsq_kernel
 # of the same run, whose traffic is known (229 376 KiB read, 114 696 KiB written): factors 1.9994 and 0.9998.
+TRAFFIC_SOURCE = ("profiles/newton_schulz_4096x14336_pmc.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command; a constant "
+                  "from that profile, not measured in this run; null when tile choice or schedule differ from the profiled ones)")
 TRI_KERNEL_TRAFFIC_BYTES = int((129117.8 * 1.9994 + 32768.0 * 0.9998) * 1024)
 GEMM_AXPY_TRAFFIC_BYTES = int(((407572.7 + 146821.6) * 1.9994 + (98328.0 + 16392.0) * 0.9998) * 1024)
 M, N, NS_STEPS = 4096, 14336, 5
@@ -75,8 +84,9 @@ STEP_WORKLOADS = {
     "muon_step": (4096, 14336),      # whole Muon.step() (momentum 0.95, Nesterov, weight decay) on the headline gradient
     "muon_step_attn": (4096, 4096),
     "muon_heads": (32, 128, 4096),   # Muon.step() over 32 separate 128 x 4096 parameters, one batched orthogonalisation
+    "muon_step_default": (4096, 14336),  # Muon(params) with every argument at the reference's default (use_syrk=False, "quintic")
 }
-DEFAULT_OTHERS = ["attn", "batched_syrk", "per_head", "moe_shard", "moe", "muon_step", "muon_step_attn", "mlp_tall",
+DEFAULT_OTHERS = ["attn", "batched_syrk", "per_head", "moe_shard", "moe", "muon_step", "muon_step_default", "muon_step_attn", "mlp_tall",
                   "syrk_8x2048x2048", "syrk_4x4096x4096", "syrk_32x512x2048", "syrk_64x256x1024", "syrk_4096x14336",
                   "syrk_4096x14336_trans", "muon_heads"]
 ALL_WORKLOADS = list(NS_WORKLOADS) + list(SYRK_WORKLOADS) + list(STEP_WORKLOADS)
@@ -130,6 +140,22 @@ def ns_fp32_reference(x):
         torch.set_float32_matmul_precision(prev)
 
 
+def ns_torch_bf16_path(x, coeffs):
+    """The reference's operator sequence under "medium" with use_syrk=False (muon_utils.py:212-273, 370-377, 403-410
+    there) on torch's own GPU operators: a stated baseline, what the reference would execute on this GPU."""
+    import torch
+
+    tall = x.shape[-2] > x.shape[-1]
+    X = x.mT if tall else x
+    X = torch.nn.functional.normalize(X, p=2, dim=(-2, -1), eps=1e-15).to(torch.bfloat16)
+    add = torch.baddbmm if X.dim() == 3 else torch.addmm
+    for a, b, c in coeffs:
+        A = X @ X.mT
+        X = add(X, add(A, A, A, alpha=c, beta=b), X, alpha=1.0, beta=a)
+    X = X.to(torch.float32)
+    return X.mT if tall else X
+
+
 def schedule_of(lib, batch, rows, cols):
     abc = (ctypes.c_float * (3 * NS_STEPS))(*[v for c in COEFFS for v in c])
     out = (ctypes.c_int * 16)()
@@ -177,14 +203,26 @@ def run_ns_workload(name, warmup, iters, lib, dev, zeros=False):
     m, n = sorted(shape[-2:])
     schedule = schedule_of(lib, batch, shape[-2], shape[-1])
     f_sym, f_full, f_exec = ns_flops(batch, m, n, schedule)
+    # stated baseline: the reference's own bf16 operator sequence on torch's operators, same counts
+    torch_ms = torch_rel = None
+    if not zeros:
+        with torch.no_grad():
+            _, tper = time_events(lambda: ns_torch_bf16_path(x, COEFFS), warmup, iters)
+            tout = ns_torch_bf16_path(x, COEFFS)
+        torch_ms = statistics.median(tper)
     # parity: every matrix of a batch (two of them for the 1.9 GB stack)
     idx = range(batch) if x.dim() == 3 and x.numel() <= (1 << 28) else (range(2) if x.dim() == 3 else [None])
     rels = [0.0] if zeros else []
+    trels = []
     for i in ([] if zeros else idx):
-        xi, oi = (x, out) if i is None else (x[i], out[i])
+        xi, oi, ti = (x, out, tout) if i is None else (x[i], out[i], tout[i])
         ref = ns_fp32_reference(xi)
         rels.append(float((oi.double() - ref.double()).norm() / ref.double().norm()))
+        trels.append(float((ti.double() - ref.double()).norm() / ref.double().norm()))
         del ref
+    if not zeros:
+        torch_rel = max(trels)
+        del tout
     med, mn = statistics.median(per), min(per)
     res = {
         "workload": f"newton_schulz {NS_STEPS} steps on {'x'.join(map(str, shape))} float32 ({name})",
@@ -194,6 +232,9 @@ def run_ns_workload(name, warmup, iters, lib, dev, zeros=False):
         "schedule": "+".join(map(str, schedule)),
         "pct_peak_executed": round(100 * f_exec / med / 1e9 / PEAK_BF16_TFLOPS, 2),
         "rel_fro": round(max(rels), 6), "parity": "ok" if max(rels) <= TOL else "FAILED",
+        "torch_bf16_path_ms": round(torch_ms, 4) if torch_ms else None,
+        "speedup_vs_torch": round(torch_ms / med, 2) if torch_ms else None,
+        "torch_bf16_path_rel_fro": round(torch_rel, 6) if torch_rel is not None else None,
     }
     if name == "per_head":
         # memory-bound: algorithmic bytes = float32 in and out once, and per step two reads and one write of the bf16 copy
@@ -223,16 +264,54 @@ def run_syrk_workload(name, warmup, iters, dev):
     sym = bool(torch.equal(out, out.mT))
     med, mn = statistics.median(per), min(per)
     flop = b * n * n * k
-    return {
+    # stated baselines, as the reference's SYRK benchmark times them (benchmarks/bench_batched_syrk.py:71-96 there):
+    # torch.bmm / torch.baddbmm on the same operands, the beta variant of the kernel, a loop of single-matrix calls
+    from emerging_optimizers.triton_kernels import tsyrk_ex
+
+    cmat = out.clone()  # a symmetric bf16 addend
+    bmm_ms = statistics.median(time_events(lambda: torch.bmm(a, a.mT), warmup, iters)[1])
+    baddbmm_ms = statistics.median(time_events(lambda: torch.baddbmm(cmat, a, a.mT, alpha=0.5, beta=0.25), warmup, iters)[1])
+    beta_ms = statistics.median(time_events(lambda: batched_tsyrk_ex(a, cmat, alpha=0.5, beta=0.25, out=out), warmup, iters)[1])
+    want = torch.baddbmm(cmat[:nref].float(), a[:nref].float(), a[:nref].float().mT, alpha=0.5, beta=0.25)
+    rel_beta = float((out[:nref].float() - want).norm() / want.norm())
+    sym = sym and bool(torch.equal(out, out.mT))
+    rel = max(rel, rel_beta)
+    loop_ms = statistics.median(time_events(lambda: [tsyrk_ex(a[i]) for i in range(b)], warmup, iters)[1])
+    extra = {
+        "torch_bmm_ms": round(bmm_ms, 4), "speedup_vs_torch": round(bmm_ms / med, 2),
+        "beta_variant_ms": round(beta_ms, 4), "torch_baddbmm_ms": round(baddbmm_ms, 4),
+        "beta_speedup_vs_torch": round(baddbmm_ms / beta_ms, 2), "loop_single_ms": round(loop_ms, 4),
+    }
+    return {**{
         "workload": f"batched_tsyrk_ex on {b}x{n}x{k} bf16{', operand stored transposed' if trans else ''} ({name})",
         "ms_median": round(med, 4), "ms_min": round(mn, 4), "ms_wall": round(wall, 4), "iters": iters,
         "tflops_sym": round(flop / med / 1e9, 1), "pct_peak": round(100 * flop / med / 1e9 / PEAK_BF16_TFLOPS, 2),
         "rel_fro": round(rel, 6), "bitwise_symmetric": sym, "parity": "ok" if (rel <= TOL and sym) else "FAILED",
-    }
+    }, **extra}
+
+
+def step_update_error(opt_cls, kw, w, opt, grad):
+    """One more step of `opt` on `w`, beside the same step taken statement by statement in float32 ("highest" matmul
+    precision, torch operators only) from a copy of the same state: relative Frobenius distance of the two updates."""
+    import torch
+
+    q = torch.nn.Parameter(w.detach().clone())
+    ref = opt_cls([q], **{**kw, "fp32_matmul_prec": "highest", "use_syrk": False})
+    ref.state[q]["momentum_buffer"] = opt.state[w]["momentum_buffer"].clone()
+    group = opt.param_groups[0]
+    lr, wd = group["lr"], group["weight_decay"]
+    before = w.detach().clone()
+    w.grad, q.grad = grad, grad.clone()
+    opt.step()
+    ref.step()
+    got = w.detach() - before * (1 - lr * wd)   # decoupled weight decay
+    want = q.detach() - before * (1 - lr * wd)
+    return float((got.double() - want.double()).norm() / want.double().norm())
 
 
 def run_step_workload(name, warmup, iters, dev):
-    """Whole Muon.step (momentum 0.95, Nesterov, decoupled weight decay 0.01, 5 'simple' steps)."""
+    """Whole Muon.step (momentum 0.95, Nesterov, decoupled weight decay 0.01, 5 'simple' steps); `muon_step_default`:
+    Muon(params) with every argument at the reference's default (use_syrk=False, 'quintic', no Nesterov)."""
     import torch
 
     from emerging_optimizers.orthogonalized_optimizers.muon import Muon
@@ -240,13 +319,17 @@ def run_step_workload(name, warmup, iters, dev):
     shape = STEP_WORKLOADS[name]
     kw = dict(lr=3e-4, momentum=0.95, nesterov=True, weight_decay=0.01, num_ns_steps=NS_STEPS, coefficient_type="simple",
               use_syrk=True, fp32_matmul_prec="medium")
+    if name == "muon_step_default":
+        kw = {}
     if name == "muon_heads":
         heads, m, n = shape
         gen = torch.Generator(device=dev).manual_seed(2)
         grads = [torch.randn(heads, m, n, device=dev, generator=gen) * 1e-3 for _ in range(2)]
         res = {}
+        finals = {}
         for grouped in (False, True):
-            ps = [torch.nn.Parameter(torch.randn(m, n, device=dev, generator=gen) * 0.02) for _ in range(heads)]
+            gen_w = torch.Generator(device=dev).manual_seed(3)
+            ps = [torch.nn.Parameter(torch.randn(m, n, device=dev, generator=gen_w) * 0.02) for _ in range(heads)]
             opt = Muon(ps, group_same_shape=grouped, **kw)
             state = {"i": 0}
 
@@ -257,11 +340,16 @@ def run_step_workload(name, warmup, iters, dev):
                 opt.step()
 
             _, per = time_events(one, warmup, iters)
-            res[grouped] = (statistics.median(per), min(per), all(bool(torch.isfinite(p).all()) for p in ps))
+            res[grouped] = (statistics.median(per), min(per))
+            finals[grouped] = torch.stack([p.detach() for p in ps])
+        # same weights, same gradients, same number of steps: the grouped step must land where the serial loop does
+        # (the kernels treat a batch entry exactly as the matrix alone)
+        drift = float((finals[True] - finals[False]).norm() / finals[False].norm())
         return {
             "workload": f"Muon.step over {heads} separate {m}x{n} float32 weights, group_same_shape=True ({name})",
             "ms_median": round(res[True][0], 4), "ms_min": round(res[True][1], 4), "iters": iters,
-            "ms_median_serial_loop": round(res[False][0], 4), "parity": "ok" if res[True][2] and res[False][2] else "FAILED",
+            "ms_median_serial_loop": round(res[False][0], 4), "rel_fro_vs_serial_loop": drift,
+            "parity": "ok" if drift <= 1e-6 and bool(torch.isfinite(finals[True]).all()) else "FAILED",
         }
     w = torch.nn.Parameter((torch.randn(*shape, generator=torch.Generator().manual_seed(1)) * 0.02).to(dev))
     opt = Muon([w], **kw)
@@ -275,14 +363,17 @@ def run_step_workload(name, warmup, iters, dev):
 
     wall, per = time_events(one, warmup, iters)
     med, mn = statistics.median(per), min(per)
+    rel = step_update_error(Muon, kw, w, opt, grads[0])
     m, n = sorted(shape)
     # elementwise traffic of the step outside the products: gradient and momentum read, momentum written, bf16 cast
     # written, weight read and written
     elementwise = m * n * (4 + 4 + 4 + 2 + 4 + 4)
+    what = "all arguments at the reference's defaults (use_syrk=False, quintic)" if name == "muon_step_default" else "llama-like gradients, warmed buffer"
     return {
-        "workload": f"Muon.step on one {'x'.join(map(str, shape))} float32 weight, llama-like gradients, warmed buffer ({name})",
+        "workload": f"Muon.step on one {'x'.join(map(str, shape))} float32 weight, {what} ({name})",
         "ms_median": round(med, 4), "ms_min": round(mn, 4), "ms_wall": round(wall, 4), "iters": iters,
-        "elementwise_bytes": elementwise, "parity": "ok" if bool(torch.isfinite(w).all()) else "FAILED",
+        "elementwise_bytes": elementwise, "update_rel_fro_vs_fp32_statements": round(rel, 6),
+        "parity": "ok" if (rel <= TOL and bool(torch.isfinite(w).all())) else "FAILED",
     }
 
 
@@ -392,9 +483,11 @@ def main():
 
     # ---- headline ----
     zeros = args.data == "zeros"
-    res, (wall_ms, per, out, x, schedule) = run_ns_workload("mlp", args.warmup, args.steps, lib, dev, zeros=zeros)
     if zeros:
         args.no_others = args.no_cpu_baseline = True
+    # the host-core baseline goes first: the GPU work then ends the run
+    cpu_line = None if args.no_cpu_baseline else cpu_baseline(llama_grad((M, N), seed=0))
+    res, (wall_ms, per, out, x, schedule) = run_ns_workload("mlp", args.warmup, args.steps, lib, dev, zeros=zeros)
     from emerging_optimizers import utils
     from emerging_optimizers.orthogonalized_optimizers import muon_utils
 
@@ -406,7 +499,6 @@ def main():
         ms_kind = (ctypes.c_float * 4)()
         n_kind = (ctypes.c_int * 4)()
         _hip.check(lib.mi_profile_end(ms_kind, n_kind))
-    x_cpu = x.cpu()
     del out
     f_sym, f_full, f_exec = ns_flops(1, M, N, schedule)
     tflops = f_sym / wall_ms / 1e9
@@ -450,6 +542,10 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "zeros (power probe)" if zeros else "synthetic",
+        "value_is": "effective throughput: the symmetric-halved FLOPs of five ordinary steps, 5 (3 m^2 n + m^3), over the "
+        "measured time; the driver executes fewer (schedule below), so this is not MFMA utilisation",
+        "pct_of_bf16_mfma_peak_nominal": round(100.0 * tflops / PEAK_BF16_TFLOPS, 2),
+        "pct_of_bf16_mfma_peak_executed": round(100.0 * f_exec / wall_ms / 1e9 / PEAK_BF16_TFLOPS, 2),
         "config": {
             "workload": f"newton_schulz, {NS_STEPS} steps ('simple' coefficients), one {M}x{N} float32 gradient "
             "(N(0,1e-3^2) with 1% entries at 50 sigma), bf16 MFMA kernels with fp32 accumulation, float32 result",
@@ -466,8 +562,13 @@ def main():
             "tolerance": TOL,
             "parity": "ok" if not failed else "FAILED: " + ", ".join(failed),
             "kernel_ms": {k: (round(v, 4) if v is not None else None) for k, v in per_kernel.items()},
+            "kernel_ms_note": "per launch group, from event pairs recorded around every group in a separate pass of the same "
+            "steps; the brackets lengthen each figure by about 3 %, so their sum exceeds ms_per_step",
+            "torch_bf16_path_ms": res.get("torch_bf16_path_ms"),
+            "speedup_vs_torch": res.get("speedup_vs_torch"),
+            "torch_bf16_path_rel_fro": res.get("torch_bf16_path_rel_fro"),
             "gemm_axpy_tflops": round(gemm_tflops, 1) if gemm_tflops else None,
-            "gemm_axpy_traffic_bytes": GEMM_AXPY_TRAFFIC_BYTES,
+            "gemm_axpy_traffic_bytes": GEMM_AXPY_TRAFFIC_BYTES if schedule == [3, 2] else None,
             "normalize_cast_gbps": round(norm_bytes / norm_ms / 1e6, 1) if norm_ms else None,
             "normalize_cast_pct_hbm_peak": round(100 * norm_bytes / norm_ms / 1e6 / PEAK_HBM_GBPS, 2) if norm_ms else None,
             "other_workloads": others,
@@ -481,11 +582,12 @@ def main():
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_BF16_TFLOPS, 4) if achieved else None,
             "frac_executed": round(achieved_exec / PEAK_BF16_TFLOPS, 4) if achieved_exec else None,
-            "traffic": TRI_KERNEL_TRAFFIC_BYTES if schedule == [3, 2] else None,
+            "traffic": TRI_KERNEL_TRAFFIC_BYTES if (schedule == [3, 2] and tile_gram == 192 and tile_poly == 192) else None,
+            "traffic_source": TRAFFIC_SOURCE,
             "avg_launch_ms": round(tri_ms, 4) if tri_ms else None,
         },
     }
-    line["cpu_baseline"] = None if args.no_cpu_baseline else cpu_baseline(x_cpu)
+    line["cpu_baseline"] = cpu_line
     print(json.dumps(line))
     if failed:
         sys.exit(1)
