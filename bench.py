@@ -102,6 +102,11 @@ def llama_grad(shape, seed):
     return torch.where(mask, sign * 50e-3, x)
 
 
+def note(msg):
+    """Progress line on stderr, flushed before the GPU step it names: a run that dies on the GPU still says where."""
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
 def time_events(fn, warmup, iters):
     """(wall ms per iteration over exactly `iters` calls between two synchronisations, [per-iteration ms from HIP event
     pairs on the current stream]).  No host synchronisation inside the timed region."""
@@ -194,6 +199,7 @@ def run_ns_workload(name, warmup, iters, lib, dev, zeros=False):
     from emerging_optimizers.orthogonalized_optimizers import muon_utils
 
     shape = NS_WORKLOADS[name]
+    note(f"{name}: newton_schulz on {shape}, kernels")
     x = torch.zeros(*shape, device=dev) if zeros else ns_input(name, shape, dev)
     run = lambda: muon_utils.newton_schulz(x, steps=NS_STEPS, coefficient_type="simple", use_syrk=True)
     with utils.fp32_matmul_precision("medium"), torch.no_grad():
@@ -206,10 +212,12 @@ def run_ns_workload(name, warmup, iters, lib, dev, zeros=False):
     # stated baseline: the reference's own bf16 operator sequence on torch's operators, same counts
     torch_ms = torch_rel = None
     if not zeros:
+        note(f"{name}: the reference's bf16 operator sequence on torch's operators")
         with torch.no_grad():
             _, tper = time_events(lambda: ns_torch_bf16_path(x, COEFFS), warmup, iters)
             tout = ns_torch_bf16_path(x, COEFFS)
         torch_ms = statistics.median(tper)
+    note(f"{name}: parity against float32")
     # parity: every matrix of a batch (two of them for the 1.9 GB stack)
     idx = range(batch) if x.dim() == 3 and x.numel() <= (1 << 28) else (range(2) if x.dim() == 3 else [None])
     rels = [0.0] if zeros else []
@@ -252,6 +260,7 @@ def run_syrk_workload(name, warmup, iters, dev):
     from emerging_optimizers.triton_kernels import batched_tsyrk_ex
 
     b, n, k = SYRK_WORKLOADS[name]
+    note(f"{name}: batched_tsyrk_ex on {b}x{n}x{k}")
     a = (torch.randn(b, n, k, device=dev, generator=torch.Generator(device=dev).manual_seed(0)) * 0.02).to(torch.bfloat16)
     trans = name.endswith("_trans")
     if trans:
@@ -269,13 +278,16 @@ def run_syrk_workload(name, warmup, iters, dev):
     from emerging_optimizers.triton_kernels import tsyrk_ex
 
     cmat = out.clone()  # a symmetric bf16 addend
+    note(f"{name}: torch.bmm / torch.baddbmm")
     bmm_ms = statistics.median(time_events(lambda: torch.bmm(a, a.mT), warmup, iters)[1])
     baddbmm_ms = statistics.median(time_events(lambda: torch.baddbmm(cmat, a, a.mT, alpha=0.5, beta=0.25), warmup, iters)[1])
+    note(f"{name}: beta variant")
     beta_ms = statistics.median(time_events(lambda: batched_tsyrk_ex(a, cmat, alpha=0.5, beta=0.25, out=out), warmup, iters)[1])
     want = torch.baddbmm(cmat[:nref].float(), a[:nref].float(), a[:nref].float().mT, alpha=0.5, beta=0.25)
     rel_beta = float((out[:nref].float() - want).norm() / want.norm())
     sym = sym and bool(torch.equal(out, out.mT))
     rel = max(rel, rel_beta)
+    note(f"{name}: loop of {b} single-matrix calls")
     loop_ms = statistics.median(time_events(lambda: [tsyrk_ex(a[i]) for i in range(b)], warmup, iters)[1])
     extra = {
         "torch_bmm_ms": round(bmm_ms, 4), "speedup_vs_torch": round(bmm_ms / med, 2),
@@ -317,6 +329,7 @@ def run_step_workload(name, warmup, iters, dev):
     from emerging_optimizers.orthogonalized_optimizers.muon import Muon
 
     shape = STEP_WORKLOADS[name]
+    note(f"{name}: Muon.step on {shape}")
     kw = dict(lr=3e-4, momentum=0.95, nesterov=True, weight_decay=0.01, num_ns_steps=NS_STEPS, coefficient_type="simple",
               use_syrk=True, fp32_matmul_prec="medium")
     if name == "muon_step_default":
@@ -363,6 +376,7 @@ def run_step_workload(name, warmup, iters, dev):
 
     wall, per = time_events(one, warmup, iters)
     med, mn = statistics.median(per), min(per)
+    note(f"{name}: update against the float32 statements")
     rel = step_update_error(Muon, kw, w, opt, grads[0])
     m, n = sorted(shape)
     # elementwise traffic of the step outside the products: gradient and momentum read, momentum written, bf16 cast
@@ -486,12 +500,14 @@ def main():
     if zeros:
         args.no_others = args.no_cpu_baseline = True
     # the host-core baseline goes first: the GPU work then ends the run
+    note("host-core baseline (CPU only)")
     cpu_line = None if args.no_cpu_baseline else cpu_baseline(llama_grad((M, N), seed=0))
     res, (wall_ms, per, out, x, schedule) = run_ns_workload("mlp", args.warmup, args.steps, lib, dev, zeros=zeros)
     from emerging_optimizers import utils
     from emerging_optimizers.orthogonalized_optimizers import muon_utils
 
     # per-kernel durations over another K steps, from HIP events the library records on the launch stream
+    note("mlp: per-kernel event pass")
     with utils.fp32_matmul_precision("medium"), torch.no_grad():
         lib.mi_profile_begin()
         for _ in range(args.steps):
