@@ -86,6 +86,21 @@ __device__ __forceinline__ void dma16(const uint16_t* g, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(g) : "memory");
 }
 
+// 16-byte global store at device scope (sc1): the line is written through the XCD's L2 as it is stored, instead of
+// staying dirty there until the write-back at the end of the kernel (a 4096 x 4096 bf16 result leaves 33.5 MB in the
+// eight L2s; written through, the tail of every launch is shorter: -1.3 .. -1.7 % per Newton-Schulz call, A/B on one
+// box).  Inline assembly, because no builtin sets the scope bit of a plain store.  The compiler does not know that
+// this is a store of more than 8 bytes, whose data registers must not be written by a VALU instruction in the next
+// two wait states, so the wait states are part of the statement (without them the 256 x 256 tile stored a few
+// per cent wrong values: the registers were refilled for the next store right behind this one).
+// Used by the lower-triangle epilogue only: the float32 write-out of the GEMM mode, 32 bytes per lane in two pieces,
+// became 24 % slower with it (390 -> 482 us at 4096 x 14336), its bf16 write-out did not change.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store16_through(void* ptr, const uint4& v) {
+  const u32x4_t w = {v.x, v.y, v.z, v.w};
+  asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(ptr), "v"(w) : "memory");
+}
+
 // XOR swizzle of the K-contiguous LDS tile: chunk c of row r is stored at slot kc_slot(r, c) of its row, so
 // that the 16 rows a quarter-wave reads (same chunk) cover all 64 banks.
 template <int BK>
@@ -635,7 +650,7 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, f32x4_t (
       const uint2 t0 = tr_read(a0), t1 = tr_read(a0 + 4 * LDT * 2);
       const int gr = grow0 + 4 * cq + (l16 & 3), gc = gcol0 + 32 * rb + 8 * (l16 >> 2);
       if (on && (!GUARD || (gr < p.N && gc < p.M)))
-        *reinterpret_cast<uint4*>(ob + (int64_t)gr * p.ldo + gc) = make_uint4(t0.x, t0.y, t1.x, t1.y);
+        store16_through(ob + (int64_t)gr * p.ldo + gc, make_uint4(t0.x, t0.y, t1.x, t1.y));
     }
   };
   // ---- the tile, row-major ----
@@ -696,7 +711,7 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, f32x4_t (
     // a diagonal tile holds nothing right of the diagonal block of a row (the wavefront that owns that block sits
     // the product out): that part comes from the mirror image, or stays unwritten when the upper triangle is skipped
     const bool held = !diag || c8 * 8 < (row / C::TM + 1) * C::TM;
-    if (held && (!GUARD || (gr < p.M && gc < p.N))) *reinterpret_cast<uint4*>(ob + (int64_t)gr * p.ldo + gc) = v;
+    if (held && (!GUARD || (gr < p.M && gc < p.N))) store16_through(ob + (int64_t)gr * p.ldo + gc, v);
   }
   // ---- the mirror image, straight from the staged rows ----
   if (!p.skip_upper) {
