@@ -18,6 +18,10 @@
 
 #include "gemm_engine.hpp"
 
+// Address arithmetic that the kernels share with the host-side bounds check (host_check.hpp): plain integer
+// functions, compiled for both sides, so that what the check replays is the code the GPU runs.
+#define MI_HD __host__ __device__ __forceinline__
+
 namespace mi {
 
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
@@ -74,7 +78,7 @@ using CfgSyrk192 = FastCfg<192, 2, 2, 64, 3, 192>;  // wavefronts of 96 x 96
 // Rotation (in 16-byte chunks) of k-row k of a K-strided LDS tile, chosen so that the k-rows which one pass of the
 // transpose read touches (32 lanes: 4 k-rows x 32 B at k and at k + 8) fall on disjoint banks: 32 B per k inside an
 // 8-row group, 128 B per group.
-__device__ __forceinline__ int ks_rot(int k) { return 2 * (k & 7) + 8 * (k >> 3); }
+MI_HD int ks_rot(int k) { return 2 * (k & 7) + 8 * (k >> 3); }
 
 // Direct-to-LDS load: every lane fetches 16 bytes from its own global address; the wavefront's 1 KB lands
 // at LDS byte address `lds_addr` + 16 * lane (`lds_addr` is wave-uniform and travels in M0).  Written as inline assembly so
@@ -104,7 +108,7 @@ __device__ __forceinline__ void store16_through(void* ptr, const uint4& v) {
 // XOR swizzle of the K-contiguous LDS tile: chunk c of row r is stored at slot kc_slot(r, c) of its row, so
 // that the 16 rows a quarter-wave reads (same chunk) cover all 64 banks.
 template <int BK>
-__device__ __forceinline__ int kc_slot(int row, int c) {
+MI_HD int kc_slot(int row, int c) {
   return BK == 64 ? (c ^ ((row >> 1) & 7)) : (c ^ ((row >> 2) & 3));
 }
 
@@ -145,7 +149,7 @@ struct FastLoader {
   int64_t step;                         // advance per K tile in bytes
 
   // lane's element offset inside block b, relative to the block's first element
-  static __device__ __forceinline__ int64_t lane_part(int b, int64_t ld, int lane) {
+  static MI_HD int64_t lane_part(int b, int64_t ld, int lane) {
     if (!KS) {
       const int lr = lane / C::CPR;
       const int c = kc_slot<C::BK>(C::ROWS_PER_KB * b + lr, lane % C::CPR);  // the swizzle is an involution
@@ -157,7 +161,7 @@ struct FastLoader {
     }
   }
 
-  __device__ __forceinline__ void init(const uint16_t* opbase, int64_t ld, int row0, int rows_valid, int wave, int lane) {
+  MI_HD void init(const uint16_t* opbase, int64_t ld, int row0, int rows_valid, int wave, int lane) {
     if constexpr (CLAMP) {
 #pragma unroll
       for (int i = 0; i < LPT; ++i) {
@@ -181,15 +185,16 @@ struct FastLoader {
       step = 2 * (KS ? (int64_t)C::BK * ld : (int64_t)C::BK);
     }
   }
-  // Issues load i (0 .. LPT-1) of the current K tile; `lds_tile` is the LDS byte address of the operand tile
-  // in the target ring slot.  advance() moves on to the next K tile once all LPT loads are out.
+  // Load i (0 .. LPT-1) of the current K tile reads 16 bytes at scalar_base(i) + lane_offset(i).
+  MI_HD uint64_t scalar_base(int i) const { return CLAMP ? base : base + (uint64_t)(i * block_step); }
+  MI_HD uint32_t lane_offset(int i) const { return voff[CLAMP ? i : (PERIODIC ? i % NV : i)]; }
+  MI_HD uint64_t address(int i) const { return scalar_base(i) + lane_offset(i); }
+  // Issues load i of the current K tile; `lds_tile` is the LDS byte address of the operand tile in the target ring
+  // slot.  advance() moves on to the next K tile once all LPT loads are out.
   __device__ __forceinline__ void issue_one(uint32_t lds_tile, int wave, int i) {
-    if constexpr (CLAMP)
-      dma16_sv(base, voff[i], lds_tile + (wave * LPT + i) * 1024);
-    else
-      dma16_sv(base + (uint64_t)(i * block_step), voff[PERIODIC ? i % NV : i], lds_tile + (wave * LPT + i) * 1024);
+    dma16_sv(scalar_base(i), lane_offset(i), lds_tile + (wave * LPT + i) * 1024);
   }
-  __device__ __forceinline__ void advance() { base += step; }
+  MI_HD void advance() { base += step; }
 };
 
 // MFMA fragment (8 bf16 along k per lane) of a K-contiguous tile for 16 consecutive rows starting at `row_base`,
@@ -243,7 +248,7 @@ __device__ __forceinline__ void mfma_drain() {
 // range of tile columns (all tile rows), walked in blocks of XCD_BLOCK_M tile rows: the ~32 tiles an XCD
 // works on at one time then form a compact block that shares P row-panels and Q column-panels in L2.
 constexpr int XCD_BLOCK_M = 8;
-__device__ __forceinline__ void gemm_tile_of(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+MI_HD void gemm_tile_of(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
   constexpr int XCDS = 8;
   if (tiles_n % XCDS != 0 || tiles_m % XCD_BLOCK_M != 0) {
     tm = pid % tiles_m;
@@ -271,14 +276,33 @@ __device__ __forceinline__ void gemm_tile_of(int pid, int tiles_m, int tiles_n, 
 // on 64 different banks.
 // RMW: the kernel variant for p.out_accum != 0, a compile-time flag so that the plain write-out carries none of its
 // registers and branches (with a run-time flag the plain float32 product of 4096 x 14336 took 7 us longer).
+// Geometry of the staged GEMM epilogue, relative to the first row and column of the wavefront's block.
+template <class C>
+struct GemmStage {
+  static constexpr int TN = C::TN, MI = C::MI;
+  static constexpr int LPR = TN / 8;    // lanes per output row (8 columns each)
+  static constexpr int RPI = 64 / LPR;  // rows per read iteration
+  static constexpr int NIT = MI / RPI;
+  static_assert(MI % RPI == 0 && 64 % LPR == 0, "wave tile width must be 32, 64 or 128");
+  // Row-wise passes (addend loads, old values, stores): piece t of 16-row block i of a lane is 8 columns of one row.
+  static MI_HD void piece_of(int lane, int i, int t, int& dm, int& dn) {
+    dm = i * MI + t * RPI + lane / LPR;
+    dn = (lane % LPR) * 8;
+  }
+  // Transposed float32 write-out: piece t of block i of a lane is four consecutive rows of one column.
+  static MI_HD void transposed_piece_of(int lane, int i, int t, int& dm, int& dn) {
+    dm = i * MI + 4 * (lane >> 4);
+    dn = 16 * t + (lane & 15);
+  }
+};
+
 template <class C, bool OUT_F32, bool GUARD, bool RMW>
 __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x4_t (&acc)[C::FM][C::FN], char* lds, int wave,
                                                   int lane, int m_base, int n_base, int64_t batch, float alpha,
                                                   float beta, float* red) {
+  using G = GemmStage<C>;
   constexpr int TN = C::TN, ROWB = TN * 4 + 16, MI = C::MI;
-  constexpr int LPR = TN / 8;    // lanes per output row (8 columns each)
-  constexpr int RPI = 64 / LPR;  // rows per read iteration
-  static_assert(MI % RPI == 0 && 64 % LPR == 0, "wave tile width must be 32, 64 or 128");
+  constexpr int LPR = G::LPR, RPI = G::RPI;
   static_assert(C::NW * MI * ROWB <= C::NS * C::SLOT_BYTES, "epilogue staging exceeds the ring");
   // two staging regions per wavefront when the ring has room: block i+1 is parked while block i is still being
   // re-read and stored
@@ -299,7 +323,9 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x4_t (
   auto load_cin = [&](int i) {
 #pragma unroll
     for (int t = 0; t < NIT; ++t) {
-      const int m = m_base + i * MI + t * RPI + rr, n = n_base + cc;
+      int dm, dn;
+      G::piece_of(lane, i, t, dm, dn);
+      const int m = m_base + dm, n = n_base + dn;
       cin[i % CW][t] = make_uint4(0u, 0u, 0u, 0u);
       if (use_c && (!GUARD || (m < p.M && n < p.N))) cin[i % CW][t] = *reinterpret_cast<const uint4*>(Cb + (int64_t)m * p.ldc + n);
     }
@@ -319,13 +345,18 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x4_t (
     if constexpr (RMW) {
       if (rmw_t) {
 #pragma unroll
-        for (int t = 0; t < TN / 16; ++t)
+        for (int t = 0; t < TN / 16; ++t) {
+          int dm, dn;
+          G::transposed_piece_of(lane, i, t, dm, dn);
           oldv[i % OW][t] = *reinterpret_cast<const f32x4_t*>(
-              reinterpret_cast<const float*>(p.Out) + batch * p.o_bs + (int64_t)(n_base + 16 * t + (lane & 15)) * p.ldo + m_base + i * MI + 4 * (lane >> 4));
+              reinterpret_cast<const float*>(p.Out) + batch * p.o_bs + (int64_t)(n_base + dn) * p.ldo + m_base + dm);
+        }
       } else {
 #pragma unroll
         for (int t = 0; t < NIT; ++t) {
-          const int m = m_base + i * MI + t * RPI + rr, n = n_base + cc;
+          int dm, dn;
+          G::piece_of(lane, i, t, dm, dn);
+          const int m = m_base + dm, n = n_base + dn;
           if (GUARD && (m >= p.M || n >= p.N)) continue;
           const float* o = reinterpret_cast<const float*>(p.Out) + batch * p.o_bs + (int64_t)m * p.ldo + n;
           oldv[i % OW][2 * t] = *reinterpret_cast<const f32x4_t*>(o);
@@ -349,7 +380,9 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x4_t (
 #pragma unroll
     for (int t = 0; t < NIT; ++t) {
       const int row = t * RPI + rr;
-      const int m = m_base + i * MI + row, n = n_base + cc;
+      int dm, dn;
+      G::piece_of(lane, i, t, dm, dn);
+      const int m = m_base + dm, n = n_base + dn;
       f32x4_t lo = *reinterpret_cast<const f32x4_t*>(reg + row * ROWB + cc * 4);
       f32x4_t hi = *reinterpret_cast<const f32x4_t*>(reg + row * ROWB + cc * 4 + 16);
       if (GUARD && (m >= p.M || n >= p.N)) continue;
@@ -403,7 +436,9 @@ __device__ __forceinline__ void gemm_epilogue_lds(const GemmParams& p, f32x4_t (
           f32x4_t w;
 #pragma unroll
           for (int e = 0; e < 4; ++e) w[e] = *reinterpret_cast<const float*>(reg + (g4 + e) * ROWB + (16 * t + col) * 4);
-          float* o = reinterpret_cast<float*>(p.Out) + batch * p.o_bs + (int64_t)(n_base + 16 * t + col) * p.ldo + m_base + i * MI + g4;
+          int dm, dn;
+          G::transposed_piece_of(lane, i, t, dm, dn);
+          float* o = reinterpret_cast<float*>(p.Out) + batch * p.o_bs + (int64_t)(n_base + dn) * p.ldo + m_base + dm;
           if constexpr (RMW) {
             const f32x4_t old = oldv[i % OW][t];
 #pragma unroll
@@ -450,6 +485,37 @@ struct SyrkStage {
   static constexpr int NQUAD = C::FM * C::FN;
   static constexpr bool CIN_EARLY = NQUAD * 2 <= 80;
   static_assert(STAGE_BYTES <= 160 * 1024 - 256, "staging area exceeds the LDS");
+  // Row-wise passes over the staged tile (the addend copy of the 256 x 256 tile, the write-out): piece u of thread tid
+  // is the 16-byte chunk c8 of tile row `row`.
+  static MI_HD void chunk_of(int tid, int u, int& row, int& c8) {
+    const int c = tid + u * C::NT;
+    row = c / CPRW;
+    c8 = c % CPRW;
+  }
+  // A diagonal tile holds nothing right of the diagonal block of a row (the wavefront that owns that block sits the
+  // product out): that part comes from the mirror image, or stays unwritten when the upper triangle is skipped.
+  static MI_HD bool chunk_held(bool diag, int row, int c8) { return !diag || c8 * 8 < (row / C::TM + 1) * C::TM; }
+  // Mirrored write-out of staged rows [r_lo, r_lo + ROWS) x columns [0, CCOLS): a unit is 4 columns x 32 rows; each
+  // 16-lane group transposes one unit with two LDS transpose reads (source lane L fetches the 4 columns at row
+  // 8 (L % 4) + L / 4, then 4 rows further down) and ends up with 16 bytes of a mirrored row per lane.  For iteration
+  // `it` of a lane: the staged element (src_row, src_col) its first read starts at, the row and first column of its
+  // piece of the mirror image relative to that image's corner, and whether it stores at all.
+  template <int ROWS, int CCOLS>
+  static MI_HD bool mirror_piece(int it, int wave, int lane, int r_lo, int& src_row, int& src_col, int& drow, int& dcol) {
+    static_assert(ROWS % 32 == 0 && CCOLS % 4 == 0, "units of 4 columns x 32 rows");
+    constexpr int NB = ROWS / 32, UNITS = CCOLS / 4 * NB;
+    const int l16 = lane & 15, unit = it * 16 + wave * 4 + (lane >> 4);
+    const bool on = UNITS % 16 == 0 || unit < UNITS;
+    const int u = (UNITS % 16 == 0 || unit < UNITS) ? unit : UNITS - 1;
+    const int cq = u / NB, rb = u % NB;
+    src_row = r_lo + 32 * rb + 8 * (l16 & 3) + (l16 >> 2);
+    src_col = 4 * cq;
+    drow = 4 * cq + (l16 & 3);
+    dcol = 32 * rb + 8 * (l16 >> 2);
+    return on;
+  }
+  template <int ROWS, int CCOLS>
+  static constexpr int mirror_iterations() { return (CCOLS / 4 * (ROWS / 32) + 15) / 16; }
 };
 // This lane's addend values of a one-pass tile, in accumulator layout: quad (i, j) covers row
 // m0 + mw + 16 i + (lane % 16), columns n0 + nw + 16 j + 4 (lane / 16) .. + 3.  One load
@@ -459,22 +525,26 @@ struct SyrkStage {
 // Exactly NQUAD load instructions, whatever the position of the tile: the K loop that follows counts them in its
 // vmcnt waits.  Quads beyond the matrix (GUARD) therefore read a clamped, valid address instead of being skipped; the
 // values they deliver belong to outputs that are never stored.
+// syrk_addend_elem: element offset (from the addend matrix of this batch entry) of the piece quad (i, j) of `lane` reads.
+template <class C, bool GUARD>
+MI_HD int64_t syrk_addend_elem(int M, int N, int64_t ldc, int lane, int m_base, int n_base, int i, int j) {
+  constexpr int MI = C::MI;
+  int m = m_base + i * MI + (lane & (MI - 1)), n = n_base + j * MI + 4 * (lane / MI);
+  if constexpr (GUARD) {
+    m = m < M ? m : M - 1;
+    n = n + 4 <= N ? n : N - 4;
+  }
+  return (int64_t)m * ldc + n;
+}
 template <class C, bool GUARD>
 __device__ __forceinline__ void syrk_addend_fetch(const GemmParams& p, const uint16_t* __restrict__ Cb, int lane, int m_base,
                                                   int n_base, uint2 (&pre)[SyrkStage<C>::NQUAD]) {
-  constexpr int MI = C::MI;
-  const int frow = lane & (MI - 1), fk = lane / MI;
 #pragma unroll
   for (int i = 0; i < C::FM; ++i)
 #pragma unroll
     for (int j = 0; j < C::FN; ++j)
 {
-        int m = m_base + i * MI + frow, n = n_base + j * MI + 4 * fk;
-        if constexpr (GUARD) {
-          m = m < p.M ? m : p.M - 1;
-          n = n + 4 <= p.N ? n : p.N - 4;
-        }
-        pre[i * C::FN + j] = *reinterpret_cast<const uint2*>(Cb + (int64_t)m * p.ldc + n);
+        pre[i * C::FN + j] = *reinterpret_cast<const uint2*>(Cb + syrk_addend_elem<C, GUARD>(p.M, p.N, p.ldc, lane, m_base, n_base, i, j));
       }
 }
 
@@ -571,7 +641,8 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, f32x4_t (
     auto request = [&](const uint16_t* __restrict__ src) {
 #pragma unroll
       for (int u = 0; u < NCH; ++u) {
-        const int c = tid + u * C::NT, row = c / CPRW, c8 = c % CPRW;
+        int row, c8;
+        S::chunk_of(tid, u, row, c8);
         const int gr = m0 + row, gc = n0 + c8 * 8;
         buf[u] = make_uint4(0u, 0u, 0u, 0u);
         if (!GUARD || (gr < p.M && gc < p.N)) buf[u] = *reinterpret_cast<const uint4*>(src + (int64_t)gr * p.ldc + gc);
@@ -581,7 +652,8 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, f32x4_t (
       __syncthreads();
 #pragma unroll
       for (int u = 0; u < NCH; ++u) {
-        const int c = tid + u * C::NT, row = c / CPRW, c8 = c % CPRW;
+        int row, c8;
+        S::chunk_of(tid, u, row, c8);
         *reinterpret_cast<uint4*>(lds + (row * LDT + c8 * 8) * 2) = buf[u];
       }
     };
@@ -633,22 +705,18 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, f32x4_t (
   };
   const bool sym = diag && !p.skip_upper;  // diagonal tile: the lower half and its mirror image make the tile
   const int wave = tid >> 6, l16 = lane & 15;
-  // Transposed write-out of staged rows [r_lo, r_lo + ROWS) x columns [0, CCOLS): a unit is 4 columns x 32 rows;
-  // each 16-lane group transposes one unit with two LDS transpose reads (source lane L fetches the 4 columns at
-  // row 8 (L % 4) + L / 4, then 4 rows further down) and ends up with 16 bytes of a mirrored row per lane.
+  // Transposed write-out of staged rows [r_lo, r_lo + ROWS) x columns [0, CCOLS) to the image whose corner is
+  // (grow0, gcol0); the geometry is SyrkStage::mirror_piece.
   auto mirror_out = [&](auto rows_c, auto ccols_c, int r_lo, int grow0, int gcol0) {
     constexpr int ROWS = decltype(rows_c)::value, CCOLS = decltype(ccols_c)::value;
-    static_assert(ROWS % 32 == 0 && CCOLS % 4 == 0, "units of 4 columns x 32 rows");
-    constexpr int NB = ROWS / 32, UNITS = CCOLS / 4 * NB, ITER = (UNITS + 15) / 16;
+    constexpr int ITER = S::template mirror_iterations<ROWS, CCOLS>();
 #pragma unroll
     for (int it = 0; it < ITER; ++it) {
-      const int unit = it * 16 + wave * 4 + (lane >> 4);
-      const bool on = UNITS % 16 == 0 || unit < UNITS;
-      const int u = UNITS % 16 == 0 ? unit : min(unit, UNITS - 1);
-      const int cq = u / NB, rb = u % NB;
-      const uint32_t a0 = (uint32_t)(((r_lo + 32 * rb + 8 * (l16 & 3) + (l16 >> 2)) * LDT + 4 * cq) * 2);
+      int src_row, src_col, drow, dcol;
+      const bool on = S::template mirror_piece<ROWS, CCOLS>(it, wave, lane, r_lo, src_row, src_col, drow, dcol);
+      const uint32_t a0 = (uint32_t)((src_row * LDT + src_col) * 2);
       const uint2 t0 = tr_read(a0), t1 = tr_read(a0 + 4 * LDT * 2);
-      const int gr = grow0 + 4 * cq + (l16 & 3), gc = gcol0 + 32 * rb + 8 * (l16 >> 2);
+      const int gr = grow0 + drow, gc = gcol0 + dcol;
       if (on && (!GUARD || (gr < p.N && gc < p.M)))
         store16_through(ob + (int64_t)gr * p.ldo + gc, make_uint4(t0.x, t0.y, t1.x, t1.y));
     }
@@ -705,12 +773,11 @@ __device__ __forceinline__ void syrk_epilogue_lds(const GemmParams& p, f32x4_t (
   // ---- row-wise write-out: LDS row -> global row m0 + row ----
 #pragma unroll
   for (int it = 0; it < NCH; ++it) {
-    const int c = tid + it * C::NT, row = c / CPRW, c8 = c % CPRW;
+    int row, c8;
+    S::chunk_of(tid, it, row, c8);
     const int gr = m0 + row, gc = n0 + c8 * 8;
     const uint4 v = *reinterpret_cast<const uint4*>(lds + (row * LDT + c8 * 8) * 2);
-    // a diagonal tile holds nothing right of the diagonal block of a row (the wavefront that owns that block sits
-    // the product out): that part comes from the mirror image, or stays unwritten when the upper triangle is skipped
-    const bool held = !diag || c8 * 8 < (row / C::TM + 1) * C::TM;
+    const bool held = S::chunk_held(diag, row, c8);
     if (held && (!GUARD || (gr < p.M && gc < p.N))) store16_through(ob + (int64_t)gr * p.ldo + gc, v);
   }
   // ---- the mirror image, straight from the staged rows ----
@@ -748,9 +815,40 @@ constexpr int waitcnt_imm(int vmcnt, int lgkmcnt) {
 // The launches follow each other on one stream; no workgroup ever waits for another one.  (Separate kernels and not
 // one with several roles: a 256 x 256 tile leaves no register to spare, and a kernel that spills to scratch memory
 // was measured 40 % slower on whole tiles.)
+// Workgroup -> tile of an ordinary lower-triangle launch (the numbering described above); -1 for the workgroups that
+// pad the last round to a multiple of 8.
+MI_HD int tri_tile_of_block(int bid, int lin_tiles, int g) {
+  const int full = lin_tiles / g * g;
+  if (bid < full) return bid / g * g + (bid % 8) * (g / 8) + (bid % g) / 8;
+  const int j = bid - full, rest = lin_tiles - full, lo = rest * (j % 8) / 8, hi = rest * (j % 8 + 1) / 8;
+  if (j / 8 >= hi - lo) return -1;
+  return full + lo + j / 8;
+}
+// SK_PARTS: workgroup -> (left-over tile, split, its K tiles [k_first, k_first + nk)); false for a padding workgroup.
+MI_HD bool sk_part_of_block(int bid, int sk_tpx, int sk_rem, int sk_splits, int nk_full, int& sk_tile, int& sk_split,
+                            int& k_first, int& nk) {
+  sk_tile = (bid % 8) * sk_tpx + (bid / 8) % sk_tpx;
+  sk_split = (bid / 8) / sk_tpx;
+  if (sk_tile >= sk_rem || sk_split >= sk_splits) return false;
+  k_first = nk_full * sk_split / sk_splits;
+  nk = nk_full * (sk_split + 1) / sk_splits - k_first;
+  return true;
+}
+// SK_FINISH: workgroup -> (left-over tile, quarter); the quarter is row half + 2 * column half = the wavefront of
+// SK_PARTS that computed it.
+MI_HD bool sk_quarter_of_block(int bid, int sk_rem, int& sk_tile, int& quarter) {
+  sk_tile = bid / 4;
+  quarter = bid % 4;
+  return sk_tile < sk_rem;
+}
 constexpr int SK_TILE = 256, SK_NT = 256, SK_FN = 8;                       // the tile, threads and fragment columns of SK_PARTS
 constexpr int64_t SK_IMAGE_FLOATS = (int64_t)SK_TILE * SK_TILE;            // one accumulator image
 enum { SK_NONE = 0, SK_FINISH = 2, SK_PARTS = 3 };
+// float4 index, in the array of accumulator images, of quad (i, j) of thread t (of the 256 x 256 tile's workgroup) in
+// the image of split `split` of left-over tile `sk_tile`: image split sk_rem + sk_tile, quad (i SK_FN + j) SK_NT + t.
+MI_HD int64_t sk_image_quad(int split, int sk_rem, int sk_tile, int i, int j, int t) {
+  return ((int64_t)split * sk_rem + sk_tile) * (SK_IMAGE_FLOATS / 4) + (int64_t)(i * SK_FN + j) * SK_NT + t;
+}
 // RMW: GEMM mode with float32 output only, the variant that launch_fast takes for p.out_accum != 0 (see
 // gemm_epilogue_lds).
 template <class C, bool P_KS, bool Q_KS, int MODE, bool OUT_F32, bool EDGE, int STREAMK = 0, bool RMW = false>
@@ -781,26 +879,13 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
     const int tri = p.tiles_m * (p.tiles_m + 1) / 2, bid = (int)blockIdx.x;
     int tile;
     if constexpr (STREAMK == SK_NONE) {
-      const int g = p.lin_g, full = p.lin_tiles / g * g;
-      if (bid < full) {
-        tile = bid / g * g + (bid % 8) * (g / 8) + (bid % g) / 8;
-      } else {
-        const int j = bid - full, rest = p.lin_tiles - full, lo = rest * (j % 8) / 8, hi = rest * (j % 8 + 1) / 8;
-        if (j / 8 >= hi - lo) return;  // padding workgroup (leaves before any barrier)
-        tile = full + lo + j / 8;
-      }
+      tile = tri_tile_of_block(bid, p.lin_tiles, p.lin_g);
+      if (tile < 0) return;  // padding workgroup (leaves before any barrier)
     } else {
       if constexpr (STREAMK == SK_PARTS) {
-        const int nk_full = p.K / C::BK;
-        sk_tile = (bid % 8) * p.sk_tpx + (bid / 8) % p.sk_tpx;
-        sk_split = (bid / 8) / p.sk_tpx;
-        if (sk_tile >= p.sk_rem || sk_split >= p.sk_splits) return;  // padding workgroup
-        k_first = nk_full * sk_split / p.sk_splits;
-        nk = nk_full * (sk_split + 1) / p.sk_splits - k_first;
+        if (!sk_part_of_block(bid, p.sk_tpx, p.sk_rem, p.sk_splits, p.K / C::BK, sk_tile, sk_split, k_first, nk)) return;  // padding workgroup
       } else {
-        sk_tile = bid / 4;
-        sk_split = bid % 4;  // (the quarter: row half + 2 * column half = the wavefront of SK_PARTS that computed it)
-        if (sk_tile >= p.sk_rem) return;
+        if (!sk_quarter_of_block(bid, p.sk_rem, sk_tile, sk_split)) return;
       }
       tile = p.lin_tiles + sk_tile;
     }
@@ -1051,11 +1136,11 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
   if constexpr (STREAMK == SK_PARTS) {
     // image of split s of left-over tile t: slot s sk_rem + t; quad (i, j) of thread t at ((i SK_FN + j) SK_NT + t) float4s
     if (!idle_wave) {
-      f32x4_t* img = reinterpret_cast<f32x4_t*>(p.sk_partials + ((int64_t)sk_split * p.sk_rem + sk_tile) * SK_IMAGE_FLOATS) + tid;
+      f32x4_t* img = reinterpret_cast<f32x4_t*>(p.sk_partials);
       static_for<FM>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
 #pragma unroll
-        for (int j = 0; j < FN; ++j) img[(int64_t)(i * FN + j) * NT] = acc[i][j];
+        for (int j = 0; j < FN; ++j) img[sk_image_quad(sk_split, p.sk_rem, sk_tile, i, j, tid)] = acc[i][j];
         __builtin_amdgcn_sched_barrier(0);  // one fragment row at a time: the image must not pile up in registers
       });
     }
@@ -1068,18 +1153,16 @@ __global__ void __launch_bounds__(C::NT) gemm_fast_kernel(GemmParams p) {
     }
     if (!idle_wave) {
       // this wavefront's 64 x 64 block inside the quarter = fragments (wm FM + i, wn FN + j) of wavefront sk_split of SK_PARTS
-      const f32x4_t* img = reinterpret_cast<const f32x4_t*>(p.sk_partials + (int64_t)sk_tile * SK_IMAGE_FLOATS) +
-                           ((wm * FM) * SK_FN + wn * FN) * SK_NT + sk_split * 64 + lane;
+      const f32x4_t* img = reinterpret_cast<const f32x4_t*>(p.sk_partials);
       for (int s = 0; s < p.sk_splits; ++s) {
 #pragma unroll
         for (int i = 0; i < FM; ++i)
 #pragma unroll
           for (int j = 0; j < FN; ++j) {
-            const f32x4_t v = img[(int64_t)(i * SK_FN + j) * SK_NT];
+            const f32x4_t v = img[sk_image_quad(s, p.sk_rem, sk_tile, wm * FM + i, wn * FN + j, sk_split * 64 + lane)];
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[i][j][e] += v[e];
           }
-        img += (int64_t)p.sk_rem * (SK_IMAGE_FLOATS / 4);
       }
     }
   }

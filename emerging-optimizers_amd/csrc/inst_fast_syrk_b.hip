@@ -50,9 +50,8 @@ int launch_streamk(const GemmParams& p, int64_t batch, int cus, void* workspace,
     q.sk_partials = static_cast<float*>(workspace);
     const int parts = 8 * q.sk_tpx * plan.splits;
     grid = (whole > 0 ? grid : 0) + parts;
-    hipLaunchKernelGGL((gemm_fast_kernel<C, false, false, MODE_SYRK, false, false, SK_PARTS>), dim3(parts), dim3(C::NT), 0, stream, q);
-    hipLaunchKernelGGL((gemm_fast_kernel<CfgT128x2, false, false, MODE_SYRK, false, false, SK_FINISH>), dim3(4 * plan.rem),
-                       dim3(CfgT128x2::NT), 0, stream, q);
+    MI_LAUNCH_FAST(C, false, false, MODE_SYRK, false, false, SK_PARTS, false, dim3(parts), stream, q);
+    MI_LAUNCH_FAST(CfgT128x2, false, false, MODE_SYRK, false, false, SK_FINISH, false, dim3(4 * plan.rem), stream, q);
   }
   g_last_launch = LastLaunch{grid, C::TILE_M, C::TILE_N, 2};
   hipError_t e = hipGetLastError();

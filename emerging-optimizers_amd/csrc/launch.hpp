@@ -8,6 +8,22 @@
 #include "gemm_fast.hpp"
 #include "norm_common.hpp"
 
+// Every launch of the fast kernel goes through MI_LAUNCH_FAST.  In the host-side bounds check build (MI_HOST_CHECK,
+// `make host-check`) nothing is launched: the fast kernel's launches are walked on the host (host_check.hpp), the other
+// kernels' launches and the runtime calls around them are compiled out.
+#ifdef MI_HOST_CHECK
+#include "host_check.hpp"
+#undef hipLaunchKernelGGL
+#define hipLaunchKernelGGL(...) ((void)0)
+#define hipGetLastError() hipSuccess
+#define hipFuncSetAttribute(...) hipSuccess
+#define MI_LAUNCH_FAST(C, P_KS, Q_KS, MODE, OUT_F32, EDGE, SK, RMW, grid, stream, q) \
+  ::mi::host_check::fast_launch<C, P_KS, Q_KS, MODE, OUT_F32, EDGE, SK, RMW>(grid, q)
+#else
+#define MI_LAUNCH_FAST(C, P_KS, Q_KS, MODE, OUT_F32, EDGE, SK, RMW, grid, stream, q) \
+  hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, EDGE, SK, RMW>), grid, dim3(C::NT), 0, stream, q)
+#endif
+
 namespace mi {
 
 // Records the text behind mi_last_error() for this host thread and returns `code`.

@@ -63,7 +63,7 @@ int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream, int64_t 
   GemmParams q = p;
   q.tiles_m = (p.M + C::TILE_M - 1) / C::TILE_M;
   q.tiles_n = (p.N + C::TILE_N - 1) / C::TILE_N;
-  dim3 grid, block(C::NT, 1, 1);
+  dim3 grid;
   int64_t tiles;
   if constexpr (MODE == MODE_SYRK) {
     // one-dimensional grid over the tiles of the whole batch: whole rounds, then a last round with the same number
@@ -92,18 +92,18 @@ int launch_fast(const GemmParams& p, int64_t batch, hipStream_t stream, int64_t 
   constexpr bool HAS_EDGE_VARIANT = MODE == MODE_SYRK && !P_KS && !Q_KS;
   if (edge) {
     if constexpr (HAS_EDGE_VARIANT)
-      hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, true>), grid, block, 0, stream, q);
+      MI_LAUNCH_FAST(C, P_KS, Q_KS, MODE, OUT_F32, true, 0, false, grid, stream, q);
     else
       return fail(MI_ERR_UNSUPPORTED_SHAPE, "internal: %d x %d is not a whole number of %d x %d tiles", p.M, p.N, C::TILE_M, C::TILE_N);
   } else {
     constexpr bool HAS_RMW_VARIANT = MODE == MODE_GEMM && OUT_F32 && (C::TN == 32 || C::TN == 64 || C::TN == 128);
     if constexpr (HAS_RMW_VARIANT) {
       if (p.out_accum != 0.0f)
-        hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, false, 0, true>), grid, block, 0, stream, q);
+        MI_LAUNCH_FAST(C, P_KS, Q_KS, MODE, OUT_F32, false, 0, true, grid, stream, q);
       else
-        hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, false>), grid, block, 0, stream, q);
+        MI_LAUNCH_FAST(C, P_KS, Q_KS, MODE, OUT_F32, false, 0, false, grid, stream, q);
     } else {
-      hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, false>), grid, block, 0, stream, q);
+      MI_LAUNCH_FAST(C, P_KS, Q_KS, MODE, OUT_F32, false, 0, false, grid, stream, q);
     }
   }
   g_last_launch = LastLaunch{(int)grid.x, C::TILE_M, C::TILE_N, 1};

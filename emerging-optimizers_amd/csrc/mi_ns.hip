@@ -1500,6 +1500,14 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
   if (reinterpret_cast<uintptr_t>(workspace) & 255u) return fail(MI_ERR_WORKSPACE, "workspace must be 256-byte aligned");
 
   char* ws = static_cast<char*>(workspace);
+#ifdef MI_HOST_CHECK
+  {  // the segments of the workspace as buffers of their own: an access that strays from one into the next is caught
+    const size_t at[] = {w.x0, w.x1, w.a, w.b, w.t, w.d2, w.partials, w.norm, w.slots, w.shift, w.xscale, w.result, w.gpart, w.total};
+    const char* const names[] = {"ws.x0", "ws.x1", "ws.gram", "ws.poly", "ws.t", "ws.d2", "ws.partials", "ws.norm", "ws.slots",
+                                 "ws.shift", "ws.xscale", "ws.result", "ws.gpart"};
+    for (int i = 0; i < 13; ++i) host_check::add_range(ws + at[i], at[i + 1] - at[i], names[i]);
+  }
+#endif
   uint16_t* xbuf[2] = {reinterpret_cast<uint16_t*>(ws + w.x0), reinterpret_cast<uint16_t*>(ws + w.x1)};
   uint16_t* gram = reinterpret_cast<uint16_t*>(ws + w.a);
   uint16_t* poly = reinterpret_cast<uint16_t*>(ws + w.b);
