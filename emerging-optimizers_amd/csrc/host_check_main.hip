@@ -201,11 +201,13 @@ int selftest() {
 int main(int argc, char** argv) {
   if (argc > 1 && std::strcmp(argv[1], "--selftest") == 0) return selftest();
   const bool quick = argc > 1 && std::strcmp(argv[1], "--quick") == 0;
+  const bool bench_only = argc > 1 && std::strcmp(argv[1], "--bench") == 0;  // the benchmark's own calls only
   validation_cases();
   // ---- lower-triangle products
   const int64_t ns_[] = {256, 384, 512, 768, 1024, 1032, 1096, 1152, 1280, 1536, 1792, 1800, 2048, 2304, 3072, 4096, 5120, 8184, 8192};
   const int64_t ks_[] = {64, 128, 192, 448, 1024, 4096, 8192, 14336};
   for (int streamk : {-1, 1}) {
+    if (bench_only) break;
     for (int transpose : {-1, 0, 1}) {
       set("streamk", streamk);
       set("syrk_transpose", transpose);
@@ -247,7 +249,7 @@ int main(int argc, char** argv) {
                               {384, 768},   {896, 256},   {128, 4096},  {256, 1024},  {1000, 2048},  {1024, 1032}, {1032, 2048}, {64, 64}};
   for (const auto& s : gemm_)
     for (int64_t batch : {1, 2, 8}) {
-      if (quick && batch > 1) continue;
+      if ((quick && batch > 1) || bench_only) continue;
       for (int x_trans : {0, 1})
         for (int out_fp32 : {0, 1}) gemm_case(batch, s[0], s[1], x_trans, out_fp32);
     }
@@ -274,10 +276,11 @@ int main(int argc, char** argv) {
         set("tall_direct", direct);
         set("head_apply", head);
         set("head_front", head);
-        if (quick && (pairs == 1 || direct == 0)) continue;
+        if ((quick && (pairs == 1 || direct == 0)) || (bench_only && !(pairs == -1 && direct == 1 && head == 1))) continue;
         for (const auto& s : nsh) {
           if (quick && s[0] * s[1] * s[2] > (int64_t)1 << 22) continue;
           for (const Kind& kd : kinds) {
+            if (bench_only && !(kd.steps == 5 && kd.abc != CUBIC)) continue;
             if (pairs != -1 && kd.steps < 4) continue;
             if (quick && (kd.steps == 4 || kd.steps == 1)) continue;
             ns_case(s[0], s[1], s[2], kd.abc, kd.steps, kd.name, false);

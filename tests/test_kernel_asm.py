@@ -194,3 +194,19 @@ def test_first_addend_is_requested_with_the_counted_number_of_loads(compiled_ker
         assert (ns - 2) * loads_per_tile + nquad in waits, (name, sorted(waits))
         seen += 1
     assert seen >= 6  # 128 x 128 (two ring depths) and 192 x 192 tiles, whole and edge variants, both operand layouts
+
+
+def test_device_scope_stores_carry_their_wait_states(compiled_kernels):
+    """The lower-triangle epilogue stores its result with an inline-assembly `global_store_dwordx4 ... sc1` (written
+    through the L2).  The compiler does not know that this is a store of more than 8 bytes, after which the data
+    registers must not be rewritten for two wait states, so the statement carries an `s_nop 1` of its own: every such
+    store in the compiled kernels must be followed by it, and there must be some (the staged epilogue of every
+    lower-triangle kernel has two store loops)."""
+    found = 0
+    for name, lines in compiled_kernels.items():
+        text = [t for _, t in instructions(lines)]
+        for k, t in enumerate(text):
+            if t.startswith("global_store_dwordx4") and t.endswith("sc1"):
+                found += 1
+                assert text[k + 1] == "s_nop 1", (name, t, text[k + 1])
+    assert found >= 20
