@@ -27,12 +27,24 @@ def _np(t):
 
 # ---------------------------------------------------------------- step functions
 def _torch_step(x, a, b, c):
-    """The operator sequence of the reference's GEMM steps (muon_utils.py:370-377, 403-410 there), on torch's matmuls."""
-    A = x @ x.mT
-    add = torch.baddbmm if x.ndim == 3 else torch.addmm
-    if c == 0.0:
-        return add(x, A, x, alpha=b, beta=a)
-    return add(x, add(A, A, A, alpha=c, beta=b), x, alpha=1.0, beta=a)
+    """The operator sequence of the reference's GEMM steps (muon_utils.py:370-377, 403-410 there) with its rounding
+    points on bf16 operands -- every product accumulated in float32 and rounded to bf16 once -- spelled out on torch's
+    float32 matmuls: `X @ X.mT`, `addmm(A, A, A, alpha=c, beta=b)`, `addmm(X, B, X, alpha=1, beta=a)` each become a
+    float32 product of the bf16 values followed by `.to(bfloat16)`.  (torch's own bf16 matmuls are not used as the
+    reference here: the float32 ones with "highest" precision give the same rounding points and an exact sum on the
+    integer cases.)  float32 input: plain float32 arithmetic."""
+    prev = torch.get_float32_matmul_precision()
+    torch.set_float32_matmul_precision("highest")
+    try:
+        rnd = (lambda t: t.to(BF).float()) if x.dtype == BF else (lambda t: t)
+        X = x.float()
+        A = rnd(X @ X.mT)
+        if c == 0.0:
+            return rnd(a * X + b * (A @ X)).to(x.dtype)
+        B = rnd(b * A + c * (A @ A))
+        return rnd(a * X + B @ X).to(x.dtype)
+    finally:
+        torch.set_float32_matmul_precision(prev)
 
 
 @pytest.fixture
@@ -68,7 +80,7 @@ def test_gemm_and_tsyrk_steps_bit_equal_to_torch_and_oracle(gpu, kernel_calls, s
     via_gemm_step = gemm(x, a, b, c)
     assert kernel_calls == {"syrk": 4, "gemm": 2}  # the GEMM step runs on the HIP kernels as well
     assert got.dtype == BF and torch.equal(got, via_gemm_step)
-    assert torch.equal(got, _torch_step(x, a, b, c))  # hipBLASLt through torch: same rounding points, exact sums
+    assert torch.equal(got, _torch_step(x, a, b, c))  # float32 torch matmuls with the same rounding points: exact sums
     assert np.array_equal(_np(got), O.newton_schulz_step(_np(x), a, b, c, bf16=True))
     if batched:
         per = torch.stack([muon_utils.newton_schulz_step(x[i], a, b, c) for i in range(shape[0])])
@@ -84,9 +96,10 @@ def test_gemm_and_tsyrk_steps_bit_equal_to_torch_and_oracle(gpu, kernel_calls, s
 
 @pytest.mark.parametrize("shape", [(1024, 2048), (2, 1024, 1280), (256, 768), (4, 128, 1024), (2048, 1024)])
 def test_gemm_step_on_the_kernels_matches_torch_operators(gpu, kernel_calls, shape):
-    """Sizes that reach the direct-to-LDS kernels: random operands, so the float32 sums differ in order from
-    hipBLASLt's and a bf16 rounding flips here and there -- agreement to bf16 resolution, as the reference asks of its
-    own SYRK against cuBLAS (rtol 0.05 in tests/test_triton_kernels.py:138-204 there), and much tighter in norm."""
+    """Sizes that reach the direct-to-LDS kernels: random operands, so the float32 sums differ in order from a
+    library's and a bf16 rounding flips here and there -- agreement to bf16 resolution with the same rounding points
+    computed on float32 matmuls, as the reference asks of its own SYRK against cuBLAS (rtol 0.05 in
+    tests/test_triton_kernels.py:138-204 there), and much tighter in norm."""
     x = torch.randn(*shape, device=gpu)
     x = (x / x.norm(dim=(-2, -1), keepdim=True)).to(BF)
     if shape[-2] > shape[-1]:
@@ -95,21 +108,23 @@ def test_gemm_step_on_the_kernels_matches_torch_operators(gpu, kernel_calls, sha
     a, b, c = 3.4445, -4.7750, 2.0315
     got = step(x, a, b, c)
     assert kernel_calls == {"syrk": 2, "gemm": 1}
-    ref = _torch_step(x.contiguous(), a, b, c)
+    ref = _torch_step(x.contiguous(), a, b, c)  # the rounding points of the reference's bf16 step
     assert got.shape == ref.shape and got.dtype == BF
     assert rel_fro(got.float().cpu(), ref.float().cpu()) <= 3e-3
-    exact = _torch_step(x.float(), a, b, c)  # float32 arithmetic on the same bf16 operand
+    torch.testing.assert_close(got.float(), ref.float(), rtol=0.05, atol=1e-3)
+    exact = _torch_step(x.float(), a, b, c)  # float32 arithmetic on the same bf16 operand, no rounding in between
     assert rel_fro(got.float().cpu(), exact.cpu()) <= 1.2 * rel_fro(ref.float().cpu(), exact.cpu()) + 1e-4
 
 
 def test_gemm_step_keeps_torch_for_what_the_kernels_do_not_take(gpu, kernel_calls):
-    """float32 operands, dims that are not multiples of 8 and CPU tensors stay on torch's matmuls (the reference's
-    path); nothing reaches the kernels."""
+    """float32 operands, dims that are not multiples of 8, rows that are neither contiguous nor transposed-contiguous and
+    CPU tensors stay on torch's matmuls (the reference's path); nothing reaches the kernels."""
     for x in (torch.randn(64, 128, device=gpu), torch.randn(12, 40, device=gpu).to(BF), torch.randn(2, 12, 40, device=gpu).to(BF),
               torch.randn(16, 32).to(BF), torch.randn(64, 128, device=gpu).to(BF)[::2]):
         step = muon_utils.batched_newton_schulz_step if x.ndim == 3 else muon_utils.newton_schulz_step
         got = step(x, 0.5, 0.25, 0.125)
-        assert torch.equal(got, _torch_step(x, 0.5, 0.25, 0.125))
+        assert got.dtype == x.dtype and got.shape == x.shape
+        torch.testing.assert_close(got.float().cpu(), _torch_step(x, 0.5, 0.25, 0.125).float().cpu(), rtol=0.05, atol=0.02)
     assert kernel_calls == {"syrk": 0, "gemm": 0}
 
 
