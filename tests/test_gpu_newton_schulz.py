@@ -111,7 +111,6 @@ def test_gemm_step_on_the_kernels_matches_torch_operators(gpu, kernel_calls, sha
     ref = _torch_step(x.contiguous(), a, b, c)  # the rounding points of the reference's bf16 step
     assert got.shape == ref.shape and got.dtype == BF
     assert rel_fro(got.float().cpu(), ref.float().cpu()) <= 3e-3
-    torch.testing.assert_close(got.float(), ref.float(), rtol=0.05, atol=1e-3)
     exact = _torch_step(x.float(), a, b, c)  # float32 arithmetic on the same bf16 operand, no rounding in between
     assert rel_fro(got.float().cpu(), exact.cpu()) <= 1.2 * rel_fro(ref.float().cpu(), exact.cpu()) + 1e-4
 
@@ -124,7 +123,8 @@ def test_gemm_step_keeps_torch_for_what_the_kernels_do_not_take(gpu, kernel_call
         step = muon_utils.batched_newton_schulz_step if x.ndim == 3 else muon_utils.newton_schulz_step
         got = step(x, 0.5, 0.25, 0.125)
         assert got.dtype == x.dtype and got.shape == x.shape
-        torch.testing.assert_close(got.float().cpu(), _torch_step(x, 0.5, 0.25, 0.125).float().cpu(), rtol=0.05, atol=0.02)
+        # (torch's own matmuls against the same rounding points on float32 matmuls: equal up to the order of the sums)
+        assert rel_fro(got.float().cpu(), _torch_step(x, 0.5, 0.25, 0.125).float().cpu()) <= 1e-2
     assert kernel_calls == {"syrk": 0, "gemm": 0}
 
 
