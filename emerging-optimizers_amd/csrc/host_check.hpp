@@ -12,8 +12,13 @@
 //
 // What is replayed by hand here, because it is control flow and not address arithmetic: which K tiles a workgroup
 // requests (all of [0, nk): the guards of the prologue and of the steady and tail loops), and which epilogue a variant
-// runs.  Launches of the other kernels (normalisation passes, transposes, the general tile kernel, the per-head
-// kernels) are skipped: they guard their own accesses.
+// runs.
+//
+// The other kernels (normalisation passes, transposes, the general tile kernel, the per-head kernels) guard their own
+// accesses or run on exact multiples of their slices; what can go wrong for them is the host side: a workspace segment
+// carved too small, a stride or a count passed wrongly.  Their launch sites state, with MI_FOOTPRINT (launch.hpp), the
+// block of memory every pointer argument of the launch covers, and footprint() below checks each block against the
+// registered buffers the same way.
 #pragma once
 #include <cstdint>
 #include <cstdio>
@@ -33,6 +38,7 @@ struct Range {
 struct State {
   std::vector<Range> ranges;
   long launches = 0, workgroups = 0, accesses = 0, failures = 0;
+  long other_launches = 0, footprints = 0;  // launches of the self-guarding kernels, blocks of memory they stated
   const char* context = "";
   uint64_t hit_lo = 1, hit_hi = 0;  // the buffer the last access fell into (consecutive accesses mostly share one)
 };
@@ -80,6 +86,55 @@ __attribute__((no_sanitize("address", "undefined"))) inline void touch(uint64_t 
 template <class T>
 inline void touch(const T* p, size_t bytes, const char* what, const char* detail = "") {
   touch((uint64_t)(uintptr_t)p, bytes, what, detail);
+}
+
+// One pointer argument of a self-guarding kernel: `batch` blocks `batch_stride` elements apart, each of `rows` rows of
+// `cols` elements that start `ld` elements apart, `elem` bytes per element.  Every block must lie inside one registered
+// buffer (all blocks of up to 4096 batch entries, the two ends beyond that: the blocks are equally spaced).
+inline void footprint(const char* what, const void* base, size_t elem, int64_t batch, int64_t batch_stride, int64_t rows, int64_t ld,
+                      int64_t cols) {
+  if (base == nullptr || batch <= 0 || rows <= 0 || cols <= 0) return;
+  State& st = state();
+  ++st.footprints;
+  if (batch_stride < 0 || ld < cols) fail("a footprint with rows that overlap");
+  const size_t bytes = (size_t)((rows - 1) * ld + cols) * elem;
+  const char* b0 = static_cast<const char*>(base);
+  for (int64_t b = 0; b < batch; ++b) {
+    if (batch > 4096 && b == 1) b = batch - 1;
+    touch(b0 + (size_t)b * batch_stride * elem, bytes, what, "whole block of a self-guarding kernel");
+  }
+}
+inline void other_launch() { ++state().other_launches; }
+
+// The scalars every tile kernel resolves per batch entry (resolve_shift in gemm_engine.hpp) and the partial sums its
+// workgroups leave: `slots` workgroups per batch entry write one float each.
+inline void scalar_footprints(const GemmParams& p, int64_t batch, int64_t slots) {
+  if (p.shift_mode == SHIFT_GRAM) {
+    footprint("partial sums read", p.slots_in, sizeof(float), batch, p.nslots_in, 1, p.nslots_in, p.nslots_in);
+    footprint("shift written", p.shift_io, sizeof(float), 1, 0, 1, batch, batch);
+  } else if (p.shift_mode != SHIFT_NONE) {
+    footprint("shift read", p.shift_io, sizeof(float), 1, 0, 1, batch, batch);
+  }
+  footprint("input scale read", p.xscale, sizeof(float), 1, 0, 1, batch, batch);
+  if (p.slots_out != nullptr) footprint("partial sums written", p.slots_out + p.slot_base, sizeof(float), batch, p.slot_stride, 1, slots, slots);
+}
+
+// A launch of the general tile kernel (gemm_engine.hpp; every access guarded by the matrix extents): operands, addends
+// and result as the extents in `p` describe them.
+inline void general_launch(const GemmParams& p, int64_t batch, bool p_ks, bool q_ks, bool syrk, bool out_f32, int64_t tiles) {
+  other_launch();
+  const int64_t inner = p.batch_inner > 1 ? p.batch_inner : 1, outer = batch / inner;
+  if (batch % inner != 0) fail("batch is not a whole number of inner batches");
+  for (int64_t in = 0; in < inner; ++in) {
+    const int64_t p2 = p.batch_inner > 1 ? in * p.p_bs2 : 0, q2 = p.batch_inner > 1 ? in * p.q_bs2 : 0;
+    footprint("operand P", p.P + p2, 2, outer, p.p_bs, p_ks ? p.K : p.M, p.ldp, p_ks ? p.M : p.K);
+    footprint("operand Q", p.Q + q2, 2, outer, p.q_bs, q_ks ? p.K : p.N, p.ldq, q_ks ? p.N : p.K);
+  }
+  // (the addends are read whenever their pointers are given: the coefficients are resolved on the device)
+  footprint("addend", p.Cin, 2, batch, p.c_bs, p.M, p.ldc, p.N);
+  footprint("second addend", p.Cin2, 2, batch, p.c_bs, p.M, p.ldc, p.N);
+  footprint("result", p.Out, out_f32 ? 4 : 2, batch, p.o_bs, p.M, p.ldo, p.N);
+  scalar_footprints(p, batch, syrk ? 0 : tiles);
 }
 
 template <class C, bool P_KS, bool Q_KS, int MODE, bool OUT_F32, bool EDGE, int STREAMK, bool RMW>

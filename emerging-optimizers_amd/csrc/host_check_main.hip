@@ -87,6 +87,18 @@ void gemm_case(int64_t batch, int64_t m, int64_t n, int x_trans, int out_fp32, i
                               out_fp32, 2.0f, nullptr));
 }
 
+void frob_case(int64_t batch, int64_t numel, int out_bf16, int f64) {
+  char what[200];
+  std::snprintf(what, sizeof what, "frob_normalize batch=%lld numel=%lld out_bf16=%d f64=%d", (long long)batch, (long long)numel, out_bf16, f64);
+  begin(what);
+  void* x = fake_alloc((size_t)batch * numel * 4, "x");
+  void* out = fake_alloc((size_t)batch * numel * (out_bf16 ? 2 : 4), "out");
+  void* partials = fake_alloc(mi_frob_partials_len(batch, numel) * 8, "partials");
+  void* norm = fake_alloc((size_t)batch * 4, "norm");
+  expect_ok(mi_frob_normalize(static_cast<const float*>(x), batch, numel, 1e-7f, f64, out, out_bf16, static_cast<double*>(partials),
+                              static_cast<float*>(norm), nullptr));
+}
+
 const float SIMPLE[15] = {3.4445f, -4.7750f, 2.0315f, 3.4445f, -4.7750f, 2.0315f, 3.4445f, -4.7750f, 2.0315f,
                           3.4445f, -4.7750f, 2.0315f, 3.4445f, -4.7750f, 2.0315f};
 const float QUINTIC[15] = {4.0848f, -6.8946f, 2.9270f, 3.9505f, -6.3029f, 2.6377f, 3.7418f, -5.5913f, 2.3037f,
@@ -193,7 +205,20 @@ int selftest() {
     found[which] = state().failures - before;
   }
   std::printf("host-check selftest: undersized result / operand / addend reported %ld / %ld / %ld times\n", found[0], found[1], found[2]);
-  return (found[0] > 0 && found[1] > 0 && found[2] > 0) ? 0 : 1;
+  // the self-guarding kernels: a normalisation call whose output, or whose array of partial sums, is too small
+  long stated[2] = {0, 0};
+  for (int which = 0; which < 2; ++which) {
+    begin("selftest");
+    const int64_t batch = 3, numel = 256 * 512;
+    void* x = fake_alloc((size_t)batch * numel * 4, "x");
+    void* out = fake_alloc((size_t)batch * numel * 2 - (which == 0 ? 16 : 0), "out");
+    void* partials = fake_alloc(which == 1 ? 8 * (size_t)batch : mi_frob_partials_len(batch, numel) * 8, "partials");  // (one per matrix: too few)
+    const long before = state().failures;
+    expect_ok(mi_frob_normalize(static_cast<const float*>(x), batch, numel, 1e-7f, 0, out, 1, static_cast<double*>(partials), nullptr, nullptr));
+    stated[which] = state().failures - before;
+  }
+  std::printf("host-check selftest: undersized normalised copy / partial sums reported %ld / %ld times\n", stated[0], stated[1]);
+  return (found[0] > 0 && found[1] > 0 && found[2] > 0 && stated[0] > 0 && stated[1] > 0) ? 0 : 1;
 }
 
 }  // namespace
@@ -256,6 +281,11 @@ int main(int argc, char** argv) {
   gemm_case(1, 4096, 14336, 0, 0, 0, 12288);  // a column range of a wider matrix, as the tail split of the library itself
   gemm_case(1, 4096, 14336, 0, 1, 12288, 2048);
   gemm_case(1, 4096, 14336, 1, 1, 12288, 2048);
+  // ---- normalisation on its own
+  for (int64_t batch : {1, 5})
+    for (int64_t numel : {8, 4096, 1 << 20, 4096 * 14336})
+      for (int out_bf16 : {0, 1})
+        for (int f64 : {0, 1}) frob_case(batch, numel, out_bf16, f64);
   // ---- the single-call driver and the fused optimizer update
   const int64_t nsh[][3] = {{1, 256, 512},   {1, 512, 256},   {1, 64, 64},      {1, 8, 16},      {3, 128, 384},   {2, 384, 128},  {1, 1024, 1280},
                             {4, 128, 1024},  {2, 256, 1536},  {1, 1536, 256},   {1, 1024, 2048}, {2, 1024, 2304}, {1, 200, 456},  {1, 1024, 2560},
@@ -289,7 +319,8 @@ int main(int argc, char** argv) {
         }
       }
   const mi::host_check::State& st = state();
-  std::printf("host-check: %ld library calls (%ld refused as unsupported), %ld fast-kernel launches, %ld workgroups, %ld accesses checked, %ld failures\n",
-              g_calls, g_refused, st.launches, st.workgroups, st.accesses, st.failures);
+  std::printf("host-check: %ld library calls (%ld refused as unsupported), %ld fast-kernel launches, %ld workgroups, %ld accesses checked, "
+              "%ld other launches with %ld stated blocks, %ld failures\n",
+              g_calls, g_refused, st.launches, st.workgroups, st.accesses, st.other_launches, st.footprints, st.failures);
   return st.failures == 0 ? 0 : 1;
 }

@@ -182,6 +182,14 @@ int launch_head_apply(const GemmParams& p, int64_t batch, int splits, float* gra
   if (q.slot_stride == 0) q.slot_stride = splits;
   if (int rc = check_slots(q, splits)) return rc;
   dim3 grid((unsigned)(batch * splits)), block(HA_NT);
+  MI_OTHER_LAUNCH();
+  MI_FOOTPRINT("multiplier S", q.P, 2, batch, q.p_bs, HA_M, q.ldp, HA_M);
+  MI_FOOTPRINT("X", q.Q, 2, batch, q.q_bs, HA_M, q.ldq, q.N);
+  MI_FOOTPRINT("X'", q.Out, out_f32 ? 4 : 2, batch, q.o_bs, HA_M, q.ldo, q.N);
+  MI_FOOTPRINT("Gram partials of X'", gram_next, 4, batch, (int64_t)splits * HA_M * HA_M, splits, HA_M * HA_M, HA_M * HA_M);
+#ifdef MI_HOST_CHECK
+  host_check::scalar_footprints(q, batch, splits);
+#endif
   if (out_f32)
     hipLaunchKernelGGL(head_apply_kernel<true>, grid, block, 0, stream, q, gram_next, splits);
   else
@@ -352,6 +360,15 @@ int launch_head_front(const float* x, int64_t batch, int64_t n, float eps, Momen
     return fail(MI_ERR_UNSUPPORTED_SHAPE, "internal: per-head input pass on %lld matrices of 128 x %lld", (long long)batch, (long long)n);
   HeadFrontArgs a{x, n, (int)(n / HA_SPLIT), eps, mom, xb, partials, gram, norm, sumsq_out, xscale};
   dim3 grid((unsigned)(batch * a.splits)), block(HA_NT);
+  MI_OTHER_LAUNCH();
+  MI_FOOTPRINT("input", x, 4, batch, HA_M * n, HA_M, n, n);
+  MI_FOOTPRINT("momentum buffer", mom.buf, 4, batch, HA_M * n, HA_M, n, n);
+  MI_FOOTPRINT("bf16 copy", xb, 2, batch, HA_M * n, HA_M, n, n);
+  MI_FOOTPRINT("partial sums of squares", partials, 8, batch, a.splits, 1, a.splits, a.splits);
+  MI_FOOTPRINT("Gram partials", gram, 4, batch, (int64_t)a.splits * HA_M * HA_M, a.splits, HA_M * HA_M, HA_M * HA_M);
+  MI_FOOTPRINT("norm", norm, 4, 1, 0, 1, batch, batch);
+  MI_FOOTPRINT("squared norm of the result", sumsq_out, 4, 1, 0, 1, batch, batch);
+  MI_FOOTPRINT("input scale", xscale, 4, 1, 0, 1, batch, batch);
   hipLaunchKernelGGL(head_front_kernel<false>, grid, block, 0, stream, a);
   hipLaunchKernelGGL(head_front_kernel<true>, grid, block, 0, stream, a);
   hipError_t e = hipGetLastError();

@@ -9,8 +9,11 @@
 #include "norm_common.hpp"
 
 // Every launch of the fast kernel goes through MI_LAUNCH_FAST.  In the host-side bounds check build (MI_HOST_CHECK,
-// `make host-check`) nothing is launched: the fast kernel's launches are walked on the host (host_check.hpp), the other
-// kernels' launches and the runtime calls around them are compiled out.
+// `make host-check`) nothing is launched: the fast kernel's launches are walked on the host lane by lane
+// (host_check.hpp); the other kernels' launches and the runtime calls around them are compiled out, and what is checked
+// for them is the block of memory each pointer argument covers, which the launch site states with
+//   MI_FOOTPRINT(what, base, bytes per element, batch, batch stride, rows, leading dimension, columns)
+// (strides in elements; a null base states nothing).  In the ordinary build MI_FOOTPRINT and MI_OTHER_LAUNCH are empty.
 #ifdef MI_HOST_CHECK
 #include "host_check.hpp"
 #undef hipLaunchKernelGGL
@@ -19,7 +22,11 @@
 #define hipFuncSetAttribute(...) hipSuccess
 #define MI_LAUNCH_FAST(C, P_KS, Q_KS, MODE, OUT_F32, EDGE, SK, RMW, grid, stream, q) \
   ::mi::host_check::fast_launch<C, P_KS, Q_KS, MODE, OUT_F32, EDGE, SK, RMW>(grid, q)
+#define MI_FOOTPRINT(...) ::mi::host_check::footprint(__VA_ARGS__)
+#define MI_OTHER_LAUNCH() ::mi::host_check::other_launch()
 #else
+#define MI_FOOTPRINT(...) ((void)0)
+#define MI_OTHER_LAUNCH() ((void)0)
 #define MI_LAUNCH_FAST(C, P_KS, Q_KS, MODE, OUT_F32, EDGE, SK, RMW, grid, stream, q) \
   hipLaunchKernelGGL((gemm_fast_kernel<C, P_KS, Q_KS, MODE, OUT_F32, EDGE, SK, RMW>), grid, dim3(C::NT), 0, stream, q)
 #endif

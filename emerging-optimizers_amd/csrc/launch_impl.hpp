@@ -35,6 +35,9 @@ int launch_one(const GemmParams& p, int64_t batch, hipStream_t stream) {
   if (int rc = check_slots(q, tiles)) return rc;
   g_last_launch = LastLaunch{(int)tiles, BM, BN, 0};
   dim3 grid((unsigned)tiles, (unsigned)batch, 1), block(WGM * WGN * 64, 1, 1);
+#ifdef MI_HOST_CHECK
+  host_check::general_launch(q, batch, P_KS, Q_KS, MODE == MODE_SYRK, OUT_F32, tiles);
+#endif
   hipLaunchKernelGGL(kern, grid, block, LDS_BYTES, stream, q);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "kernel launch failed: %s", hipGetErrorString(e));

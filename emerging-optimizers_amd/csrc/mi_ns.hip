@@ -940,6 +940,18 @@ static int frob_impl(const float* x, int64_t batch, int64_t numel, float eps, in
     // tall input, deferred divide: the first pass already transposes (one partial per workgroup of the tile walk)
     const int64_t ntiles = ((t_rows + 63) / 64) * ((t_cols + 63) / 64);
     nparts = (int)(ntiles < NORM_MAX_BLOCKS ? ntiles : NORM_MAX_BLOCKS);
+  }
+  // what the two passes cover: the input (and the momentum buffer, updated in place), the cast or the normalised
+  // copy, one float64 partial per workgroup of the first pass, one value per matrix of each scalar output
+  MI_OTHER_LAUNCH();
+  MI_FOOTPRINT("input", x, 4, batch, numel, 1, numel, numel);
+  MI_FOOTPRINT("momentum buffer", mom.buf, 4, batch, numel, 1, numel, numel);
+  MI_FOOTPRINT("normalised copy", out, out_bf16 ? 2 : 4, batch, numel, 1, numel, numel);
+  MI_FOOTPRINT("partial sums of squares", partials, 8, batch, nparts, 1, nparts, nparts);
+  MI_FOOTPRINT("norm", dev_norm, 4, 1, 0, 1, batch, batch);
+  MI_FOOTPRINT("squared norm of the result", sumsq_out, 4, 1, 0, 1, batch, batch);
+  MI_FOOTPRINT("input scale", xscale, 4, 1, 0, 1, batch, batch);
+  if (t_rows > 0 && xscale) {
     dim3 gridw((unsigned)nparts, (unsigned)batch);
     if (f64)
       hipLaunchKernelGGL(sumsq_transpose_kernel<true>, gridw, block, 0, stream, x, t_rows, t_cols, partials, mom, raw_out);
@@ -1328,6 +1340,12 @@ static int small_gram(const uint16_t* X, int64_t batch, int64_t m, int64_t n, in
   int rc = small_gram_partials(X, batch, m, n, splits, partials, stream);
   if (rc != MI_OK) return rc;
   dim3 grid((unsigned)((m * m + 255) / 256), (unsigned)batch), block(256);
+  MI_OTHER_LAUNCH();
+  MI_FOOTPRINT("Gram partials", partials, 4, batch, splits * m * m, splits, m * m, m * m);
+  MI_FOOTPRINT("partial sums read", slots_in, 4, batch, nslots_in, 1, nslots_in, nslots_in);
+  MI_FOOTPRINT("shift written", shift_io, 4, 1, 0, 1, batch, batch);
+  MI_FOOTPRINT("Gram matrix", gram, 2, batch, m * m, m, m, m);
+  MI_FOOTPRINT("input scale read", xscale, 4, 1, 0, 1, batch, batch);
   hipLaunchKernelGGL(gram_reduce_kernel, grid, block, 0, stream, partials, splits, (int)m, slots_in, nslots_in, shift_io, gram, xscale);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "gram_reduce launch failed: %s", hipGetErrorString(e));
@@ -1354,6 +1372,12 @@ static int small_chain(const uint16_t* X, int64_t batch, int64_t n, int splits, 
     for (int e = 0; e < 3; ++e) a.co[k][e] = abc[3 * k + e];
   a.group = group;
   a.out = out;
+  MI_OTHER_LAUNCH();
+  MI_FOOTPRINT("Gram partials", partials, 4, batch, (int64_t)splits * CH_M * CH_M, splits, CH_M * CH_M, CH_M * CH_M);
+  MI_FOOTPRINT("partial sums read", slots_in, 4, batch, nslots_in, 1, nslots_in, nslots_in);
+  MI_FOOTPRINT("shift written", shift_io, 4, 1, 0, 1, batch, batch);
+  MI_FOOTPRINT("input scale read", xscale, 4, 1, 0, 1, batch, batch);
+  MI_FOOTPRINT("multiplier of X", out, 2, batch, CH_M * CH_M, CH_M, CH_M, CH_M);
   hipLaunchKernelGGL(small_chain_kernel, dim3((unsigned)batch), dim3(CH_THREADS), 0, stream, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "small_chain launch failed: %s", hipGetErrorString(e));
@@ -1677,6 +1701,9 @@ static int ns_impl(const float* x, float* out, int64_t batch, int64_t rows, int6
   if (tall && !direct_t) {
     ProfScope prof(PROF_NORMALIZE, stream);
     dim3 gridt((unsigned)((n + 63) / 64), (unsigned)((m + 63) / 64), (unsigned)batch), blockt(256);
+    MI_OTHER_LAUNCH();
+    MI_FOOTPRINT("staged result", result, 4, batch, m * n, m, n, n);
+    MI_FOOTPRINT("result, transposed back", out, 4, batch, m * n, n, m, m);
     hipLaunchKernelGGL(transpose_f32_kernel, gridt, blockt, 0, stream, result, m, n, out, out_accum);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(MI_ERR_LAUNCH, "transpose launch failed: %s", hipGetErrorString(e));
@@ -1721,6 +1748,9 @@ int mi_syrk_bf16_ws(const void* A, int64_t batch, int64_t n, int64_t k, int64_t 
       // the operand, K-contiguous, in the first part of the workspace; the rest serves the product itself
       uint16_t* At = static_cast<uint16_t*>(workspace);
       dim3 grid((unsigned)((n + 63) / 64), (unsigned)((k + 63) / 64), (unsigned)batch);
+      MI_OTHER_LAUNCH();
+      MI_FOOTPRINT("operand stored as K rows", A, 2, batch, a_batch_stride, k, a_ld, n);
+      MI_FOOTPRINT("operand copy, K-contiguous", At, 2, batch, n * k, n, k, k);
       hipLaunchKernelGGL(transpose_bf16_kernel, grid, dim3(256), 0, st, static_cast<const uint16_t*>(A), a_batch_stride, a_ld, At,
                          n * k, k, (int)n, (int)k);
       hipError_t e = hipGetLastError();
