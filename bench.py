@@ -64,7 +64,7 @@ MIN_WARMUP, MIN_TIMED = 3, 20
 # with none of this library's kernels in flight, two at a place that could not be read back; no run without them
 # faulted, on the same kernels, before or after.  The default run therefore calls no torch bf16 matmul at all (its
 # float32 parity references are torch float32 matmuls, as in every earlier run).  The figures of the one complete run
-# with comparators are recorded in DESIGN.md.
+# with comparators are kept under profiles/ (bench_all_workloads_with_torch_comparators).
 TORCH_COMPARATOR_ROWS = ("mlp", "attn", "batched_syrk")
 TORCH_COMPARATORS = False  # set by --torch-comparators
 
