@@ -40,6 +40,7 @@ struct State {
   long launches = 0, workgroups = 0, accesses = 0, failures = 0;
   long other_launches = 0, footprints = 0;  // launches of the self-guarding kernels, blocks of memory they stated
   const char* context = "";
+  bool exhaustive = false;  // walk the lanes of every workgroup and every K tile instead of the sample described below
   uint64_t hit_lo = 1, hit_hi = 0;  // the buffer the last access fell into (consecutive accesses mostly share one)
 };
 inline State g_state;
@@ -156,13 +157,13 @@ void fast_launch(dim3 grid, const GemmParams& p) {
 
   // Every workgroup is decoded (tile coverage); the lanes of all workgroups are walked for grids of up to 640
   // workgroups, of the first and last 128 and of every (total / 256)-th one for larger grids (addresses are affine in
-  // the tile indices between the ends).
+  // the tile indices between the ends).  `exhaustive` drops both samples: every workgroup, every K tile.
   const long total = (long)grid.x * (long)grid.y;
   const long every = total > 640 ? total / 256 : 1;
   for (unsigned by = 0; by < grid.y; ++by) {
     for (unsigned bx = 0; bx < grid.x; ++bx) {
       const long index = (long)by * grid.x + bx;
-      const bool walk_lanes = total <= 640 || index < 128 || index >= total - 128 || index % every == 0;
+      const bool walk_lanes = st.exhaustive || total <= 640 || index < 128 || index >= total - 128 || index % every == 0;
       const int bid = (int)bx;
       int64_t batch = by;
       int tm, tn, k_first = 0, nk = nk_full, sk_tile = 0, sk_split = 0;
@@ -230,7 +231,7 @@ void fast_launch(dim3 grid, const GemmParams& p) {
             lp.init(p.P + p_off + (STREAMK ? (int64_t)k_first * C::BK : 0), p.ldp, m0, p.M, wave, lane);
             lq.init(p.Q + q_off + (STREAMK ? (int64_t)k_first * C::BK : 0), p.ldq, n0, p.N, wave, lane);
             for (int kt = 0; kt < nk; ++kt) {
-              if (kt < 2 || kt >= nk - 2) {  // (the address of a load is affine in kt: the ends bound the rest)
+              if (kt < 2 || kt >= nk - 2 || st.exhaustive) {  // (the address of a load is affine in kt: the ends bound the rest)
                 for (int i = 0; i < decltype(lp)::LPT; ++i) touch(lp.address(i), 16, "operand P load");
                 for (int i = 0; i < decltype(lq)::LPT; ++i) touch(lq.address(i), 16, "operand Q load");
               }

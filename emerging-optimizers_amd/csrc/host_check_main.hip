@@ -226,7 +226,10 @@ int selftest() {
 int main(int argc, char** argv) {
   if (argc > 1 && std::strcmp(argv[1], "--selftest") == 0) return selftest();
   const bool quick = argc > 1 && std::strcmp(argv[1], "--quick") == 0;
-  const bool bench_only = argc > 1 && std::strcmp(argv[1], "--bench") == 0;  // the benchmark's own calls only
+  // --bench: the benchmark's own calls only; --bench-exhaustive: the same calls with no sampling of workgroups or K tiles
+  const bool bench_exhaustive = argc > 1 && std::strcmp(argv[1], "--bench-exhaustive") == 0;
+  const bool bench_only = bench_exhaustive || (argc > 1 && std::strcmp(argv[1], "--bench") == 0);
+  state().exhaustive = bench_exhaustive;
   validation_cases();
   // ---- lower-triangle products
   const int64_t ns_[] = {256, 384, 512, 768, 1024, 1032, 1096, 1152, 1280, 1536, 1792, 1800, 2048, 2304, 3072, 4096, 5120, 8184, 8192};
